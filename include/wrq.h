@@ -1,0 +1,153 @@
+/*
+ * wrq.h -- C ABI of libwrq_hip.so: web-rwkv's quantized-weight matrix path
+ * (Int8 / NF4 packing and the products on packed weights) for MI355X (gfx950).
+ *
+ * Every entry point replaces one constructor of the reference's `TensorOp`
+ * (src/tensor/ops.rs) and takes the same operands in the same order.  Where the
+ * reference builds a deferred op that `Context::encode` later records into the
+ * single wgpu queue (src/tensor/ops.rs:78-144), these calls enqueue the work on
+ * the HIP stream given as first argument and return at once; work on one stream
+ * runs in call order with no host synchronisation, like ops of one command
+ * buffer.  All pointers inside tensors are device pointers owned by the caller
+ * and must stay valid until the stream has passed the call.  No entry point
+ * allocates, frees or copies to the host.  All are thread-safe.
+ *
+ * Shapes use the reference's order, x fastest (src/tensor/shape.rs:97): a matrix
+ * `[K, R, B, 1]` holds B * R rows of K contiguous elements.
+ *
+ * Return value: WRQ_OK or a wrq_status error; the checks of the reference's
+ * op constructors (`check_shape`, src/tensor/mod.rs:213-219) are made before
+ * anything is launched, and its unchecked preconditions (R % 4, K % 4 ...) are
+ * checked here too.  wrq_last_error() gives the message of the calling thread's
+ * last failure, worded like the reference's TensorErrorKind (src/tensor/mod.rs:127-155).
+ */
+#ifndef WRQ_H
+#define WRQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WRQ_ABI_VERSION 1
+#define WRQ_INT8_BLOCK_SIZE 128u /* TensorOp::INT8_BLOCK_SIZE, src/tensor/ops.rs:292 */
+#define WRQ_NF4_BLOCK_SIZE 64u   /* TensorOp::NF4_BLOCK_SIZE, src/tensor/ops.rs:291 */
+
+typedef enum wrq_status {
+    WRQ_OK = 0,
+    WRQ_ERR_SHAPE = 1,       /* TensorErrorKind::Shape(got, want) */
+    WRQ_ERR_SIZE = 2,        /* TensorErrorKind::Size */
+    WRQ_ERR_TYPE = 3,        /* TensorErrorKind::Type: dtype is neither F16 nor F32 */
+    WRQ_ERR_ALIGNMENT = 4,   /* a precondition the reference leaves unchecked: row/column multiples, pointer alignment */
+    WRQ_ERR_UNSUPPORTED = 5, /* legal in the reference, not provided here (sliced matrix views) */
+    WRQ_ERR_NULL = 6,        /* null pointer argument */
+    WRQ_ERR_DEVICE = 7       /* HIP runtime error at launch */
+} wrq_status;
+
+/* `Float::DEF` of the reference: "FP16" / "FP32" (src/num.rs:98-108). */
+typedef enum wrq_dtype { WRQ_F16 = 0, WRQ_F32 = 1 } wrq_dtype;
+
+/* `Activation`, in declaration order (src/tensor/ops.rs:146-160). */
+typedef enum wrq_activation {
+    WRQ_ACT_NONE = 0,
+    WRQ_ACT_SQUARED_RELU = 1,
+    WRQ_ACT_TANH = 2, /* "custom_tanh": 1.0 above 42 */
+    WRQ_ACT_STABLE_EXP = 3,
+    WRQ_ACT_OPPOSITE_EXP = 4,
+    WRQ_ACT_SOFTPLUS = 5,
+    WRQ_ACT_SIGMOID = 6,
+    WRQ_ACT_SILU = 7
+} wrq_activation;
+
+/* `TensorGpu<T, K>`: a device buffer and its shape (src/tensor/mod.rs). */
+typedef struct wrq_tensor {
+    void *data;
+    uint32_t shape[4];
+} wrq_tensor;
+
+/* `View`, byte for byte the reference's uniform (src/tensor/mod.rs:26-43):
+ * `stride` is the shape of the parent tensor, `offset` the start of the slice. */
+typedef struct wrq_view {
+    uint32_t shape[4];
+    uint32_t stride[4];
+    uint32_t offset[4];
+} wrq_view;
+
+/* `TensorGpuView<F>`: parent buffer + view + element type. */
+typedef struct wrq_tensor_view {
+    void *data; /* start of the parent tensor */
+    wrq_view view;
+    wrq_dtype dtype;
+} wrq_tensor_view;
+
+/* `hipStream_t`, spelled as a plain pointer so that bindings need no HIP headers;
+ * NULL is the default stream. */
+typedef void *wrq_stream;
+
+/* Loads the code object on the current device and checks that it is a gfx950.
+ * Optional: every entry point does this on first use. */
+int wrq_init(void);
+
+int wrq_abi_version(void);
+const char *wrq_status_string(int status);
+const char *wrq_last_error(void);
+
+/*
+ * TensorOp::quantize_mat_int8(input, minmax, output)       src/tensor/ops.rs:2393-2486
+ *   input  f16 [K, R, B, 1]; output u8 [K, R, B, 1];
+ *   minmax f16 [2 * ceil(len / 128), 1, 1, 1], (min, max) per flat 128-block.
+ *   len % 128 == 0 is required (the two minmax-shape formulas of the reference,
+ *   ops.rs:809 and :2402-2403, agree only then).
+ */
+int wrq_quantize_mat_int8(wrq_stream stream, const wrq_tensor *input, const wrq_tensor *minmax,
+                          const wrq_tensor *output);
+
+/*
+ * TensorOp::quantize_mat_nf4(input, quant, absmax, output)  src/tensor/ops.rs:2488-2589
+ *   input f16 [K, R, B, 1]; quant f32 [16, 1, 1, 1] (device); output u8 [K/2, R, B, 1];
+ *   absmax f16 [ceil(len / 64), 1, 1, 1].  len % 64 == 0 is required.  The f32
+ *   temporary and the f32 -> f16 blit of the reference (ops.rs:2505, :2586) are fused.
+ */
+int wrq_quantize_mat_nf4(wrq_stream stream, const wrq_tensor *input, const wrq_tensor *quant,
+                         const wrq_tensor *absmax, const wrq_tensor *output);
+
+/*
+ * TensorOp::matmul_vec_int8(matrix, minmax, input, output, act, sparse)
+ *                                                          src/tensor/ops.rs:791-886
+ *   matrix u8 [K, R, B, 1]; input view [K, T, B, 1]; output view [R, T, B, 1].
+ *   Any T: tokens share one pass over the weights.  `sparse` (SPARSE_INPUT) never
+ *   changes results for finite weights and is accepted as a hint.
+ */
+int wrq_matmul_vec_int8(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor *minmax,
+                        const wrq_tensor_view *input, const wrq_tensor_view *output, int act,
+                        int sparse);
+
+/* TensorOp::matmul_vec_nf4(matrix, quant, absmax, input, output, act, sparse)
+ *                                                          src/tensor/ops.rs:892-991
+ *   matrix u8 [K/2, R, B, 1]. */
+int wrq_matmul_vec_nf4(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor *quant,
+                       const wrq_tensor *absmax, const wrq_tensor_view *input,
+                       const wrq_tensor_view *output, int act, int sparse);
+
+/*
+ * TensorOp::matmul_mat_int8(matrix, minmax, input, output, act)
+ *                                                          src/tensor/ops.rs:1072-1140
+ *   matrix: view of a u8 tensor, `[K, R, B, 1]`; it must cover its whole parent.
+ *   R and T multiples of 4 (ops.rs:1068-1069), K a multiple of 32.
+ */
+int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
+                        const wrq_tensor_view *input, const wrq_tensor_view *output, int act);
+
+/* TensorOp::matmul_mat_nf4(matrix, quant, absmax, input, output, act)
+ *                                                          src/tensor/ops.rs:1150-1221
+ *   matrix: view `[K/2, R, B, 1]` of u8, whole parent; K a multiple of 64. */
+int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *quant,
+                       const wrq_tensor *absmax, const wrq_tensor_view *input,
+                       const wrq_tensor_view *output, int act);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WRQ_H */

@@ -18,3 +18,21 @@ def oracle():
 
     wrq_oracle.lib()
     return wrq_oracle
+
+
+@pytest.fixture(scope="session")
+def wrq():
+    import importlib
+
+    return importlib.import_module("web-rwkv_amd")
+
+
+@pytest.fixture(scope="session")
+def gpu(wrq):
+    """The binding with the library loaded on a real GPU; fails (never skips) without one."""
+    import torch
+
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    status = wrq.lib().wrq_init()
+    assert status == 0, wrq.lib().wrq_last_error().decode()
+    return wrq

@@ -1,0 +1,338 @@
+"""Parity of the HIP path against the CPU oracle and float64 truth, through the C ABI.
+
+Bars: packed bytes and scale blocks bit-exact; products within
+|a - b| <= max(eps, eps * max(|a|, |b|)), eps = 2e-3 (f16 output, f32 accumulate).
+"""
+import numpy as np
+import pytest
+
+from helpers import (ACTS, EPS, NF4_QUANT, assert_close, gen_f16, int8_dequant64, nf4_dequant64,
+                     truth_matmul)
+
+pytestmark = pytest.mark.gpu
+
+SEED = 0x57525100
+
+
+def dev(a):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    import torch
+
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def announce(*what):
+    print("case:", *what, flush=True)
+
+
+# ---------------------------------------------------------------- packing
+
+
+PACK_SHAPES = [(64, 320), (2048, 2560), (2048, 2048), (2048, 7168), (7168, 2048), (768, 2688), (3, 8, 512)]
+
+
+def special_blocks(rng):
+    """Edge cases: constant and zero blocks, +-max f16, subnormals, exact ties, +-absmax."""
+    w = gen_f16(rng, (16, 1024), 0.02)
+    w[0, :128] = np.float16(0.25)  # constant int8 block -> all codes 0
+    w[1, :] = 0  # zero nf4 blocks -> nibble 0, absmax 0
+    w[2, :4] = [65504, -65504, 6e-8, -6e-8]
+    w[3, :256] = np.linspace(-1, 1, 256).astype(np.float16)  # many exact ties after scaling
+    w[4, :64] = 0.5
+    w[4, 1] = -0.5
+    w[5, :128] = np.arange(128, dtype=np.float16) * np.float16(2.0)  # (v-min)/(max-min)*255 hits n + 0.5 often
+    return w
+
+
+@pytest.mark.parametrize("shape", PACK_SHAPES, ids=str)
+def test_quant_int8_bit_exact(gpu, oracle, shape):
+    import torch
+
+    announce("quant_int8", shape)
+    rng = np.random.default_rng(SEED + 2)
+    w = gen_f16(rng, shape, 0.02)
+    m = gpu.Matrix.quant_u8(dev(w))
+    want_w, want_m, flagged = oracle.quant_int8(w)
+    assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+    got = host(m.w)
+    assert got.shape == w.shape
+    assert np.array_equal(got, want_w), f"{(got != want_w).sum()} bytes differ ({flagged} policy-sensitive)"
+
+
+def test_quant_int8_edge_cases(gpu, oracle):
+    announce("quant_int8 edge cases")
+    w = special_blocks(np.random.default_rng(SEED + 20))
+    m = gpu.Matrix.quant_u8(dev(w))
+    want_w, want_m, _ = oracle.quant_int8(w)
+    assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+    assert np.array_equal(host(m.w), want_w)
+    assert (host(m.w)[0, :128] == 0).all()
+
+
+@pytest.mark.parametrize("shape", PACK_SHAPES, ids=str)
+def test_quant_nf4_bit_exact(gpu, oracle, shape):
+    announce("quant_nf4", shape)
+    rng = np.random.default_rng(SEED + 3)
+    w = gen_f16(rng, shape, 0.02)
+    m = gpu.Matrix.quant_nf4(dev(w))
+    want_w, want_m = oracle.quant_nf4(w)
+    assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+    got = host(m.w)
+    assert got.shape == want_w.shape
+    assert np.array_equal(got, want_w), f"{(got != want_w).sum()} bytes differ"
+    assert np.array_equal(host(m.q), NF4_QUANT)
+
+
+def test_quant_nf4_edge_cases_and_custom_table(gpu, oracle):
+    announce("quant_nf4 edge cases")
+    w = special_blocks(np.random.default_rng(SEED + 30))
+    for table in (None, np.linspace(-1, 1, 16).astype(np.float32) ** 3):
+        m = gpu.Matrix.quant_nf4(dev(w), None if table is None else table.tolist())
+        want_w, want_m = oracle.quant_nf4(w, NF4_QUANT if table is None else table)
+        assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+        assert np.array_equal(host(m.w), want_w)
+    assert (host(m.w)[1] == 0).all()
+
+
+def test_quant_every_f16_value(gpu, oracle):
+    announce("quant every finite f16")
+    allh = np.arange(65536, dtype=np.uint16).view(np.float16)
+    fin = allh[np.isfinite(allh)]
+    fin = np.concatenate([fin, np.zeros((-len(fin)) % 128, np.float16)])
+    rng = np.random.default_rng(SEED + 40)
+    for order in (fin, rng.permutation(fin)):
+        w = order.reshape(-1, 128)
+        m8, m4 = gpu.Matrix.quant_u8(dev(w)), gpu.Matrix.quant_nf4(dev(w))
+        w8, s8, _ = oracle.quant_int8(w)
+        w4, s4 = oracle.quant_nf4(w)
+        assert np.array_equal(host(m8.w), w8) and np.array_equal(host(m8.m).view(np.uint16), s8.view(np.uint16))
+        assert np.array_equal(host(m4.w), w4) and np.array_equal(host(m4.m).view(np.uint16), s4.view(np.uint16))
+
+
+# --------------------------------------------------------------- products
+
+
+def pack(oracle, kind, w):
+    if kind == "int8":
+        u8, mm, _ = oracle.quant_int8(w)
+        return u8, mm, int8_dequant64(u8, mm)
+    p, am = oracle.quant_nf4(w)
+    return p, am, nf4_dequant64(p, am)
+
+
+def gpu_matrix(gpu, kind, wp, scale):
+    import torch
+
+    q = torch.tensor(gpu.NF4_QUANT, dtype=torch.float32, device="cuda") if kind == "nf4" else None
+    return gpu.Matrix("Int8" if kind == "int8" else "Fp4", dev(wp), dev(scale), q)
+
+
+def run(gpu, m, x, R, entry, out_dtype=np.float16, act=0, sparse=False):
+    import torch
+
+    T = x.shape[-2]
+    shape = x.shape[:-2] + (T, R)
+    out = torch.full(shape, float("nan"), dtype=torch.float16 if out_dtype == np.float16 else torch.float32, device="cuda")
+    xd = dev(x)
+    if entry == "vec":
+        m.matmul_vec_op(xd, out, act, sparse)
+    else:
+        m.matmul_mat_op(xd, out, act)
+    return host(out)
+
+
+# (K, R): config-2/3 operator sweep at RWKV-v6 1.6B shapes, 7B shapes, and the v5 config-1 shapes
+SWEEP = [(2048, 2048), (2048, 7168), (7168, 2048), (2048, 65536), (4096, 4096), (4096, 14336), (14336, 4096),
+         (768, 768), (768, 2688), (2688, 768)]
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("K,R", SWEEP, ids=str)
+def test_gemv_against_oracle(gpu, oracle, kind, K, R):
+    announce("gemv", kind, K, R)
+    rng = np.random.default_rng(SEED + 2 + K * 7 + R)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (1, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    ofn = oracle.matmul_vec_int8 if kind == "int8" else oracle.matmul_vec_nf4
+    for out_dtype in (np.float16, np.float32):
+        got = run(gpu, m, x, R, "vec", out_dtype)
+        want = ofn(wp, scale, x, out_dtype=out_dtype)[0]
+        assert_close(got, want, EPS, f"{kind} {K}x{R} vs oracle")
+        assert_close(got, truth_matmul(wdeq, x), EPS, f"{kind} {K}x{R} vs float64")
+    if out_dtype == np.float32:  # f32 output: accumulation error only, far inside the bar
+        assert_close(got, truth_matmul(wdeq, x), 1e-4, f"{kind} {K}x{R} f32 vs float64")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("T", [2, 3, 4, 5, 8, 15, 16, 17, 31])
+def test_multi_token_vec_entry(gpu, oracle, kind, T):
+    # T < 32 or T % 32 != 0 reaches the vec entry point in the reference (grid.y = T)
+    announce("vec multi-token", kind, T)
+    K, R = 2048, 512
+    rng = np.random.default_rng(SEED + 5 + T)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (T, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    ofn = oracle.matmul_vec_int8 if kind == "int8" else oracle.matmul_vec_nf4
+    got = run(gpu, m, x, R, "vec", np.float32)
+    assert_close(got, ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
+    assert_close(got, truth_matmul(wdeq, x), EPS, "vs float64")
+
+
+# (K, R, T) for the chunk kernels: config 3 (T in 32, 128, 256), config 4 (T = 128 at 7B), the
+# reference's own test shapes (ops.rs:3058-3059), and T below one MFMA tile
+GEMM = [(2048, 2048, 32), (2048, 2048, 128), (2048, 2048, 256), (2048, 7168, 32), (7168, 2048, 128),
+        (4096, 4096, 128), (2560, 2048, 64), (320, 64, 320), (768, 2688, 32), (2688, 768, 32), (2048, 512, 4),
+        (2048, 512, 20), (2048, 65536, 32)]
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("K,R,T", GEMM, ids=str)
+def test_gemm_against_truth(gpu, oracle, kind, K, R, T):
+    announce("gemm", kind, K, R, T)
+    if kind == "nf4" and K % 64:
+        pytest.skip("nf4 needs K % 64 == 0")
+    rng = np.random.default_rng(SEED + 3 + K * 7 + R + T)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (T, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    for out_dtype in (np.float16, np.float32):
+        got = run(gpu, m, x, R, "mat", out_dtype)
+        assert_close(got, truth, EPS, f"{kind} {K}x{R}x{T} vs float64")
+    assert_close(got, truth, 2e-4, "f32 output vs float64")  # exact operands: only f32 accumulation differs
+    if R * T * K <= 2048 * 2048 * 32:
+        ofn = oracle.matmul_mat_int8 if kind == "int8" else oracle.matmul_mat_nf4
+        assert_close(got, ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_reference_test_data_scale(gpu, oracle, kind):
+    # the reference's unit tests draw weights/inputs of magnitude ~1..5, outputs ~100 (ops.rs:2929-2937, 3072-3093)
+    announce("reference test scale", kind)
+    K, R, T = 2560, 2048, 64
+    rng = np.random.default_rng(42)
+    w = gen_f16(rng, (R, K), 1.0)
+    x = (2.0 * rng.random((T, K), dtype=np.float32) - 1.0).astype(np.float16)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    assert_close(run(gpu, m, x, R, "mat", np.float32), truth, EPS, "mat")
+    assert_close(run(gpu, m, x[:8], R, "vec", np.float32), truth[:8], EPS, "vec")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("act", list(ACTS))
+def test_activations(gpu, oracle, kind, act):
+    announce("activation", kind, act)
+    K, R = 1024, 256
+    rng = np.random.default_rng(SEED + 11)
+    w = gen_f16(rng, (R, K), 0.03)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    code = list(ACTS).index(act)
+    for T, entry in ((1, "vec"), (3, "vec"), (32, "mat")):
+        x = gen_f16(rng, (T, K), 1.0)
+        got = run(gpu, m, x, R, entry, np.float32, act=code)
+        assert_close(got, truth_matmul(wdeq, x, act), EPS, f"{act} {entry} T={T}")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_offset_views_f32_and_batch(gpu, oracle, kind):
+    import torch
+
+    announce("views", kind)
+    K, R, T = 1024, 128, 4
+    rng = np.random.default_rng(SEED + 17)
+    w = gen_f16(rng, (R, K), 0.02)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    # v6: att_sx.view(.., .., i, ..) of a [C, T, 5] tensor (src/runtime/v6.rs:806-829), f32 outputs for k/v/r
+    for in_dtype in (np.float16, np.float32):
+        parent = rng.standard_normal((5, T, K), dtype=np.float32).astype(in_dtype)
+        pd = dev(parent)
+        for entry in ("vec", "mat"):
+            for i in (1, 4):
+                out = torch.full((3, T + 2, R), -7.0, dtype=torch.float32, device="cuda")
+                views = dict(input_view=((K, T, 1), (K, T, 5), (0, 0, i)), output_view=((R, T, 1), (R, T + 2, 3), (0, 1, 2)))
+                (m.matmul_vec_op if entry == "vec" else m.matmul_mat_op)(pd, out, **views)
+                got = host(out)
+                assert_close(got[2, 1:1 + T], truth_matmul(wdeq, parent[i]), EPS, f"{entry} view {i}")
+                got[2, 1:1 + T] = -7.0
+                assert (got == -7.0).all(), "wrote outside the output view"
+    # batch axis B > 1: matrix [K, R, B], per-batch inputs
+    B = 3
+    wb = gen_f16(rng, (B, R, K), 0.02)
+    xb = gen_f16(rng, (B, T, K), 1.0)
+    wpb, sb, wdq = pack(oracle, kind, wb)
+    mb = gpu_matrix(gpu, kind, wpb, sb)
+    truth = np.stack([truth_matmul(wdq[b], xb[b]) for b in range(B)])
+    assert_close(run(gpu, mb, xb, R, "vec", np.float32), truth, EPS, "batched vec")
+    assert_close(run(gpu, mb, xb, R, "mat", np.float32), truth, EPS, "batched mat")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_sparse_flag_and_turbo_dispatch(gpu, oracle, kind):
+    announce("sparse/turbo", kind)
+    K, R = 2688, 768  # ffn.value of the v5 config: sparse (squared-relu) input
+    rng = np.random.default_rng(SEED + 19)
+    w = gen_f16(rng, (R, K), 0.02)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    x = np.maximum(gen_f16(rng, (1, K), 1.0), 0).astype(np.float16) ** 2
+    a = run(gpu, m, x, R, "vec", np.float32, sparse=False)
+    b = run(gpu, m, x, R, "vec", np.float32, sparse=True)
+    assert np.array_equal(a, b)
+    assert_close(a, truth_matmul(wdeq, x), EPS, "sparse input")
+    # Matrix::matmul_op picks the chunk kernel iff T % 32 == 0 (src/runtime/v6.rs:568-570)
+    import torch
+
+    assert gpu.turbo(32) and gpu.turbo(128) and not gpu.turbo(1) and not gpu.turbo(31)
+    for T in (1, 31, 32):
+        xt = gen_f16(rng, (T, K), 1.0)
+        out = torch.empty((T, R), dtype=torch.float16, device="cuda")
+        m.matmul_op_sparse(dev(xt), out, turbo=gpu.turbo(T))
+        assert_close(host(out), truth_matmul(wdeq, xt), EPS, f"matmul_op T={T}")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_full_size_properties(gpu, oracle, kind):
+    # size-independent checks at a 7B shape: linearity in x, and row permutation of W permutes outputs
+    import torch
+
+    announce("full-size properties", kind)
+    K, R = 4096, 14336
+    g = torch.Generator(device="cuda").manual_seed(SEED)
+    w = (torch.randn((R, K), generator=g, device="cuda") * 0.02).half()
+    m = gpu.Matrix.quant_u8(w) if kind == "int8" else gpu.Matrix.quant_nf4(w)
+    x1 = torch.randn((1, K), generator=g, device="cuda").half()
+    x2 = torch.randn((1, K), generator=g, device="cuda").half()
+    xs = (x1.float() + x2.float())  # exact in f32
+    o1, o2, os_ = (torch.empty((1, R), dtype=torch.float32, device="cuda") for _ in range(3))
+    m.matmul_vec_op(x1, o1)
+    m.matmul_vec_op(x2, o2)
+    m.matmul_vec_op(xs, os_)
+    assert_close(host(os_), host(o1 + o2), 1e-4, "linearity")
+    perm = torch.randperm(R, generator=g, device="cuda")
+    mp = gpu.Matrix.quant_u8(w[perm].contiguous()) if kind == "int8" else gpu.Matrix.quant_nf4(w[perm].contiguous())
+    assert torch.equal(mp.w, m.w[perm])  # K % 128 == 0: blocks never straddle rows, packing is per row
+    op = torch.empty((1, R), dtype=torch.float32, device="cuda")
+    mp.matmul_vec_op(x1, op)
+    assert torch.equal(op, o1[:, perm])
+    # chunk kernel agrees with the decode kernel on the same tokens
+    xt = torch.randn((32, K), generator=g, device="cuda").half()
+    ov, om = (torch.empty((32, R), dtype=torch.float32, device="cuda") for _ in range(2))
+    for t in range(32):
+        m.matmul_vec_op(xt[t:t + 1].contiguous(), ov[t:t + 1])
+    m.matmul_mat_op(xt, om)
+    assert_close(host(om), host(ov), 2e-4, "mat vs vec")

@@ -1,0 +1,244 @@
+"""ctypes binding of ``libwrq_hip.so`` for tests and benchmarks.
+
+The product is the shared library (C ABI in ``include/wrq.h``); this module only loads it
+and wraps torch device tensors into the ``wrq_tensor`` / ``wrq_tensor_view`` structs.  It
+never computes anything itself: without the library, or without a GPU, calls fail loudly.
+
+Names mirror the reference (``TensorOp::matmul_vec_int8`` ... in src/tensor/ops.rs,
+``Matrix::quant_u8`` ... in src/tensor/matrix.rs).  Shapes are given in the reference's
+order, x fastest: a torch tensor of shape ``(B, R, K)`` is the reference's ``[K, R, B, 1]``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwrq_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+INT8_BLOCK_SIZE = 128
+NF4_BLOCK_SIZE = 64
+
+OK, ERR_SHAPE, ERR_SIZE, ERR_TYPE, ERR_ALIGNMENT, ERR_UNSUPPORTED, ERR_NULL, ERR_DEVICE = range(8)
+F16, F32 = 0, 1
+
+ACTIVATIONS = ["", "squared_relu", "custom_tanh", "stable_exp", "opposite_exp", "softplus", "sigmoid", "silu"]
+ACT_NONE, ACT_SQUARED_RELU, ACT_TANH, ACT_STABLE_EXP, ACT_OPPOSITE_EXP, ACT_SOFTPLUS, ACT_SIGMOID, ACT_SILU = range(8)
+
+# Float4Quant::new, src/tensor/matrix.rs:46-70
+NF4_QUANT = [
+    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
+    -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
+    0.07958029955625534, 0.16093020141124725, 0.24611230194568634, 0.33791524171829224,
+    0.44070982933044434, 0.5626170039176941, 0.7229568362236023, 1.0,
+]
+
+EXPORTS = [
+    "wrq_init", "wrq_abi_version", "wrq_status_string", "wrq_last_error",
+    "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
+    "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
+]
+
+
+class TensorError(RuntimeError):
+    """A failed op constructor; ``status`` is the wrq_status code."""
+
+    def __init__(self, status, message):
+        super().__init__(message)
+        self.status = status
+
+
+class CTensor(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("shape", C.c_uint32 * 4)]
+
+
+class CView(C.Structure):
+    _fields_ = [("shape", C.c_uint32 * 4), ("stride", C.c_uint32 * 4), ("offset", C.c_uint32 * 4)]
+
+
+class CTensorView(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("view", CView), ("dtype", C.c_int)]
+
+
+def build(verbose=False):
+    """Compile every HIP source for gfx950 into ``libwrq_hip.so`` (always recompiles)."""
+    r = subprocess.run(["make", "-C", CSRC, "-B", "-j8"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building libwrq_hip.so failed:\n" + r.stdout[-4000:] + r.stderr[-4000:])
+    if verbose:
+        print(r.stdout[-2000:])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(hipcc --offload-arch=gfx950); this package has no CPU or eager fallback"
+            )
+        L = C.CDLL(LIB_PATH)
+        T, V, vp, i = C.POINTER(CTensor), C.POINTER(CTensorView), C.c_void_p, C.c_int
+        L.wrq_init.restype = i
+        L.wrq_abi_version.restype = i
+        L.wrq_status_string.restype = C.c_char_p
+        L.wrq_status_string.argtypes = [i]
+        L.wrq_last_error.restype = C.c_char_p
+        L.wrq_quantize_mat_int8.argtypes = [vp, T, T, T]
+        L.wrq_quantize_mat_nf4.argtypes = [vp, T, T, T, T]
+        L.wrq_matmul_vec_int8.argtypes = [vp, T, T, V, V, i, i]
+        L.wrq_matmul_vec_nf4.argtypes = [vp, T, T, T, V, V, i, i]
+        L.wrq_matmul_mat_int8.argtypes = [vp, V, T, V, V, i]
+        L.wrq_matmul_mat_nf4.argtypes = [vp, V, T, T, V, V, i]
+        for name in EXPORTS[4:]:
+            getattr(L, name).restype = i
+        _lib = L
+    return _lib
+
+
+def _check(status):
+    if status != OK:
+        raise TensorError(status, lib().wrq_last_error().decode())
+
+
+def _stream():
+    import torch
+
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def shape_of(t):
+    """Reference-order shape [x, y, z, w] of a torch tensor (last dim is x)."""
+    s = list(t.shape)[::-1]
+    assert len(s) <= 4
+    return s + [1] * (4 - len(s))
+
+
+def as_tensor(t, shape=None):
+    """``TensorGpu``: a contiguous device tensor and its shape."""
+    assert t.is_contiguous()
+    return CTensor(t.data_ptr(), tuple(shape if shape is not None else shape_of(t)))
+
+
+def _dtype(t):
+    import torch
+
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.float32:
+        return F32
+    return 2  # rejected by the library with ERR_TYPE
+
+
+def as_view(t, view=None, dtype=None):
+    """``TensorGpuView``: parent tensor plus (shape, stride, offset); default the whole tensor."""
+    assert t.is_contiguous()
+    if view is None:
+        s = shape_of(t)
+        view = (s, s, [0, 0, 0, 0])
+    pad = lambda v, f: tuple(v) + (f,) * (4 - len(v))
+    cv = CView(pad(view[0], 1), pad(view[1], 1), pad(view[2], 0))
+    return CTensorView(t.data_ptr(), cv, _dtype(t) if dtype is None else dtype)
+
+
+class TensorOp:
+    """The six constructors of the path; each enqueues on torch's current stream."""
+
+    INT8_BLOCK_SIZE = INT8_BLOCK_SIZE
+    NF4_BLOCK_SIZE = NF4_BLOCK_SIZE
+
+    @staticmethod
+    def quantize_mat_int8(input, minmax, output):
+        _check(lib().wrq_quantize_mat_int8(_stream(), C.byref(as_tensor(input)), C.byref(as_tensor(minmax)), C.byref(as_tensor(output))))
+
+    @staticmethod
+    def quantize_mat_nf4(input, quant, absmax, output):
+        _check(lib().wrq_quantize_mat_nf4(_stream(), C.byref(as_tensor(input)), C.byref(as_tensor(quant)), C.byref(as_tensor(absmax)), C.byref(as_tensor(output))))
+
+    @staticmethod
+    def matmul_vec_int8(matrix, minmax, input, output, act=ACT_NONE, sparse=False, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_vec_int8(_stream(), C.byref(as_tensor(matrix)), C.byref(as_tensor(minmax)),
+                                         C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act, int(sparse)))
+
+    @staticmethod
+    def matmul_vec_nf4(matrix, quant, absmax, input, output, act=ACT_NONE, sparse=False, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_vec_nf4(_stream(), C.byref(as_tensor(matrix)), C.byref(as_tensor(quant)), C.byref(as_tensor(absmax)),
+                                        C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act, int(sparse)))
+
+    @staticmethod
+    def matmul_mat_int8(matrix, minmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_mat_int8(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(minmax)),
+                                         C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
+
+    @staticmethod
+    def matmul_mat_nf4(matrix, quant, absmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_mat_nf4(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(quant)), C.byref(as_tensor(absmax)),
+                                        C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
+
+
+class Matrix:
+    """``Matrix::{Int8, Fp4}`` (src/tensor/matrix.rs:80-94): packed weights plus scales."""
+
+    def __init__(self, kind, w, m, q=None):
+        self.kind, self.w, self.m, self.q = kind, w, m, q
+
+    @staticmethod
+    def quant_u8(matrix):
+        """Matrix::quant_u8, src/tensor/matrix.rs:162-178."""
+        import torch
+
+        w = torch.empty(matrix.shape, dtype=torch.uint8, device=matrix.device)
+        n = (matrix.numel() * 2 + INT8_BLOCK_SIZE - 1) // INT8_BLOCK_SIZE
+        m = torch.empty(n, dtype=torch.float16, device=matrix.device)
+        TensorOp.quantize_mat_int8(matrix, m, w)
+        return Matrix("Int8", w, m)
+
+    @staticmethod
+    def quant_nf4(matrix, quant=None):
+        """Matrix::quant_nf4 / quant_sf4 (a caller-supplied table), src/tensor/matrix.rs:180-222."""
+        import torch
+
+        q = torch.tensor(NF4_QUANT if quant is None else quant, dtype=torch.float32, device=matrix.device)
+        w = torch.empty(matrix.shape[:-1] + (matrix.shape[-1] // 2,), dtype=torch.uint8, device=matrix.device)
+        n = (matrix.numel() + NF4_BLOCK_SIZE - 1) // NF4_BLOCK_SIZE
+        m = torch.empty(n, dtype=torch.float16, device=matrix.device)
+        TensorOp.quantize_mat_nf4(matrix, q, m, w)
+        return Matrix("Fp4", w, m, q)
+
+    def matmul_vec_op(self, input, output, act=ACT_NONE, sparse=False, **views):
+        if self.kind == "Int8":
+            TensorOp.matmul_vec_int8(self.w, self.m, input, output, act, sparse, **views)
+        else:
+            TensorOp.matmul_vec_nf4(self.w, self.q, self.m, input, output, act, sparse, **views)
+
+    def matmul_mat_op(self, input, output, act=ACT_NONE, **views):
+        if self.kind == "Int8":
+            TensorOp.matmul_mat_int8(self.w, self.m, input, output, act, **views)
+        else:
+            TensorOp.matmul_mat_nf4(self.w, self.q, self.m, input, output, act, **views)
+
+    def matmul_op(self, input, output, act=ACT_NONE, turbo=False, **views):
+        """Matrix::matmul_op, src/tensor/matrix.rs:136-147."""
+        if turbo:
+            self.matmul_mat_op(input, output, act, **views)
+        else:
+            self.matmul_vec_op(input, output, act, **views)
+
+    def matmul_op_sparse(self, input, output, act=ACT_NONE, turbo=False, **views):
+        """Matrix::matmul_op_sparse, src/tensor/matrix.rs:149-160."""
+        if turbo:
+            self.matmul_mat_op(input, output, act, **views)
+        else:
+            self.matmul_vec_op(input, output, act, sparse=True, **views)
+
+
+def turbo(num_token):
+    """Kernel choice of the model builders: chunk kernels iff T % 32 == 0 (src/runtime/v6.rs:568-570)."""
+    return num_token % 32 == 0

@@ -1,0 +1,298 @@
+// C ABI of libwrq_hip.so: argument checks of the reference's op constructors, view
+// resolution and kernel selection.  No kernel lives here.
+#include "wrq_device.h"
+#include "wrq_host.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace wrq {
+
+namespace {
+thread_local char g_error[512] = "";
+}
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int check_launch(const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    return WRQ_OK;
+}
+
+namespace {
+
+struct Shape4 {
+    uint64_t d[4];
+    uint64_t len() const { return d[0] * d[1] * d[2] * d[3]; }
+    bool operator==(const Shape4 &o) const { return memcmp(d, o.d, sizeof(d)) == 0; }
+};
+
+Shape4 shape_of(const uint32_t s[4]) { return Shape4{{s[0], s[1], s[2], s[3]}}; }
+
+// TensorShape::check_shape, src/tensor/mod.rs:213-219
+int check_shape(const Shape4 &got, const Shape4 &want) {
+    if (got == want) return WRQ_OK;
+    return fail(WRQ_ERR_SHAPE, "tensor shape not match: (%llu, %llu, %llu, %llu) vs. (%llu, %llu, %llu, %llu)",
+                (unsigned long long)got.d[0], (unsigned long long)got.d[1], (unsigned long long)got.d[2],
+                (unsigned long long)got.d[3], (unsigned long long)want.d[0], (unsigned long long)want.d[1],
+                (unsigned long long)want.d[2], (unsigned long long)want.d[3]);
+}
+
+uint64_t div_ceil(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+
+#define WRQ_TRY(expr)                  \
+    do {                               \
+        const int _s = (expr);         \
+        if (_s != WRQ_OK) return _s;   \
+    } while (0)
+
+int need(const void *p, const char *name) {
+    return p ? WRQ_OK : fail(WRQ_ERR_NULL, "null pointer: %s", name);
+}
+
+int need_tensor(const wrq_tensor *t, const char *name) {
+    WRQ_TRY(need(t, name));
+    if (!t->data) return fail(WRQ_ERR_NULL, "null pointer: %s.data", name);
+    return WRQ_OK;
+}
+
+int need_view(const wrq_tensor_view *v, const char *name, bool typed) {
+    WRQ_TRY(need(v, name));
+    if (!v->data) return fail(WRQ_ERR_NULL, "null pointer: %s.data", name);
+    if (typed && v->dtype != WRQ_F16 && v->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "data type mismatch");
+    for (int i = 0; i < 4; i++) {
+        // a view is a slice of its parent (src/tensor/mod.rs:1121-1141)
+        if ((uint64_t)v->view.offset[i] + v->view.shape[i] > v->view.stride[i])
+            return fail(WRQ_ERR_SHAPE, "slice %u..%llu out of range for dimension size %u", v->view.offset[i],
+                        (unsigned long long)v->view.offset[i] + v->view.shape[i], v->view.stride[i]);
+    }
+    if (v->view.shape[3] != 1 || v->view.offset[3] != 0)
+        return fail(WRQ_ERR_UNSUPPORTED, "views along the fourth axis are not supported");
+    return WRQ_OK;
+}
+
+bool covers_parent(const wrq_view &v) {
+    for (int i = 0; i < 4; i++)
+        if (v.offset[i] != 0 || v.shape[i] != v.stride[i]) return false;
+    return true;
+}
+
+// Resolves views into element strides and offset pointers (compute_index of the
+// shaders, src/shaders/matmul_vec_int8.wgsl:31-35).
+void resolve(const wrq_tensor_view &in, const wrq_tensor_view &out, MatmulArgs &a) {
+    const wrq_view &vi = in.view, &vo = out.view;
+    const size_t si = in.dtype == WRQ_F16 ? 2 : 4, so = out.dtype == WRQ_F16 ? 2 : 4;
+    a.x_token_stride = vi.stride[0];
+    a.x_batch_stride = (uint64_t)vi.stride[0] * vi.stride[1];
+    a.out_token_stride = vo.stride[0];
+    a.out_batch_stride = (uint64_t)vo.stride[0] * vo.stride[1];
+    const uint64_t xo = ((uint64_t)vi.offset[2] * vi.stride[1] + vi.offset[1]) * vi.stride[0] + vi.offset[0];
+    const uint64_t oo = ((uint64_t)vo.offset[2] * vo.stride[1] + vo.offset[1]) * vo.stride[0] + vo.offset[0];
+    a.x = static_cast<const uint8_t *>(in.data) + xo * si;
+    a.out = static_cast<uint8_t *>(out.data) + oo * so;
+    a.out_f16 = out.dtype == WRQ_F16;
+}
+
+enum Entry { kVec, kMat };
+
+// Shared body of the four product entry points.  `mshape` is the matrix shape in
+// bytes-per-row terms as the reference sees it: [K, R, B, 1] (int8) or [K/2, R, B, 1] (nf4).
+int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Shape4 &mshape,
+           const wrq_tensor *scale, const wrq_tensor *table, const wrq_tensor_view *input,
+           const wrq_tensor_view *output, int act) {
+    if (act < WRQ_ACT_NONE || act > WRQ_ACT_SILU) return fail(WRQ_ERR_UNSUPPORTED, "unknown activation %d", act);
+    const Shape4 os = shape_of(output->view.shape), is = shape_of(input->view.shape);
+    const uint64_t m = os.d[0], n = os.d[1], b = os.d[2], k = is.d[0];
+    // src/tensor/ops.rs:805-813 (int8), :907-916 (nf4), :1094-1103, :1172-1181
+    if (quant == kInt8) {
+        const uint64_t len = mshape.len();
+        WRQ_TRY(check_shape(shape_of(scale->shape), Shape4{{div_ceil(len << 1, WRQ_INT8_BLOCK_SIZE), 1, 1, 1}}));
+        WRQ_TRY(check_shape(mshape, Shape4{{k, m, b, 1}}));
+    } else {
+        const uint64_t len = mshape.len() << 1;
+        WRQ_TRY(check_shape(shape_of(scale->shape), Shape4{{div_ceil(len, WRQ_NF4_BLOCK_SIZE), 1, 1, 1}}));
+        WRQ_TRY(check_shape(mshape, Shape4{{k >> 1, m, b, 1}}));
+        WRQ_TRY(check_shape(shape_of(table->shape), Shape4{{16, 1, 1, 1}}));
+    }
+    WRQ_TRY(check_shape(is, Shape4{{k, n, b, 1}}));
+    WRQ_TRY(check_shape(os, Shape4{{m, n, b, 1}}));
+
+    // preconditions the reference leaves to the caller
+    const uint64_t block = quant == kInt8 ? WRQ_INT8_BLOCK_SIZE : WRQ_NF4_BLOCK_SIZE;
+    const uint64_t group = quant == kInt8 ? 4 : 8; // elements per u32 of packed weights
+    if ((k * m * b) % block)
+        return fail(WRQ_ERR_ALIGNMENT, "matrix size %llu is not a multiple of the %llu-element block",
+                    (unsigned long long)(k * m * b), (unsigned long long)block);
+    if (m % 4) return fail(WRQ_ERR_ALIGNMENT, "output rows %llu not a multiple of 4", (unsigned long long)m);
+    if (k % group) return fail(WRQ_ERR_ALIGNMENT, "input columns %llu not a multiple of %llu", (unsigned long long)k, (unsigned long long)group);
+    if (input->view.offset[0] % group || input->view.stride[0] % group)
+        return fail(WRQ_ERR_ALIGNMENT, "input view offset/stride along x not a multiple of %llu", (unsigned long long)group);
+    if (output->view.offset[0] % 4 || output->view.stride[0] % 4)
+        return fail(WRQ_ERR_ALIGNMENT, "output view offset/stride along x not a multiple of 4");
+    if ((uintptr_t)w % 4 || (uintptr_t)scale->data % 4 || (uintptr_t)input->data % 16 || (uintptr_t)output->data % 16)
+        return fail(WRQ_ERR_ALIGNMENT, "device pointers must be 16-byte aligned");
+    if (entry == kMat) {
+        // src/tensor/ops.rs:1068-1070, :1146-1149; the k-step of the shaders fetches one
+        // scale per 32 (int8) / 64 (nf4) columns
+        if (n % 4) return fail(WRQ_ERR_ALIGNMENT, "tokens %llu not a multiple of 4", (unsigned long long)n);
+        const uint64_t kstep = quant == kInt8 ? 32 : 64;
+        if (k % kstep) return fail(WRQ_ERR_ALIGNMENT, "input columns %llu not a multiple of %llu", (unsigned long long)k, (unsigned long long)kstep);
+    }
+    if (m > 0xffffffffull || n > 0xffffffffull || k > 0xffffffffull) return fail(WRQ_ERR_SIZE, "data size not match");
+
+    MatmulArgs a{};
+    a.w = static_cast<const uint8_t *>(w);
+    a.scale = static_cast<const uint16_t *>(scale->data);
+    a.quant = table ? static_cast<const float *>(table->data) : nullptr;
+    a.K = (uint32_t)k;
+    a.R = (uint32_t)m;
+    a.T = (uint32_t)n;
+    a.B = (uint32_t)b;
+    a.act = act;
+    resolve(*input, *output, a);
+    const int in_f16 = input->dtype == WRQ_F16;
+
+    // Matrix cores need K in whole 128-steps, 16-byte activation rows and output quads on
+    // their natural alignment; everything else runs on the VALU kernels, which accept
+    // every shape the reference accepts.
+    const size_t xs = in_f16 ? 2 : 4, osz = a.out_f16 ? 2 : 4;
+    const bool mfma_ok = (k % 128 == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
+                         ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0) &&
+                         ((uintptr_t)a.out % (4 * osz) == 0) && ((a.out_token_stride * osz) % (4 * osz) == 0) &&
+                         ((a.out_batch_stride * osz) % (4 * osz) == 0);
+    const bool chunk = entry == kMat ? true : n >= 16;
+    if (chunk && mfma_ok) return launch_gemm(stream, quant, in_f16, a);
+    return launch_gemv(stream, quant, in_f16, a);
+}
+
+} // namespace
+} // namespace wrq
+
+using namespace wrq;
+
+extern "C" {
+
+int wrq_abi_version(void) { return WRQ_ABI_VERSION; }
+
+const char *wrq_last_error(void) { return g_error; }
+
+const char *wrq_status_string(int status) {
+    switch (status) {
+    case WRQ_OK: return "ok";
+    case WRQ_ERR_SHAPE: return "tensor shape not match";
+    case WRQ_ERR_SIZE: return "data size not match";
+    case WRQ_ERR_TYPE: return "data type mismatch";
+    case WRQ_ERR_ALIGNMENT: return "operand alignment or multiple not met";
+    case WRQ_ERR_UNSUPPORTED: return "not supported";
+    case WRQ_ERR_NULL: return "null pointer";
+    case WRQ_ERR_DEVICE: return "device error";
+    default: return "unknown status";
+    }
+}
+
+int wrq_init(void) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(WRQ_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+    return WRQ_OK;
+}
+
+int wrq_quantize_mat_int8(wrq_stream stream, const wrq_tensor *input, const wrq_tensor *minmax,
+                          const wrq_tensor *output) {
+    WRQ_TRY(need_tensor(input, "input"));
+    WRQ_TRY(need_tensor(minmax, "minmax"));
+    WRQ_TRY(need_tensor(output, "output"));
+    // src/tensor/ops.rs:2400-2406
+    const Shape4 shape = shape_of(output->shape);
+    const uint64_t len = shape.len();
+    WRQ_TRY(check_shape(shape_of(input->shape), shape));
+    WRQ_TRY(check_shape(shape_of(minmax->shape), Shape4{{div_ceil(len, WRQ_INT8_BLOCK_SIZE) << 1, 1, 1, 1}}));
+    if (len % WRQ_INT8_BLOCK_SIZE)
+        return fail(WRQ_ERR_ALIGNMENT, "matrix size %llu is not a multiple of the 128-element block", (unsigned long long)len);
+    if ((uintptr_t)input->data % 16 || (uintptr_t)output->data % 8 || (uintptr_t)minmax->data % 4)
+        return fail(WRQ_ERR_ALIGNMENT, "device pointers must be 16-byte aligned");
+    return launch_quant_int8(static_cast<hipStream_t>(stream), input->data, minmax->data, output->data, len);
+}
+
+int wrq_quantize_mat_nf4(wrq_stream stream, const wrq_tensor *input, const wrq_tensor *quant,
+                         const wrq_tensor *absmax, const wrq_tensor *output) {
+    WRQ_TRY(need_tensor(input, "input"));
+    WRQ_TRY(need_tensor(quant, "quant"));
+    WRQ_TRY(need_tensor(absmax, "absmax"));
+    WRQ_TRY(need_tensor(output, "output"));
+    // src/tensor/ops.rs:2496-2503
+    const Shape4 shape = shape_of(output->shape);
+    const Shape4 input_shape{{shape.d[0] << 1, shape.d[1], shape.d[2], shape.d[3]}};
+    const uint64_t len = input_shape.len();
+    WRQ_TRY(check_shape(shape_of(input->shape), input_shape));
+    WRQ_TRY(check_shape(shape_of(absmax->shape), Shape4{{div_ceil(len, WRQ_NF4_BLOCK_SIZE), 1, 1, 1}}));
+    WRQ_TRY(check_shape(shape_of(quant->shape), Shape4{{16, 1, 1, 1}}));
+    if (len % WRQ_NF4_BLOCK_SIZE)
+        return fail(WRQ_ERR_ALIGNMENT, "matrix size %llu is not a multiple of the 64-element block", (unsigned long long)len);
+    if ((uintptr_t)input->data % 16 || (uintptr_t)output->data % 4 || (uintptr_t)absmax->data % 2 || (uintptr_t)quant->data % 4)
+        return fail(WRQ_ERR_ALIGNMENT, "device pointers must be 16-byte aligned");
+    return launch_quant_nf4(static_cast<hipStream_t>(stream), input->data, quant->data, absmax->data, output->data, len);
+}
+
+int wrq_matmul_vec_int8(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor *minmax,
+                        const wrq_tensor_view *input, const wrq_tensor_view *output, int act, int sparse) {
+    (void)sparse; // skipping all-zero input groups never changes a finite result
+    WRQ_TRY(need_tensor(matrix, "matrix"));
+    WRQ_TRY(need_tensor(minmax, "minmax"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    return matmul(static_cast<hipStream_t>(stream), kVec, kInt8, matrix->data, shape_of(matrix->shape), minmax,
+                  nullptr, input, output, act);
+}
+
+int wrq_matmul_vec_nf4(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor *quant,
+                       const wrq_tensor *absmax, const wrq_tensor_view *input,
+                       const wrq_tensor_view *output, int act, int sparse) {
+    (void)sparse;
+    WRQ_TRY(need_tensor(matrix, "matrix"));
+    WRQ_TRY(need_tensor(quant, "quant"));
+    WRQ_TRY(need_tensor(absmax, "absmax"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    return matmul(static_cast<hipStream_t>(stream), kVec, kNf4, matrix->data, shape_of(matrix->shape), absmax, quant,
+                  input, output, act);
+}
+
+int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
+                        const wrq_tensor_view *input, const wrq_tensor_view *output, int act) {
+    WRQ_TRY(need_view(matrix, "matrix", false));
+    WRQ_TRY(need_tensor(minmax, "minmax"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    return matmul(static_cast<hipStream_t>(stream), kMat, kInt8, matrix->data, shape_of(matrix->view.shape), minmax,
+                  nullptr, input, output, act);
+}
+
+int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *quant,
+                       const wrq_tensor *absmax, const wrq_tensor_view *input,
+                       const wrq_tensor_view *output, int act) {
+    WRQ_TRY(need_view(matrix, "matrix", false));
+    WRQ_TRY(need_tensor(quant, "quant"));
+    WRQ_TRY(need_tensor(absmax, "absmax"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    return matmul(static_cast<hipStream_t>(stream), kMat, kNf4, matrix->data, shape_of(matrix->view.shape), absmax,
+                  quant, input, output, act);
+}
+
+} // extern "C"

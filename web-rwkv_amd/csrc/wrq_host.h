@@ -1,0 +1,30 @@
+// Host-side declarations shared by the translation units of libwrq_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/wrq.h"
+
+namespace wrq {
+
+struct MatmulArgs;
+
+// Records a message for wrq_last_error() of the calling thread and returns `status`.
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Turns a launch failure (hipGetLastError) into WRQ_ERR_DEVICE.
+int check_launch(const char *what);
+
+int launch_quant_int8(hipStream_t stream, const void *in, void *minmax, void *out, uint64_t len);
+int launch_quant_nf4(hipStream_t stream, const void *in, const void *quant, void *absmax, void *out,
+                     uint64_t len);
+
+enum Quant { kInt8 = 0, kNf4 = 1 };
+
+// Decode-shaped products (few tokens): VALU dequantisation, wave reductions.
+int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+// Chunk-shaped products (T >= 16): f16 MFMA.
+int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+
+} // namespace wrq
