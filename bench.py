@@ -1,0 +1,305 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight matrix path on one MI355X.
+
+Default workload (config 4 of the baseline): one decode step, batch 1, of an RWKV-v6
+7B-shaped model (32 layers, d_model 4096, FFN 14336) with every layer Int8-quantized.  A
+"step" streams all packed weights of the path once: per layer the products att.key /
+value / receptance / gate / output (4096 -> 4096), ffn.key (4096 -> 14336, squared ReLU),
+ffn.value (14336 -> 4096, sparse hint) and ffn.receptance, with the reference's operand
+types and views (src/runtime/v6.rs:806-829, :880-885, :920-938).  Only this path is timed:
+the recurrent, normalisation and head ops of the model are not part of this library.
+
+Weights are random-init f16 ~ N(0, 0.02) (att.output and ffn.value pre-multiplied by
+2^-(layer / 6), src/runtime/loader.rs:734-762) packed on the GPU by the library itself;
+inputs are resident in HBM before the timed region.
+
+Prints one JSON line; see README/DESIGN for the fields.  `--sweep` prints the per-operator
+figures of configs 2 and 3 instead.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+SEED = 0x57525100
+
+
+def int8_bytes(K, R, T=1, out_size=2):
+    """Algorithmic bytes of one int8 product: weights + (min,max) pairs + input + output."""
+    return K * R + 4 * K * R // 128 + 2 * K * T + out_size * R * T
+
+
+def nf4_bytes(K, R, T=1, out_size=2):
+    return K * R // 2 + 2 * K * R // 64 + 64 + 2 * K * T + out_size * R * T
+
+
+class Layer:
+    pass
+
+
+def build_model(wrq, torch, quant, n_layer, C, H, rescale=6):
+    """Random-init packed weights of the eight quantized matrices per layer."""
+    g = torch.Generator(device="cuda").manual_seed(SEED + 4)
+    pack = wrq.Matrix.quant_u8 if quant == "int8" else wrq.Matrix.quant_nf4
+    layers = []
+    for i in range(n_layer):
+        discount = 2.0 ** -(i // rescale)
+        L = Layer()
+
+        def mat(R, K, scale=1.0):
+            w = (torch.randn((R, K), generator=g, device="cuda") * (0.02 * scale)).half()
+            return pack(w)
+
+        L.att_k, L.att_v, L.att_r, L.att_g = (mat(C, C) for _ in range(4))
+        L.att_o = mat(C, C, discount)
+        L.ffn_k = mat(H, C)
+        L.ffn_v = mat(C, H, discount)
+        L.ffn_r = mat(C, C)
+        layers.append(L)
+    torch.cuda.synchronize()
+    return layers
+
+
+class Decode:
+    """The op list of one run of the quantized path for T tokens (Appendix-B call sites of v6)."""
+
+    def __init__(self, wrq, torch, layers, C, H, T):
+        self.wrq, self.layers, self.C, self.H, self.T = wrq, layers, C, H, T
+        g = torch.Generator(device="cuda").manual_seed(SEED + 5)
+        f16, f32 = torch.float16, torch.float32
+        self.att_sx = torch.randn((5, T, C), generator=g, device="cuda").to(f16)  # [C, T, 5]
+        self.att_x = torch.randn((T, C), generator=g, device="cuda").to(f16)
+        self.ffn_kx = torch.randn((T, C), generator=g, device="cuda").to(f16)
+        self.ffn_rx = torch.randn((T, C), generator=g, device="cuda").to(f16)
+        self.att_k = torch.empty((T, C), dtype=f32, device="cuda")
+        self.att_v = torch.empty((T, C), dtype=f32, device="cuda")
+        self.att_r = torch.empty((T, C), dtype=f32, device="cuda")
+        self.att_g = torch.empty((T, C), dtype=f16, device="cuda")
+        self.att_o = torch.empty((T, C), dtype=f16, device="cuda")
+        self.ffn_k = torch.empty((T, H), dtype=f16, device="cuda")
+        self.ffn_v = torch.empty((T, C), dtype=f16, device="cuda")
+        self.ffn_r = torch.empty((T, C), dtype=f16, device="cuda")
+        self.turbo = wrq.turbo(T)
+        self.launches = 8 * len(layers)
+
+    def step_grouped(self):
+        """The same products with the independent ones of a layer sharing launches: {k, v, r, g},
+        then output, then {ffn.key, ffn.receptance}, then ffn.value (decode only)."""
+        wrq, C, T = self.wrq, self.C, self.T
+        sq, no = wrq.ACT_SQUARED_RELU, wrq.ACT_NONE
+        for L in self.layers:
+            wrq.matmul_vec_group([
+                (m, self.att_sx, out, no, False, dict(input_view=((C, T, 1), (C, T, 5), (0, 0, i))))
+                for i, (m, out) in enumerate(((L.att_k, self.att_k), (L.att_v, self.att_v), (L.att_r, self.att_r), (L.att_g, self.att_g)), 1)])
+            L.att_o.matmul_op(self.att_x, self.att_o, turbo=False)
+            wrq.matmul_vec_group([(L.ffn_k, self.ffn_kx, self.ffn_k, sq, False, {}), (L.ffn_r, self.ffn_rx, self.ffn_r, no, False, {})])
+            L.ffn_v.matmul_op_sparse(self.ffn_k, self.ffn_v, turbo=False)
+
+    def step(self):
+        wrq, C, T, turbo = self.wrq, self.C, self.T, self.turbo
+        sq = wrq.ACT_SQUARED_RELU
+        for L in self.layers:
+            for i, (m, out) in enumerate(((L.att_k, self.att_k), (L.att_v, self.att_v), (L.att_r, self.att_r), (L.att_g, self.att_g)), 1):
+                m.matmul_op(self.att_sx, out, turbo=turbo, input_view=((C, T, 1), (C, T, 5), (0, 0, i)))
+            L.att_o.matmul_op(self.att_x, self.att_o, turbo=turbo)
+            L.ffn_k.matmul_op(self.ffn_kx, self.ffn_k, sq, turbo=turbo)
+            L.ffn_v.matmul_op_sparse(self.ffn_k, self.ffn_v, turbo=turbo)
+            L.ffn_r.matmul_op(self.ffn_rx, self.ffn_r, turbo=turbo)
+
+    def bytes_per_step(self, quant):
+        f = int8_bytes if quant == "int8" else nf4_bytes
+        C, H, T = self.C, self.H, self.T
+        per_layer = 3 * f(C, C, T, 4) + 3 * f(C, C, T, 2) + f(C, H, T, 2) + f(H, C, T, 2)
+        return per_layer * len(self.layers)
+
+
+def time_steps(torch, fn, steps, warmup):
+    """ms per step over exactly `steps` calls, bracketed by synchronisation; HIP events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms / steps
+
+
+def cpu_baseline(wrq, torch, layers, dec, quant, sample_layers):
+    """The oracle (a port of the reference's kernels, OpenMP over rows) on the host cores, on a
+    bounded sample: `sample_layers` layers of the same decode step, scaled to the full depth."""
+    from oracle import wrq_oracle as oracle
+
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    vec = oracle.matmul_vec_int8 if quant == "int8" else oracle.matmul_vec_nf4
+    host = []
+    for L in layers[:sample_layers]:
+        host.append([(m.w.cpu().numpy(), m.m.cpu().numpy()) for m in (L.att_k, L.att_v, L.att_r, L.att_g, L.att_o, L.ffn_k, L.ffn_v, L.ffn_r)])
+    xc = dec.att_x[:1].cpu().numpy()
+    xh = np.maximum(dec.ffn_k[:1].cpu().numpy(), 0)
+    tokens = 0
+    t0 = time.perf_counter()
+    while True:
+        for mats in host:
+            for j, (w, s) in enumerate(mats):
+                x = xh if j == 6 else xc
+                vec(w, s, x, act=1 if j == 5 else 0, sparse=(j == 6))
+        tokens += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or tokens >= 64:
+            break
+    tok_s = tokens / (dt * len(layers) / sample_layers)
+    return {
+        "value": round(tok_s, 4), "unit": "tok/s", "cores": cores, "kind": "port",
+        "sample": f"{tokens} pass(es) over {sample_layers} of {len(layers)} layers of the same decode step ({dt:.1f} s of CPU work), scaled to full depth; "
+                  "CPU restatement of the reference kernels, not lavapipe",
+    }
+
+
+def sweep(wrq, torch, args):
+    """Per-operator figures of configs 2 and 3: cold (rotating weight copies) GB/s per shape."""
+    rows = []
+    g = torch.Generator(device="cuda").manual_seed(SEED + 2)
+    shapes = [(2048, 2048), (2048, 7168), (7168, 2048), (2048, 65536), (4096, 4096), (4096, 14336), (14336, 4096)]
+    for quant in ("int8", "nf4"):
+        for K, R in shapes:
+            w = (torch.randn((R, K), generator=g, device="cuda") * 0.02).half()
+            m0 = wrq.Matrix.quant_u8(w) if quant == "int8" else wrq.Matrix.quant_nf4(w)
+            del w
+            ncopy = max(2, int(1.5e9 // m0.w.numel()) + 1)
+            ncopy = min(ncopy, 64)
+            mats = [m0] + [wrq.Matrix(m0.kind, m0.w.clone(), m0.m.clone(), m0.q) for _ in range(ncopy - 1)]
+            for T in ([1] if quant == "int8" and not args.all_t else [1, 8, 32, 128, 256]):
+                x = torch.randn((T, K), generator=g, device="cuda").half()
+                out = torch.empty((T, R), dtype=torch.float16, device="cuda")
+                turbo = wrq.turbo(T)
+                it = [0]
+
+                def fn():
+                    mats[it[0] % ncopy].matmul_op(x, out, turbo=turbo)
+                    it[0] += 1
+
+                # one HIP graph of `reps` back-to-back launches over rotating weight copies, so
+                # that neither host launch cost nor cache reuse enters the figure
+                reps = max(ncopy, 50)
+                fn()
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(reps):
+                        fn()
+                ms, _ = time_steps(torch, graph.replay, 5, 2)
+                us = ms * 1e3 / reps
+                nbytes = (int8_bytes if quant == "int8" else nf4_bytes)(K, R, T)
+                flops = 2.0 * K * R * T
+                rows.append({"quant": quant, "K": K, "R": R, "T": T, "us": round(us, 2),
+                             "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
+                             "TFLOPs": round(flops / us / 1e6, 1), "copies": ncopy})
+                print(json.dumps(rows[-1]), flush=True)
+            del mats, m0
+            torch.cuda.empty_cache()
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--quant", choices=["int8", "nf4"], default="int8")
+    ap.add_argument("--tokens", type=int, default=1, help="tokens per step (1 = decode; 128 = a prefill chunk)")
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-group", action="store_true", help="one launch per product instead of grouped launches of independent products")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-layers", type=int, default=8)
+    ap.add_argument("--sweep", action="store_true", help="per-operator sweep (configs 2 and 3) instead of the decode step")
+    ap.add_argument("--all-t", action="store_true", help="with --sweep: all token counts for int8 too")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported (the path shards by weight rows, see DESIGN.md)")
+
+    import torch
+
+    wrq = importlib.import_module("web-rwkv_amd")
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    torch.cuda.set_device(0)
+    assert wrq.lib().wrq_init() == 0, wrq.lib().wrq_last_error().decode()
+
+    if args.sweep:
+        sweep(wrq, torch, args)
+        return
+
+    C, H = 4096, 14336
+    layers = build_model(wrq, torch, args.quant, args.layers, C, H)
+    dec = Decode(wrq, torch, layers, C, H, args.tokens)
+
+    grouped = not args.no_group and not dec.turbo
+    step = dec.step_grouped if grouped else dec.step
+    if grouped:
+        dec.launches = 4 * len(layers)
+    if args.no_graph:
+        fn = step
+    else:
+        # the launches of one step are captured once and replayed: the per-step host cost of
+        # 256 launches otherwise bounds batch-1 decode
+        step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        fn = graph.replay
+
+    ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
+    nbytes = dec.bytes_per_step(args.quant)
+    tok_s = args.tokens * 1e3 / wall_ms
+    launch_us = ms * 1e3 / dec.launches
+    achieved = nbytes / dec.launches / launch_us / 1e3  # GB/s
+    kernel = {("int8", True): "gemv_int8_kernel", ("nf4", True): "gemv_nf4_kernel"}.get((args.quant, args.tokens < 16), "gemm_kernel")
+    out = {
+        "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8" if args.quant == "int8" else "u4",
+        "data": "synthetic",
+        "config": {
+            "workload": f"config 4: RWKV-v6 7B-shape ({args.layers} layers, d_model 4096, FFN 14336), all layers {args.quant}, "
+                        f"batch 1, {args.tokens} token(s) per step, quantized-matrix path only (8 products per layer)",
+            "quant": args.quant, "tokens_per_step": args.tokens, "hip_graph": not args.no_graph, "grouped_launches": grouped,
+        },
+        "hbm_gbps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+        "bytes_per_step": nbytes,
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "kernel": kernel, "launches_per_step": dec.launches,
+            "avg_launch_us": round(launch_us, 3), "bytes_per_launch": nbytes // dec.launches,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wrq, torch, layers, dec, args.quant, min(args.cpu_sample_layers, args.layers))
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

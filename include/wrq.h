@@ -132,6 +132,42 @@ int wrq_matmul_vec_nf4(wrq_stream stream, const wrq_tensor *matrix, const wrq_te
                        const wrq_tensor_view *output, int act, int sparse);
 
 /*
+ * Grouped decode products.  No counterpart in the reference's op constructors: it is the
+ * HIP side of `TensorOp::List` (src/tensor/ops.rs:280-288), for the step where
+ * `Context::encode` (ops.rs:78-144) walks a list of ops.  `count` decode-shaped products
+ * that do not depend on each other -- the attention key / value / receptance / gate
+ * projections of a layer (src/runtime/v6.rs:806-829), or ffn.key and ffn.receptance
+ * (v6.rs:920-938) -- run as if wrq_matmul_vec_* were called on each in order, but share
+ * kernel launches: at batch 1 a 4096 x 4096 product is a few microseconds of HBM time and a
+ * dispatch of its own costs about as much.  The caller guarantees that no op of a group
+ * reads or writes the output of another.  Every op is checked like the single call, before
+ * anything is launched.  count <= WRQ_MAX_GROUP.
+ */
+#define WRQ_MAX_GROUP 8
+
+typedef struct wrq_vec_int8_op {
+    const wrq_tensor *matrix;
+    const wrq_tensor *minmax;
+    const wrq_tensor_view *input;
+    const wrq_tensor_view *output;
+    int act;
+    int sparse;
+} wrq_vec_int8_op;
+
+typedef struct wrq_vec_nf4_op {
+    const wrq_tensor *matrix;
+    const wrq_tensor *quant;
+    const wrq_tensor *absmax;
+    const wrq_tensor_view *input;
+    const wrq_tensor_view *output;
+    int act;
+    int sparse;
+} wrq_vec_nf4_op;
+
+int wrq_matmul_vec_int8_group(wrq_stream stream, const wrq_vec_int8_op *ops, int count);
+int wrq_matmul_vec_nf4_group(wrq_stream stream, const wrq_vec_nf4_op *ops, int count);
+
+/*
  * TensorOp::matmul_mat_int8(matrix, minmax, input, output, act)
  *                                                          src/tensor/ops.rs:1072-1140
  *   matrix: view of a u8 tensor, `[K, R, B, 1]`; it must cover its whole parent.

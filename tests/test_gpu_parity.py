@@ -336,3 +336,58 @@ def test_full_size_properties(gpu, oracle, kind):
         m.matmul_vec_op(xt[t:t + 1].contiguous(), ov[t:t + 1])
     m.matmul_mat_op(xt, om)
     assert_close(host(om), host(ov), 2e-4, "mat vs vec")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind):
+    # the independent products of a layer in shared launches: same results as one call each
+    import torch
+
+    announce("grouped", kind)
+    C, H, T = 1024, 3584, 1
+    rng = np.random.default_rng(SEED + 23)
+    shapes = [(C, C), (C, C), (C, C), (C, C), (C, H), (H, C)]  # (K, R); the last two differ in K
+    mats, truths = [], []
+    att_sx = gen_f16(rng, (5, T, C), 1.0)
+    xh = gen_f16(rng, (T, H), 1.0)
+    for j, (K, R) in enumerate(shapes):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        mats.append(gpu_matrix(gpu, kind, wp, scale))
+        x = att_sx[j + 1] if j < 4 else (att_sx[0] if K == C else xh)
+        truths.append(truth_matmul(wdeq, x, "squared_relu" if j == 4 else "none"))
+    sxd, xhd = dev(att_sx), dev(xh)
+    outs_dt = [torch.float32, torch.float32, torch.float32, torch.float16, torch.float16, torch.float16]
+    single = [torch.empty((T, R), dtype=dt, device="cuda") for (K, R), dt in zip(shapes, outs_dt)]
+    group = [torch.full((T, R), float("nan"), dtype=dt, device="cuda") for (K, R), dt in zip(shapes, outs_dt)]
+    ops = []
+    for j, (K, R) in enumerate(shapes):
+        if j < 4:
+            x, views = sxd, dict(input_view=((C, T, 1), (C, T, 5), (0, 0, j + 1)))
+        elif K == C:
+            x, views = sxd, dict(input_view=((C, T, 1), (C, T, 5), (0, 0, 0)))
+        else:
+            x, views = xhd, {}
+        act = gpu.ACT_SQUARED_RELU if j == 4 else gpu.ACT_NONE
+        mats[j].matmul_vec_op(x, single[j], act, **views)
+        ops.append((mats[j], x, group[j], act, j == 5, views))
+    gpu.matmul_vec_group(ops)
+    for j in range(len(shapes)):
+        assert_close(host(group[j]), truths[j], EPS, f"group op {j} vs float64")
+        assert torch.equal(group[j], single[j]), f"group op {j} differs from the single call"
+    # mixed token counts and a chunk-shaped op inside one list are split, not rejected
+    x32 = gen_f16(rng, (32, C), 1.0)
+    o32 = torch.empty((32, C), dtype=torch.float16, device="cuda")
+    o1 = torch.empty((1, C), dtype=torch.float16, device="cuda")
+    gpu.matmul_vec_group([(mats[0], dev(x32), o32, 0, False, {}), (mats[1], dev(x32[:1]), o1, 0, False, {})])
+    w0 = truth_matmul  # noqa: F841
+    torch.cuda.synchronize()
+    assert torch.isfinite(o32).all() and torch.isfinite(o1).all()
+    # an invalid op anywhere in the list fails the whole call before any launch
+    bad = torch.empty((1, C + 4), dtype=torch.float16, device="cuda")
+    group[0].fill_(7.0)
+    with pytest.raises(gpu.TensorError) as e:
+        gpu.matmul_vec_group([ops[0], (mats[1], sxd, bad, 0, False, dict(input_view=((C, T, 1), (C, T, 5), (0, 0, 2))))])
+    assert e.value.status == gpu.ERR_SHAPE
+    torch.cuda.synchronize()
+    assert (group[0] == 7.0).all()

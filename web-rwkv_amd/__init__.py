@@ -39,7 +39,9 @@ EXPORTS = [
     "wrq_init", "wrq_abi_version", "wrq_status_string", "wrq_last_error",
     "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
     "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
+    "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
 ]
+MAX_GROUP = 8
 
 
 class TensorError(RuntimeError):
@@ -60,6 +62,16 @@ class CView(C.Structure):
 
 class CTensorView(C.Structure):
     _fields_ = [("data", C.c_void_p), ("view", CView), ("dtype", C.c_int)]
+
+
+class CVecInt8Op(C.Structure):
+    _fields_ = [("matrix", C.POINTER(CTensor)), ("minmax", C.POINTER(CTensor)), ("input", C.POINTER(CTensorView)),
+                ("output", C.POINTER(CTensorView)), ("act", C.c_int), ("sparse", C.c_int)]
+
+
+class CVecNf4Op(C.Structure):
+    _fields_ = [("matrix", C.POINTER(CTensor)), ("quant", C.POINTER(CTensor)), ("absmax", C.POINTER(CTensor)),
+                ("input", C.POINTER(CTensorView)), ("output", C.POINTER(CTensorView)), ("act", C.c_int), ("sparse", C.c_int)]
 
 
 def build(verbose=False):
@@ -97,6 +109,8 @@ def lib():
         L.wrq_matmul_vec_nf4.argtypes = [vp, T, T, T, V, V, i, i]
         L.wrq_matmul_mat_int8.argtypes = [vp, V, T, V, V, i]
         L.wrq_matmul_mat_nf4.argtypes = [vp, V, T, T, V, V, i]
+        L.wrq_matmul_vec_int8_group.argtypes = [vp, C.POINTER(CVecInt8Op), i]
+        L.wrq_matmul_vec_nf4_group.argtypes = [vp, C.POINTER(CVecNf4Op), i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -181,6 +195,33 @@ class TensorOp:
     def matmul_mat_nf4(matrix, quant, absmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
         _check(lib().wrq_matmul_mat_nf4(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(quant)), C.byref(as_tensor(absmax)),
                                         C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
+
+
+def matmul_vec_group(ops):
+    """Independent decode products in shared launches (``wrq_matmul_vec_*_group``).
+
+    ``ops``: list of ``(matrix: Matrix, input, output, act, sparse, views: dict)``, all Int8 or all Fp4.
+    """
+    if not ops:
+        return
+    kind = ops[0][0].kind
+    keep = []  # ctypes structs must outlive the call
+    if kind == "Int8":
+        arr = (CVecInt8Op * len(ops))()
+        for k, (m, x, out, act, sparse, views) in enumerate(ops):
+            assert m.kind == kind
+            t = (as_tensor(m.w), as_tensor(m.m), as_view(x, views.get("input_view")), as_view(out, views.get("output_view")))
+            keep.append(t)
+            arr[k] = CVecInt8Op(C.pointer(t[0]), C.pointer(t[1]), C.pointer(t[2]), C.pointer(t[3]), act, int(sparse))
+        _check(lib().wrq_matmul_vec_int8_group(_stream(), arr, len(ops)))
+    else:
+        arr = (CVecNf4Op * len(ops))()
+        for k, (m, x, out, act, sparse, views) in enumerate(ops):
+            assert m.kind == kind
+            t = (as_tensor(m.w), as_tensor(m.q), as_tensor(m.m), as_view(x, views.get("input_view")), as_view(out, views.get("output_view")))
+            keep.append(t)
+            arr[k] = CVecNf4Op(C.pointer(t[0]), C.pointer(t[1]), C.pointer(t[2]), C.pointer(t[3]), C.pointer(t[4]), act, int(sparse))
+        _check(lib().wrq_matmul_vec_nf4_group(_stream(), arr, len(ops)))
 
 
 class Matrix:

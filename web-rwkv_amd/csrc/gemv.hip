@@ -3,22 +3,29 @@
 // out[t, r] = ACT( sum_k deq(W[r, k]) * x[t, k] )      (src/shaders/matmul_vec_int8.wgsl:57-115,
 //                                                        src/shaders/matmul_vec_nf4.wgsl:90-173)
 //
-// The kernels are HBM-bound: every packed byte is read exactly once with 16-byte
-// lane loads (1 KiB per wave instruction, contiguous along a weight row), all loads
-// of a lane are issued before the first use, and a workgroup owns ROWS consecutive
-// rows so the activation chunk a lane converts to f32 is reused ROWS times.
+// One launch serves a *group* of up to kMaxGroup independent products (the four
+// attention projections of a layer, or ffn.key + ffn.receptance): at batch 1 a single
+// 4096 x 4096 product is 17 MB, a few microseconds of HBM time, and a dispatch of its
+// own costs about as much again.
 //
-//   int8: 16 weights per lane load lie inside one 128-block, so the affine dequant
-//         factors out of the dot product:
-//             sum_j (u_j * s + m) * x_j = s * sum_j u_j x_j + m * sum_j x_j
-//         with s = (max - min) / 255; one v_cvt_f32_ubyteN + one FMA per weight.
-//   nf4:  32 weights per lane load lie inside one 64-block; the 16-entry table sits
-//         in LDS (16 consecutive dwords = 16 distinct banks, lanes reading the same
-//         entry are a broadcast, so lookups never conflict); absmax scales the
-//         32-term partial sum once.
-//
-// Lanes reduce with DPP inside rows of 16 and readlane across rows, waves through
-// one LDS exchange.  Accumulation is f32 throughout.
+// Structure (HBM-bound; every packed byte is read once, 16 bytes per lane, 1 KiB per
+// wave instruction, contiguous along a weight row):
+//   * resident workgroups of 8 waves (two per CU) stage the activation rows of the group
+//     in LDS once, then every wave pulls tasks -- ROWS consecutive weight rows over the
+//     full K -- from a strided sequence, so consecutive tasks land on different CUs;
+//   * a wave walks its rows in slices of 64 lanes x 16 bytes, loads of slice s+1 in
+//     flight while slice s is consumed, and finishes a task with a DPP/readlane
+//     reduction: no barrier and no LDS exchange after the prologue;
+//   * int8: the 16 weights of a lane load lie inside one 128-block, so the affine
+//     dequantisation factors out of the dot product,
+//         sum_j (u_j s + m) x_j = s sum_j u_j x_j + m sum_j x_j ,  s = (max - min) / 255:
+//     one v_cvt_f32_ubyteN and one FMA per weight;
+//   * nf4: a 256-entry LDS table maps a packed byte to its two f32 table values with one
+//     ds_read_b64 (2 address ops + 2 FMA per two weights instead of 4 + 2); each of 16
+//     lane groups reads its own copy of the table, which puts the 16 lanes served in
+//     one LDS cycle in 16 different bank pairs whatever bytes they hold; absmax scales
+//     the 32-term partial sum of a lane load, which lies inside one 64-block.
+// Accumulation is f32 throughout.
 #include "wrq_device.h"
 #include "wrq_host.h"
 
@@ -26,55 +33,158 @@
 
 namespace wrq {
 
-template <int ROWS, int TT, int NT>
-__device__ __forceinline__ void reduce_and_store(const MatmulArgs &a, float (&acc)[ROWS][TT],
-                                                 uint32_t row0, uint32_t t0, uint32_t b) {
-    constexpr int NW = NT / kWave;
-    __shared__ float red[NW][ROWS * TT];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+constexpr int kGemvWaves = 8;                 // waves per workgroup
+constexpr int kGemvThreads = kGemvWaves * 64; //
+constexpr int kTabCopies = 32;                // nf4 byte-pair table: copies (one per lane & 31), 256 B per entry
+constexpr size_t kTabBytes = 256 * kTabCopies * sizeof(float2);
+constexpr size_t kGemvLdsBudget = 128 * 1024;
+
+struct GemvProblem {
+    const uint8_t *w;      // packed rows of this product
+    const uint16_t *scale; // its scale blocks, indexed by flat element index as below
+    const void *x;         // first activation row (view offset applied)
+    void *out;             // first output row (view offset applied)
+    uint64_t e_base;       // flat element index of w's first element inside the matrix (batch offset)
+    uint64_t x_token_stride, out_token_stride;
+    uint32_t K, R;
+    uint32_t x_lds;      // byte offset of this product's activations in LDS
+    uint32_t task_begin; // first task of this product
+    int out_f16, act;
+};
+
+struct GemvGroup {
+    GemvProblem p[kMaxGroup];
+    const float *quant;
+    uint32_t n, T, total_tasks;
+    uint32_t x_pieces; // 16-byte pieces of activations staged in LDS (all products, TT tokens)
+};
+
+// What a wave needs to know about the task it is working on (all wave-uniform).
+struct TaskCtx;
+template <int ROWS, int TT>
+__device__ __forceinline__ void finish_task(const TaskCtx &p, float (&acc)[ROWS][TT], uint32_t t0, uint32_t T,
+                                            uint32_t lane);
+
+
+struct TaskCtx {
+    uint32_t task, K, R, row0, rows_valid, nslice, x_lds;
+    uint64_t e0;           // flat element index of (row0, 0) in the matrix
+    const uint8_t *wbase;  // packed bytes of (row0, 0)
+    const uint16_t *scale; // scale blocks of the product
+    void *out;
+    uint64_t out_token_stride;
+    int out_f16, act;
+};
+
+
+template <int ROWS, int TT>
+__device__ __forceinline__ void finish_task(const TaskCtx &p, float (&acc)[ROWS][TT], uint32_t t0, uint32_t T,
+                                            uint32_t lane) {
+    float mine = 0.0f;
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
+    for (int t = 0; t < TT; t++)
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
+        for (int r = 0; r < ROWS; r++) {
             const float s = wave_sum(acc[r][t]);
-            if (NW == 1) {
-                acc[r][t] = s;
-            } else if (lane == 0) {
-                red[wave][t * ROWS + r] = s;
-            }
+            if (lane == (uint32_t)(t * ROWS + r)) mine = s;
         }
-    if (NW > 1) __syncthreads();
-    if (tid < ROWS * TT) {
-        float s = 0.0f;
-        if (NW == 1) {
-            // every lane holds all sums; pick this lane's one without dynamic indexing
-#pragma unroll
-            for (int r = 0; r < ROWS; r++)
-#pragma unroll
-                for (int t = 0; t < TT; t++)
-                    if (tid == (uint32_t)(t * ROWS + r)) s = acc[r][t];
-        } else {
-#pragma unroll
-            for (int w = 0; w < NW; w++) s += red[w][tid];
-        }
-        const uint32_t r = row0 + tid % ROWS, t = t0 + tid / ROWS;
-        if (r < a.R && t < a.T) {
-            const uint64_t idx = (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + r;
-            store_out(a.out, a.out_f16, idx, act_apply(a.act, s));
-        }
+    if (lane < ROWS * TT) {
+        const uint32_t r = p.row0 + lane % ROWS, t = t0 + lane / ROWS;
+        if (r < p.R && t < T)
+            store_out(p.out, p.out_f16, (uint64_t)t * p.out_token_stride + r, act_apply(p.act, mine));
     }
 }
 
-template <typename XT, int ROWS, int TT, int NT>
-__global__ __launch_bounds__(NT) void gemv_int8_kernel(const MatmulArgs a) {
-    const uint32_t tid = threadIdx.x;
-    const uint32_t row0 = blockIdx.x * ROWS, t0 = blockIdx.y * TT, b = blockIdx.z;
-    const uint32_t K = a.K, nchunk = K >> 4;
-    const uint64_t e0 = ((uint64_t)b * a.R + row0) * K; // flat index of element (row0, 0)
-    const uint8_t *wbase = a.w + e0;
-    const uint32_t *mm = reinterpret_cast<const uint32_t *>(a.scale);
-    const XT *xb = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
-    const uint32_t rows_valid = min((uint32_t)ROWS, a.R - row0);
+template <int QUANT, typename XT, int ROWS, int SL, int TT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvGroup g) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int CH = QUANT == kInt8 ? 16 : 32; // weights per 16-byte lane load
+    float2 *tab = reinterpret_cast<float2 *>(smem);
+    uint8_t *xs = smem + (QUANT == kNf4 ? kTabBytes : 0);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform, and known to be
+    const uint32_t t0 = blockIdx.y * TT;
+    const uint32_t stride = gridDim.x * kGemvWaves;
+
+    auto setup = [&](uint32_t task) {
+        TaskCtx c;
+        c.task = task;
+        uint32_t pi = 0;
+        for (uint32_t i = 1; i < g.n; i++)
+            if (task >= g.p[i].task_begin) pi = i;
+        pi = __builtin_amdgcn_readfirstlane(pi); // uniform: the descriptor is read with scalar loads
+        const GemvProblem &p = g.p[pi];
+        c.K = p.K;
+        c.R = p.R;
+        c.x_lds = p.x_lds;
+        c.scale = p.scale;
+        c.out = p.out;
+        c.out_token_stride = p.out_token_stride;
+        c.out_f16 = p.out_f16;
+        c.act = p.act;
+        c.row0 = (task - p.task_begin) * ROWS;
+        c.rows_valid = min((uint32_t)ROWS, c.R - c.row0);
+        c.e0 = p.e_base + (uint64_t)c.row0 * c.K;
+        c.wbase = p.w + (QUANT == kInt8 ? (uint64_t)c.row0 * c.K : ((uint64_t)c.row0 * c.K) >> 1);
+        c.nslice = (c.K + 64 * SL * CH - 1) / (64 * SL * CH);
+        return c;
+    };
+    // 16-byte loads of slice s of a task: ROWS rows x SL chunks per lane, lanes along K (a wave
+    // instruction covers 1 KiB of one row); scale blocks beside them
+    auto issue = [&](const TaskCtx &c, uint32_t s, uint4(&wdst)[ROWS * SL], uint32_t(&sdst)[ROWS * SL]) {
+        const uint16_t *scale = c.scale;
+#pragma unroll
+        for (int i = 0; i < SL; i++) {
+            // lanes past the row end re-read its last chunk
+            const uint32_t k0 = min(((s * SL + i) * 64 + lane) * CH, c.K - CH);
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t rr = min((uint32_t)r, c.rows_valid - 1);
+                const uint64_t off = (uint64_t)rr * c.K + k0; // elements from (row0, 0)
+                if (QUANT == kInt8) {
+                    wdst[i * ROWS + r] = load128_stream(c.wbase + off);
+                    sdst[i * ROWS + r] = reinterpret_cast<const uint32_t *>(scale)[(c.e0 + off) >> 7];
+                } else {
+                    wdst[i * ROWS + r] = load128_stream(c.wbase + (off >> 1));
+                    sdst[i * ROWS + r] = scale[(c.e0 + off) >> 6];
+                }
+            }
+        }
+    };
+
+    // ---- prologue: the first weight slice is requested before anything else so that HBM is
+    // busy while the activations of the group (TT tokens) are staged in LDS
+    uint4 wa[ROWS * SL], wb[ROWS * SL];
+    uint32_t sa[ROWS * SL], sb[ROWS * SL]; // int8: (min, max) pair; nf4: absmax f16 in the low half
+    const uint32_t first = blockIdx.x + gridDim.x * wave;
+    bool have = first < g.total_tasks;
+    TaskCtx cur = setup(have ? first : 0);
+    if (have) issue(cur, 0, wa, sa);
+    for (uint32_t i = 0; i < g.n; i++) {
+        const GemvProblem &p = g.p[i];
+        const uint32_t per_row = p.K * sizeof(XT) / 16; // 16-byte pieces per token row
+        for (uint32_t j = tid; j < per_row * TT; j += kGemvThreads) {
+            const uint32_t t = j / per_row, c = j - t * per_row;
+            const uint32_t tt = min(t0 + t, g.T - 1);
+            const XT *src = reinterpret_cast<const XT *>(p.x) + (uint64_t)tt * p.x_token_stride;
+            *reinterpret_cast<uint4 *>(xs + p.x_lds + (size_t)j * 16) =
+                load128(reinterpret_cast<const uint8_t *>(src) + (size_t)c * 16);
+        }
+    }
+    if (QUANT == kNf4) {
+        // entry for byte v: (q[v & 15], q[v >> 4]); copy c of the table at tab[v * 32 + c]
+        for (uint32_t j = tid; j < 256 * kTabCopies; j += kGemvThreads) {
+            const uint32_t v = j / kTabCopies;
+            tab[j] = make_float2(g.quant[v & 15], g.quant[v >> 4]);
+        }
+    }
+    lds_barrier();
+
+    // byte address of table entry v for this lane: v * 256 + (lane & 31) * 8, built by one
+    // v_perm_b32 from the packed word (entry byte -> address byte 1, lane offset -> byte 0)
+    const uint32_t lane_off = (lane & (kTabCopies - 1)) * 8;
+    const uint8_t *tabb = reinterpret_cast<const uint8_t *>(tab);
 
     float acc[ROWS][TT];
 #pragma unroll
@@ -82,7 +192,137 @@ __global__ __launch_bounds__(NT) void gemv_int8_kernel(const MatmulArgs a) {
 #pragma unroll
         for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
 
+    // consume slice s of task c from (wv, sc); the last slice of a task reduces and stores
+    auto compute = [&](const TaskCtx &c, uint32_t s, const uint4(&wv)[ROWS * SL], const uint32_t(&sc)[ROWS * SL]) {
+        const uint32_t K = c.K;
+        const XT *xl = reinterpret_cast<const XT *>(xs + c.x_lds);
+#pragma unroll
+        for (int i = 0; i < SL; i++) {
+            const uint32_t k0 = ((s * SL + i) * 64 + lane) * CH;
+            if (k0 < K) {
+#pragma unroll
+                for (int t = 0; t < TT; t++) {
+                    float xf[CH];
+                    const XT *xp = xl + (size_t)t * K + k0;
+                    if constexpr (sizeof(XT) == 2) {
+#pragma unroll
+                        for (int u = 0; u < CH / 8; u++) unpack8h(*reinterpret_cast<const uint4 *>(xp + 8 * u), xf + 8 * u);
+                    } else {
+#pragma unroll
+                        for (int u = 0; u < CH / 4; u++) {
+                            const float4 v = *reinterpret_cast<const float4 *>(xp + 4 * u);
+                            xf[4 * u] = v.x; xf[4 * u + 1] = v.y; xf[4 * u + 2] = v.z; xf[4 * u + 3] = v.w;
+                        }
+                    }
+                    if (QUANT == kInt8) {
+                        float sx = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < 16; j++) sx += xf[j];
+#pragma unroll
+                        for (int r = 0; r < ROWS; r++) {
+                            const uint4 &v = wv[i * ROWS + r];
+                            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                            float pr = 0.0f;
+#pragma unroll
+                            for (int j = 0; j < 16; j++)
+                                pr = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xffu), xf[j], pr);
+                            const uint32_t mm = sc[i * ROWS + r];
+                            const float mn = h2f((uint16_t)(mm & 0xffffu));
+                            const float mx = h2f((uint16_t)(mm >> 16));
+                            const float sc1 = (mx - mn) * (1.0f / 255.0f);
+                            acc[r][t] = fmaf(sc1, pr, fmaf(mn, sx, acc[r][t]));
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < ROWS; r++) {
+                            const uint4 &v = wv[i * ROWS + r];
+                            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                            float pr = 0.0f;
+#pragma unroll
+                            for (int j = 0; j < 16; j++) {
+                                const uint32_t addr = __builtin_amdgcn_perm(lane_off, w[j >> 2], 0x0c0c0004u | ((j & 3) << 8));
+                                const float2 e = *reinterpret_cast<const float2 *>(tabb + addr);
+                                pr = fmaf(e.x, xf[2 * j], pr);
+                                pr = fmaf(e.y, xf[2 * j + 1], pr);
+                            }
+                            acc[r][t] = fmaf(pr, h2f((uint16_t)sc[i * ROWS + r]), acc[r][t]);
+                        }
+                    }
+                }
+            }
+        }
+        if (s + 1 == c.nslice) {
+            finish_task<ROWS, TT>(c, acc, t0, g.T, lane);
+#pragma unroll
+            for (int r = 0; r < ROWS; r++)
+#pragma unroll
+                for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
+        }
+    };
+    // the step after (c, s): next slice of the task, or slice 0 of this wave's next task;
+    // consecutive tasks go to different workgroups first, then to the next wave
+    auto advance = [&](TaskCtx &c, uint32_t &s) {
+        if (s + 1 < c.nslice) {
+            s++;
+            return true;
+        }
+        const uint32_t next = c.task + stride;
+        if (next >= g.total_tasks) return false;
+        c = setup(next);
+        s = 0;
+        return true;
+    };
+
+    // two register buffers in ping-pong: the loads of step i+1 are in flight while step i is consumed
+    uint32_t s = 0;
+    while (have) {
+        TaskCtx nx = cur;
+        uint32_t ns = s;
+        const bool nhave = advance(nx, ns);
+        if (nhave) issue(nx, ns, wb, sb);
+        compute(cur, s, wa, sa);
+        if (!nhave) break;
+        cur = nx;
+        s = ns;
+        have = advance(nx, ns);
+        if (have) issue(nx, ns, wa, sa);
+        compute(cur, s, wb, sb);
+        cur = nx;
+        s = ns;
+    }
+}
+
+// int8, one token: one workgroup per task, everything it needs requested at once.  At the
+// 7B shapes the whole matrix is a fraction of what the CUs can keep in flight, so a task
+// (ROWS rows, NT lanes along K) issues all its loads -- activations first, they are needed
+// first and come from L2 -- and consumes the rows in arrival order; waves meet once in LDS.
+template <typename XT, int ROWS, int NT>
+__global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g) {
+    constexpr int NW = NT / kWave;
+    __shared__ float red[NW][ROWS];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t task = blockIdx.x;
+    uint32_t pi = 0;
+    for (uint32_t i = 1; i < g.n; i++)
+        if (task >= g.p[i].task_begin) pi = i;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const GemvProblem &p = g.p[pi];
+    const uint32_t K = p.K, nchunk = K >> 4;
+    const uint32_t row0 = (task - p.task_begin) * ROWS;
+    const uint32_t rows_valid = min((uint32_t)ROWS, p.R - row0);
+    const uint64_t e0 = p.e_base + (uint64_t)row0 * K; // flat index of element (row0, 0)
+    const uint8_t *wbase = p.w + (uint64_t)row0 * K;
+    const uint32_t *mm = reinterpret_cast<const uint32_t *>(p.scale);
+    const XT *x = reinterpret_cast<const XT *>(p.x);
+
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+
     for (uint32_t c = tid; c < nchunk; c += NT) {
+        float xf[16];
+        load_x<XT, 16>(x + ((uint64_t)c << 4), xf);
         uint4 wv[ROWS];
         uint32_t sc[ROWS];
 #pragma unroll
@@ -92,78 +332,43 @@ __global__ __launch_bounds__(NT) void gemv_int8_kernel(const MatmulArgs a) {
             wv[r] = load128_stream(wbase + off);
             sc[r] = mm[(e0 + off) >> 7];
         }
+        float sx = 0.0f;
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
-            const uint32_t tt = min(t0 + t, a.T - 1);
-            float xf[16];
-            load_x<XT, 16>(xb + (uint64_t)tt * a.x_token_stride + ((uint64_t)c << 4), xf);
-            float sx = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 16; j++) sx += xf[j];
-#pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float p = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; j++)
-                    p = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xffu), xf[j], p);
-                const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
-                const float mx = h2f((uint16_t)(sc[r] >> 16));
-                const float s = (mx - mn) * (1.0f / 255.0f);
-                acc[r][t] = fmaf(s, p, fmaf(mn, sx, acc[r][t]));
-            }
-        }
-    }
-    reduce_and_store<ROWS, TT, NT>(a, acc, row0, t0, b);
-}
-
-template <typename XT, int ROWS, int TT, int NT>
-__global__ __launch_bounds__(NT) void gemv_nf4_kernel(const MatmulArgs a) {
-    __shared__ float q[16];
-    const uint32_t tid = threadIdx.x;
-    if (tid < 16) q[tid] = a.quant[tid];
-    __syncthreads();
-
-    const uint32_t row0 = blockIdx.x * ROWS, t0 = blockIdx.y * TT, b = blockIdx.z;
-    const uint32_t K = a.K, nchunk = K >> 5;
-    const uint64_t e0 = ((uint64_t)b * a.R + row0) * K; // flat element index of (row0, 0)
-    const uint8_t *wbase = a.w + (e0 >> 1);
-    const XT *xb = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
-    const uint32_t rows_valid = min((uint32_t)ROWS, a.R - row0);
-
-    float acc[ROWS][TT];
-#pragma unroll
-    for (int r = 0; r < ROWS; r++)
-#pragma unroll
-        for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
-
-    for (uint32_t c = tid; c < nchunk; c += NT) {
-        uint4 wv[ROWS];
-        float am[ROWS];
+        for (int j = 0; j < 16; j++) sx += xf[j];
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
-            const uint32_t rr = min((uint32_t)r, rows_valid - 1);
-            const uint64_t off = (uint64_t)rr * K + ((uint64_t)c << 5); // elements
-            wv[r] = load128_stream(wbase + (off >> 1));
-            am[r] = h2f(a.scale[(e0 + off) >> 6]);
-        }
+            const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+            float pr = 0.0f;
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
-            const uint32_t tt = min(t0 + t, a.T - 1);
-            float xf[32];
-            load_x<XT, 32>(xb + (uint64_t)tt * a.x_token_stride + ((uint64_t)c << 5), xf);
-#pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float p = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 32; j++)
-                    p = fmaf(q[(w[j >> 3] >> (4 * (j & 7))) & 0xfu], xf[j], p);
-                acc[r][t] = fmaf(p, am[r], acc[r][t]);
-            }
+            for (int j = 0; j < 16; j++) pr = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xffu), xf[j], pr);
+            const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
+            const float mx = h2f((uint16_t)(sc[r] >> 16));
+            const float s = (mx - mn) * (1.0f / 255.0f);
+            acc[r] = fmaf(s, pr, fmaf(mn, sx, acc[r]));
         }
     }
-    reduce_and_store<ROWS, TT, NT>(a, acc, row0, t0, b);
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const float s = wave_sum(acc[r]);
+        if (NW == 1)
+            acc[r] = s;
+        else if (lane == 0)
+            red[wave][r] = s;
+    }
+    if (NW > 1) __syncthreads();
+    if (tid < ROWS) {
+        float s = 0.0f;
+        if (NW == 1) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++)
+                if (tid == (uint32_t)r) s = acc[r];
+        } else {
+#pragma unroll
+            for (int w = 0; w < NW; w++) s += red[w][tid];
+        }
+        const uint32_t r = row0 + tid;
+        if (r < p.R) store_out(p.out, p.out_f16, r, act_apply(p.act, s));
+    }
 }
 
 // Any K the reference accepts (K % 4 for int8, K % 8 for nf4, with blocks that may
@@ -218,80 +423,203 @@ __global__ __launch_bounds__(64) void gemv_generic_kernel(const MatmulArgs a) {
 
 namespace {
 
-template <typename XT, int ROWS, int TT, int NT>
-void launch_fast(hipStream_t stream, Quant quant, const MatmulArgs &a) {
-    dim3 grid((a.R + ROWS - 1) / ROWS, (a.T + TT - 1) / TT, a.B);
-    if (quant == kInt8)
-        hipLaunchKernelGGL((gemv_int8_kernel<XT, ROWS, TT, NT>), grid, dim3(NT), 0, stream, a);
-    else
-        hipLaunchKernelGGL((gemv_nf4_kernel<XT, ROWS, TT, NT>), grid, dim3(NT), 0, stream, a);
-}
-
-template <typename XT, int ROWS, int TT>
-void launch_fast_nt(hipStream_t stream, Quant quant, const MatmulArgs &a, int nt) {
-    if (nt >= 256)
-        launch_fast<XT, ROWS, TT, 256>(stream, quant, a);
-    else if (nt >= 128)
-        launch_fast<XT, ROWS, TT, 128>(stream, quant, a);
-    else
-        launch_fast<XT, ROWS, TT, 64>(stream, quant, a);
-}
-
-template <typename XT>
-void launch_fast_xt(hipStream_t stream, Quant quant, const MatmulArgs &a, int rows, int tt, int nt) {
-    if (tt >= 4)
-        launch_fast_nt<XT, 4, 4>(stream, quant, a, nt);
-    else if (tt == 2)
-        launch_fast_nt<XT, 4, 2>(stream, quant, a, nt);
-    else if (rows >= 8)
-        launch_fast_nt<XT, 8, 1>(stream, quant, a, nt);
-    else
-        launch_fast_nt<XT, 4, 1>(stream, quant, a, nt);
-}
-
 int env_int(const char *name, int fallback) {
     const char *s = getenv(name);
     return (s && *s) ? atoi(s) : fallback;
 }
 
-} // namespace
+template <int QUANT, typename XT, int ROWS, int SL, int TT>
+int launch_group_rt(hipStream_t stream, const GemvGroup &g, uint32_t grid_x, uint32_t grid_y, size_t lds) {
+    auto *kern = &gemv_kernel<QUANT, XT, ROWS, SL, TT>;
+    if (lds > 48 * 1024) {
+        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                           (int)kGemvLdsBudget);
+        (void)once;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid_x, grid_y), dim3(kGemvThreads), lds, stream, g);
+    return check_launch("matmul_vec");
+}
 
-int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
-    if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
+// (rows per task, chunks per lane and row in one slice): rows * sl 16-byte loads per lane are in
+// flight per register buffer, two buffers
+template <int QUANT, typename XT>
+int launch_group_xt(hipStream_t stream, const GemvGroup &g, int rows, int sl, int tt, uint32_t grid_x,
+                    uint32_t grid_y, size_t lds) {
+    if (tt == 4) return launch_group_rt<QUANT, XT, 4, 1, 4>(stream, g, grid_x, grid_y, lds);
+    if (tt == 2) return launch_group_rt<QUANT, XT, 4, 1, 2>(stream, g, grid_x, grid_y, lds);
+    if (rows == 2 && sl == 4) return launch_group_rt<QUANT, XT, 2, 4, 1>(stream, g, grid_x, grid_y, lds);
+    if (rows == 2 && sl == 2) return launch_group_rt<QUANT, XT, 2, 2, 1>(stream, g, grid_x, grid_y, lds);
+    if (rows == 4 && sl == 2) return launch_group_rt<QUANT, XT, 4, 2, 1>(stream, g, grid_x, grid_y, lds);
+    if (rows == 4 && sl == 4) return launch_group_rt<QUANT, XT, 4, 4, 1>(stream, g, grid_x, grid_y, lds);
+    if (rows == 2) return launch_group_rt<QUANT, XT, 2, 1, 1>(stream, g, grid_x, grid_y, lds);
+    return launch_group_rt<QUANT, XT, 4, 1, 1>(stream, g, grid_x, grid_y, lds);
+}
+
+template <typename XT, int ROWS>
+int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+    const dim3 grid(g.total_tasks);
+    if (nt >= 256)
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, g);
+    else if (nt >= 128)
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64>), grid, dim3(64), 0, stream, g);
+    return check_launch("matmul_vec_int8");
+}
+
+bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
     const uint32_t chunk = quant == kInt8 ? 16 : 32;
     const size_t xs = in_f16 ? 2 : 4;
-    const bool aligned = (a.K % chunk == 0) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
-                         ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0);
-    if (a.R > 0x7fffffffu || a.T > 65535u || a.B > 65535u)
+    return (a.K % chunk == 0) && (a.K >= chunk) && ((uintptr_t)a.w % 16 == 0) && ((uintptr_t)a.x % 16 == 0) &&
+           ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0);
+}
+
+int launch_generic(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
+    if (a.T > 65535u || a.B > 65535u)
         return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.T > a.B ? a.T : a.B, 65535u);
-    if (!aligned) {
-        dim3 grid(a.R, a.T, a.B);
-        if (quant == kInt8) {
-            if (in_f16)
-                hipLaunchKernelGGL((gemv_generic_kernel<__half, kInt8>), grid, dim3(64), 0, stream, a);
-            else
-                hipLaunchKernelGGL((gemv_generic_kernel<float, kInt8>), grid, dim3(64), 0, stream, a);
-        } else {
-            if (in_f16)
-                hipLaunchKernelGGL((gemv_generic_kernel<__half, kNf4>), grid, dim3(64), 0, stream, a);
-            else
-                hipLaunchKernelGGL((gemv_generic_kernel<float, kNf4>), grid, dim3(64), 0, stream, a);
-        }
-        return check_launch("matmul_vec (generic)");
+    dim3 grid(a.R, a.T, a.B);
+    if (quant == kInt8) {
+        if (in_f16)
+            hipLaunchKernelGGL((gemv_generic_kernel<__half, kInt8>), grid, dim3(64), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemv_generic_kernel<float, kInt8>), grid, dim3(64), 0, stream, a);
+    } else {
+        if (in_f16)
+            hipLaunchKernelGGL((gemv_generic_kernel<__half, kNf4>), grid, dim3(64), 0, stream, a);
+        else
+            hipLaunchKernelGGL((gemv_generic_kernel<float, kNf4>), grid, dim3(64), 0, stream, a);
     }
-    const uint32_t nchunk = a.K / chunk;
-    // workgroup width: enough lanes to cover a row in one pass, at most 256
-    int nt = nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
-    int tt = a.T >= 3 ? 4 : (int)a.T;
-    // rows per workgroup: 8 unless that leaves too few workgroups to fill 256 CUs
-    int rows = (a.R / 8) * a.B >= 512 ? 8 : 4;
-    rows = env_int("WRQ_GEMV_ROWS", rows);
-    nt = env_int("WRQ_GEMV_NT", nt);
-    if (in_f16)
-        launch_fast_xt<__half>(stream, quant, a, rows, tt, nt);
-    else
-        launch_fast_xt<float>(stream, quant, a, rows, tt, nt);
-    return check_launch("matmul_vec");
+    return check_launch("matmul_vec (generic)");
+}
+
+} // namespace
+
+// `n` independent products with the same quantisation, input type and token count.
+// Products that do not fit the streaming kernel (odd K, unaligned views, activations too
+// large for LDS together) are launched one by one on the generic kernel.
+int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n) {
+    if (n <= 0) return WRQ_OK;
+    const uint32_t T = args[0].T;
+    const int tt = T >= 3 ? 4 : (int)T;
+    const size_t xsz = in_f16 ? 2 : 4;
+    const size_t lds_base = quant == kNf4 ? kTabBytes : 0;
+
+    int i = 0;
+    while (i < n) {
+        GemvGroup g{};
+        g.quant = args[i].quant;
+        g.T = T;
+        size_t lds = lds_base;
+        uint32_t tasks = 0;
+        uint64_t bytes = 0;
+        // rows per task: 4, or 2 when the group is too small to give every wave of 256 CUs a task
+        uint64_t rows_total = 0;
+        for (int j = i; j < n; j++) rows_total += (uint64_t)args[j].R * args[j].B;
+        // int8 at one token: the one-shot kernel (4 rows per workgroup; 8 once that still gives
+        // every CU eight workgroups)
+        const bool oneshot = quant == kInt8 && T == 1 && env_int("WRQ_GEMV_ONESHOT", 1);
+        int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
+        if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
+        // chunks per lane: cover a whole row at once when it is short enough
+        const uint32_t groups = (args[i].K / (quant == kInt8 ? 16 : 32) + 63) / 64;
+        int sl = groups >= 4 ? 4 : groups >= 2 ? 2 : 1;
+        if (rows == 4 && sl == 4) sl = 2;
+        rows = env_int("WRQ_GEMV_ROWS", rows);
+        sl = env_int("WRQ_GEMV_SL", sl);
+        if (tt > 1) rows = 4, sl = 1;
+        if (oneshot && rows != 8) rows = 4;
+        while (i < n && g.n < (uint32_t)kMaxGroup) {
+            const MatmulArgs &a = args[i];
+            if (a.R == 0 || a.T == 0 || a.B == 0) {
+                i++;
+                continue;
+            }
+            const size_t need = (size_t)a.K * tt * xsz;
+            if (!fast_ok(quant, in_f16, a) || lds_base + need > kGemvLdsBudget) {
+                if (g.n) break; // flush what is collected, then come back to this one
+                const int s = launch_generic(stream, quant, in_f16, a);
+                if (s != WRQ_OK) return s;
+                i++;
+                continue;
+            }
+            if (a.B > 1 && g.n + a.B > (uint32_t)kMaxGroup && g.n) break;
+            if (lds + need * a.B > kGemvLdsBudget && g.n) break;
+            // the batch axis unrolls into products of its own
+            uint32_t b = 0;
+            for (; b < a.B && g.n < (uint32_t)kMaxGroup && lds + need <= kGemvLdsBudget; b++) {
+                GemvProblem &p = g.p[g.n++];
+                const uint64_t e_base = (uint64_t)b * a.R * a.K;
+                p.w = a.w + (quant == kInt8 ? e_base : e_base >> 1);
+                p.scale = a.scale;
+                p.e_base = e_base;
+                p.x = static_cast<const uint8_t *>(a.x) + (uint64_t)b * a.x_batch_stride * xsz;
+                p.out = static_cast<uint8_t *>(a.out) + (uint64_t)b * a.out_batch_stride * (a.out_f16 ? 2 : 4);
+                p.x_token_stride = a.x_token_stride;
+                p.out_token_stride = a.out_token_stride;
+                p.K = a.K;
+                p.R = a.R;
+                p.x_lds = (uint32_t)(lds - lds_base);
+                p.task_begin = tasks;
+                p.out_f16 = a.out_f16;
+                p.act = a.act;
+                lds += need;
+                tasks += (a.R + rows - 1) / rows;
+                bytes += (uint64_t)a.R * a.K;
+            }
+            if (b < a.B) {
+                // a batch too deep for one group: finish it with single-product launches
+                for (; b < a.B; b++) {
+                    MatmulArgs one = a;
+                    const uint64_t e_base = (uint64_t)b * a.R * a.K;
+                    // keep flat scale indexing: shift pointers instead of the batch index
+                    if ((quant == kInt8 ? e_base % 128 : e_base % 64) != 0) return fail(WRQ_ERR_UNSUPPORTED, "batched matrix rows not block aligned");
+                    one.B = 1;
+                    one.w = a.w + (quant == kInt8 ? e_base : e_base >> 1);
+                    one.scale = a.scale + (quant == kInt8 ? 2 * (e_base >> 7) : (e_base >> 6));
+                    one.x = static_cast<const uint8_t *>(a.x) + (uint64_t)b * a.x_batch_stride * xsz;
+                    one.out = static_cast<uint8_t *>(a.out) + (uint64_t)b * a.out_batch_stride * (a.out_f16 ? 2 : 4);
+                    const int s = launch_gemv_group(stream, quant, in_f16, &one, 1);
+                    if (s != WRQ_OK) return s;
+                }
+            }
+            i++;
+        }
+        if (!g.n) continue;
+        g.total_tasks = tasks;
+        if (oneshot) {
+            const uint32_t nchunk = g.p[0].K / 16;
+            int nt = nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
+            nt = env_int("WRQ_GEMV_NT", nt);
+            int s1;
+            if (rows == 8)
+                s1 = in_f16 ? launch_oneshot_nt<__half, 8>(stream, g, nt) : launch_oneshot_nt<float, 8>(stream, g, nt);
+            else
+                s1 = in_f16 ? launch_oneshot_nt<__half, 4>(stream, g, nt) : launch_oneshot_nt<float, 4>(stream, g, nt);
+            if (s1 != WRQ_OK) return s1;
+            continue;
+        }
+        g.x_pieces = (uint32_t)((lds - lds_base) / 16);
+        const uint32_t want = (tasks + kGemvWaves - 1) / kGemvWaves;
+        const uint32_t cap = quant == kNf4 ? 256u : 512u; // resident workgroups: the nf4 table leaves LDS for one per CU
+        uint32_t grid_x = want < cap ? want : cap;
+        grid_x = (uint32_t)env_int("WRQ_GEMV_GRID", (int)grid_x);
+        const uint32_t grid_y = (T + tt - 1) / tt;
+        if (grid_y > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", T, 65535u * 4);
+        int s;
+        if (quant == kInt8)
+            s = in_f16 ? launch_group_xt<kInt8, __half>(stream, g, rows, sl, tt, grid_x, grid_y, lds)
+                       : launch_group_xt<kInt8, float>(stream, g, rows, sl, tt, grid_x, grid_y, lds);
+        else
+            s = in_f16 ? launch_group_xt<kNf4, __half>(stream, g, rows, sl, tt, grid_x, grid_y, lds)
+                       : launch_group_xt<kNf4, float>(stream, g, rows, sl, tt, grid_x, grid_y, lds);
+        if (s != WRQ_OK) return s;
+    }
+    return WRQ_OK;
+}
+
+int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
+    return launch_gemv_group(stream, quant, in_f16, &a, 1);
 }
 
 } // namespace wrq

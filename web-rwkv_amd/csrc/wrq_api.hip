@@ -105,9 +105,15 @@ enum Entry { kVec, kMat };
 
 // Shared body of the four product entry points.  `mshape` is the matrix shape in
 // bytes-per-row terms as the reference sees it: [K, R, B, 1] (int8) or [K/2, R, B, 1] (nf4).
-int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Shape4 &mshape,
-           const wrq_tensor *scale, const wrq_tensor *table, const wrq_tensor_view *input,
-           const wrq_tensor_view *output, int act) {
+struct Prepared {
+    MatmulArgs a;
+    int in_f16;
+    bool mfma; // route to the matrix-core kernel
+};
+
+int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const wrq_tensor *scale,
+            const wrq_tensor *table, const wrq_tensor_view *input, const wrq_tensor_view *output, int act,
+            Prepared &out) {
     if (act < WRQ_ACT_NONE || act > WRQ_ACT_SILU) return fail(WRQ_ERR_UNSUPPORTED, "unknown activation %d", act);
     const Shape4 os = shape_of(output->view.shape), is = shape_of(input->view.shape);
     const uint64_t m = os.d[0], n = os.d[1], b = os.d[2], k = is.d[0];
@@ -148,7 +154,8 @@ int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Sh
     }
     if (m > 0xffffffffull || n > 0xffffffffull || k > 0xffffffffull) return fail(WRQ_ERR_SIZE, "data size not match");
 
-    MatmulArgs a{};
+    MatmulArgs &a = out.a;
+    a = MatmulArgs{};
     a.w = static_cast<const uint8_t *>(w);
     a.scale = static_cast<const uint16_t *>(scale->data);
     a.quant = table ? static_cast<const float *>(table->data) : nullptr;
@@ -169,8 +176,40 @@ int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Sh
                          ((uintptr_t)a.out % (4 * osz) == 0) && ((a.out_token_stride * osz) % (4 * osz) == 0) &&
                          ((a.out_batch_stride * osz) % (4 * osz) == 0);
     const bool chunk = entry == kMat ? true : n >= 16;
-    if (chunk && mfma_ok) return launch_gemm(stream, quant, in_f16, a);
-    return launch_gemv(stream, quant, in_f16, a);
+    out.in_f16 = in_f16;
+    out.mfma = chunk && mfma_ok;
+    return WRQ_OK;
+}
+
+int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Shape4 &mshape,
+           const wrq_tensor *scale, const wrq_tensor *table, const wrq_tensor_view *input,
+           const wrq_tensor_view *output, int act) {
+    Prepared p;
+    WRQ_TRY(prepare(entry, quant, w, mshape, scale, table, input, output, act, p));
+    if (p.mfma) return launch_gemm(stream, quant, p.in_f16, p.a);
+    return launch_gemv(stream, quant, p.in_f16, p.a);
+}
+
+// Runs of consecutive decode-shaped ops with one input type and token count share launches.
+int dispatch_group(hipStream_t stream, Quant quant, const Prepared *ops, int n) {
+    int i = 0;
+    while (i < n) {
+        if (ops[i].mfma) {
+            WRQ_TRY(launch_gemm(stream, quant, ops[i].in_f16, ops[i].a));
+            i++;
+            continue;
+        }
+        MatmulArgs run[kMaxGroup];
+        int m = 0;
+        while (i + m < n && m < kMaxGroup && !ops[i + m].mfma && ops[i + m].in_f16 == ops[i].in_f16 &&
+               ops[i + m].a.T == ops[i].a.T && ops[i + m].a.quant == ops[i].a.quant) {
+            run[m] = ops[i + m].a;
+            m++;
+        }
+        WRQ_TRY(launch_gemv_group(stream, quant, ops[i].in_f16, run, m));
+        i += m;
+    }
+    return WRQ_OK;
 }
 
 } // namespace
@@ -269,6 +308,41 @@ int wrq_matmul_vec_nf4(wrq_stream stream, const wrq_tensor *matrix, const wrq_te
     WRQ_TRY(need_view(output, "output", true));
     return matmul(static_cast<hipStream_t>(stream), kVec, kNf4, matrix->data, shape_of(matrix->shape), absmax, quant,
                   input, output, act);
+}
+
+int wrq_matmul_vec_int8_group(wrq_stream stream, const wrq_vec_int8_op *ops, int count) {
+    if (count < 0 || count > WRQ_MAX_GROUP) return fail(WRQ_ERR_SIZE, "data size not match: %d vs. %d", count, WRQ_MAX_GROUP);
+    if (count == 0) return WRQ_OK;
+    WRQ_TRY(need(ops, "ops"));
+    Prepared prepared[WRQ_MAX_GROUP];
+    for (int i = 0; i < count; i++) { // every op is checked before anything is launched
+        const wrq_vec_int8_op &o = ops[i];
+        WRQ_TRY(need_tensor(o.matrix, "matrix"));
+        WRQ_TRY(need_tensor(o.minmax, "minmax"));
+        WRQ_TRY(need_view(o.input, "input", true));
+        WRQ_TRY(need_view(o.output, "output", true));
+        WRQ_TRY(prepare(kVec, kInt8, o.matrix->data, shape_of(o.matrix->shape), o.minmax, nullptr, o.input, o.output,
+                        o.act, prepared[i]));
+    }
+    return dispatch_group(static_cast<hipStream_t>(stream), kInt8, prepared, count);
+}
+
+int wrq_matmul_vec_nf4_group(wrq_stream stream, const wrq_vec_nf4_op *ops, int count) {
+    if (count < 0 || count > WRQ_MAX_GROUP) return fail(WRQ_ERR_SIZE, "data size not match: %d vs. %d", count, WRQ_MAX_GROUP);
+    if (count == 0) return WRQ_OK;
+    WRQ_TRY(need(ops, "ops"));
+    Prepared prepared[WRQ_MAX_GROUP];
+    for (int i = 0; i < count; i++) {
+        const wrq_vec_nf4_op &o = ops[i];
+        WRQ_TRY(need_tensor(o.matrix, "matrix"));
+        WRQ_TRY(need_tensor(o.quant, "quant"));
+        WRQ_TRY(need_tensor(o.absmax, "absmax"));
+        WRQ_TRY(need_view(o.input, "input", true));
+        WRQ_TRY(need_view(o.output, "output", true));
+        WRQ_TRY(prepare(kVec, kNf4, o.matrix->data, shape_of(o.matrix->shape), o.absmax, o.quant, o.input, o.output,
+                        o.act, prepared[i]));
+    }
+    return dispatch_group(static_cast<hipStream_t>(stream), kNf4, prepared, count);
 }
 
 int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,

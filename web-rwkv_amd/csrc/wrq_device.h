@@ -84,6 +84,14 @@ __device__ __forceinline__ uint2 load64_stream(const void *p) {
     return make_uint2(v.x, v.y);
 }
 
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in
+// flight across it (a full __syncthreads() would wait for them).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Sum over the 64 lanes of a wave; the result is valid in every lane.
 __device__ __forceinline__ float wave_sum(float v) {
     // within rows of 16 lanes: quad permutes, then half-mirror and mirror

@@ -22,8 +22,13 @@ int launch_quant_nf4(hipStream_t stream, const void *in, const void *quant, void
 
 enum Quant { kInt8 = 0, kNf4 = 1 };
 
+constexpr int kMaxGroup = 8; // products per grouped decode launch
+
 // Decode-shaped products (few tokens): VALU dequantisation, wave reductions.
 int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+// The same for `n` independent products of one quantisation, input type and token count,
+// in as few launches as their activations fit in LDS together.
+int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
 // Chunk-shaped products (T >= 16): f16 MFMA.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
 
