@@ -292,16 +292,38 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvGroup g) {
     }
 }
 
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// acc + a.lo * b.lo + a.hi * b.hi on two packed f16 pairs, f32 accumulate (v_dot2_f32_f16)
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b), acc, false);
+}
+
+// Sum inside rows of 16 lanes (DPP only); every lane of a row ends with the row's sum.
+__device__ __forceinline__ float row_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xf, 0xf, true)); // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xf, 0xf, true)); // row_mirror
+    return v;
+}
+
 // int8, one token: one workgroup per task, everything it needs requested at once.  At the
 // 7B shapes the whole matrix is a fraction of what the CUs can keep in flight, so a task
 // (ROWS rows, NT lanes along K) issues all its loads -- activations first, they are needed
-// first and come from L2 -- and consumes the rows in arrival order; waves meet once in LDS.
+// first and come from L2 -- and consumes the rows in arrival order.
+//
+// With f16 activations the products run on v_dot2_f32_f16: one v_perm_b32 turns two codes
+// into the f16 pair (1024 + u0, 1024 + u1) (exact), the pair meets two activations in one
+// dot2, and the bias joins the affine term:
+//     sum_j (u_j s + m) x_j = s * sum_j (1024 + u_j) x_j + (m - 1024 s) * sum_j x_j
+// -- one VALU op per weight.  f32 activations keep v_cvt_f32_ubyteN + FMA.
+// Lanes reduce inside DPP rows; rows and waves meet once in LDS.
 template <typename XT, int ROWS, int NT>
 __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g) {
-    constexpr int NW = NT / kWave;
-    __shared__ float red[NW][ROWS];
-    const uint32_t tid = threadIdx.x, lane = tid & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int NROW16 = NT / 16; // DPP rows per workgroup
+    __shared__ float red[ROWS][NROW16];
+    const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
     for (uint32_t i = 1; i < g.n; i++)
@@ -321,8 +343,10 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
 
     for (uint32_t c = tid; c < nchunk; c += NT) {
-        float xf[16];
-        load_x<XT, 16>(x + ((uint64_t)c << 4), xf);
+        uint4 xv[sizeof(XT) == 2 ? 2 : 4];
+#pragma unroll
+        for (int i = 0; i < (sizeof(XT) == 2 ? 2 : 4); i++)
+            xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)c << 4)) + 16 * i);
         uint4 wv[ROWS];
         uint32_t sc[ROWS];
 #pragma unroll
@@ -332,42 +356,66 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
             wv[r] = load128_stream(wbase + off);
             sc[r] = mm[(e0 + off) >> 7];
         }
-        float sx = 0.0f;
+        if constexpr (sizeof(XT) == 2) {
+            const uint32_t xd[8] = {xv[0].x, xv[0].y, xv[0].z, xv[0].w, xv[1].x, xv[1].y, xv[1].z, xv[1].w};
+            float sx = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 16; j++) sx += xf[j];
+            for (int j = 0; j < 8; j++) sx = dot2(xd[j], 0x3c003c00u, sx); // (1.0, 1.0)
 #pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-            float pr = 0.0f;
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+                float pr = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 16; j++) pr = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xffu), xf[j], pr);
-            const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
-            const float mx = h2f((uint16_t)(sc[r] >> 16));
-            const float s = (mx - mn) * (1.0f / 255.0f);
-            acc[r] = fmaf(s, pr, fmaf(mn, sx, acc[r]));
+                for (int d = 0; d < 4; d++) {
+                    pr = dot2(__builtin_amdgcn_perm(0x64646464u, w[d], 0x04010400u), xd[2 * d], pr);
+                    pr = dot2(__builtin_amdgcn_perm(0x64646464u, w[d], 0x04030402u), xd[2 * d + 1], pr);
+                }
+                const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
+                const float mx = h2f((uint16_t)(sc[r] >> 16));
+                const float s = (mx - mn) * (1.0f / 255.0f);
+                acc[r] = fmaf(s, pr, fmaf(fmaf(-1024.0f, s, mn), sx, acc[r]));
+            }
+        } else {
+            float xf[16];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                xf[4 * i] = __uint_as_float(xv[i].x);
+                xf[4 * i + 1] = __uint_as_float(xv[i].y);
+                xf[4 * i + 2] = __uint_as_float(xv[i].z);
+                xf[4 * i + 3] = __uint_as_float(xv[i].w);
+            }
+            float sx = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 16; j++) sx += xf[j];
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+                float pr = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; j++) pr = fmaf((float)((w[j >> 2] >> (8 * (j & 3))) & 0xffu), xf[j], pr);
+                const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
+                const float mx = h2f((uint16_t)(sc[r] >> 16));
+                const float s = (mx - mn) * (1.0f / 255.0f);
+                acc[r] = fmaf(s, pr, fmaf(mn, sx, acc[r]));
+            }
         }
     }
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-        const float s = wave_sum(acc[r]);
-        if (NW == 1)
-            acc[r] = s;
-        else if (lane == 0)
-            red[wave][r] = s;
+        const float s = row_sum(acc[r]);
+        if ((tid & 15) == 0) red[r][tid >> 4] = s;
     }
-    if (NW > 1) __syncthreads();
-    if (tid < ROWS) {
+    __syncthreads();
+    // NROW16 partials per output row: 16 lanes per row sum them, again with DPP
+    if (tid < ROWS * 16) {
+        const uint32_t r = tid >> 4, l = tid & 15;
         float s = 0.0f;
-        if (NW == 1) {
 #pragma unroll
-            for (int r = 0; r < ROWS; r++)
-                if (tid == (uint32_t)r) s = acc[r];
-        } else {
-#pragma unroll
-            for (int w = 0; w < NW; w++) s += red[w][tid];
-        }
-        const uint32_t r = row0 + tid;
-        if (r < p.R) store_out(p.out, p.out_f16, r, act_apply(p.act, s));
+        for (int i = 0; i < NROW16 / 16; i++) s += red[r][l + 16 * i];
+        if (NROW16 < 16) s = l < NROW16 ? red[r][l] : 0.0f;
+        s = row_sum(s);
+        const uint32_t row = row0 + r;
+        if (l == 0 && row < p.R) store_out(p.out, p.out_f16, row, act_apply(p.act, s));
     }
 }
 
@@ -459,7 +507,11 @@ int launch_group_xt(hipStream_t stream, const GemvGroup &g, int rows, int sl, in
 template <typename XT, int ROWS>
 int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
-    if (nt >= 256)
+    if (nt >= 1024)
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024>), grid, dim3(1024), 0, stream, g);
+    else if (nt >= 512)
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512>), grid, dim3(512), 0, stream, g);
+    else if (nt >= 256)
         hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, g);
     else if (nt >= 128)
         hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, g);
@@ -589,10 +641,11 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         g.total_tasks = tasks;
         if (oneshot) {
             const uint32_t nchunk = g.p[0].K / 16;
-            int nt = nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
+            // one lane per 16-byte chunk of a row where a workgroup can hold that many
+            int nt = nchunk > 512 ? 1024 : nchunk > 256 ? 512 : nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
             nt = env_int("WRQ_GEMV_NT", nt);
             int s1;
-            if (rows == 8)
+            if (rows == 8 && nt >= 128) // the final reduction uses 16 lanes per output row
                 s1 = in_f16 ? launch_oneshot_nt<__half, 8>(stream, g, nt) : launch_oneshot_nt<float, 8>(stream, g, nt);
             else
                 s1 = in_f16 ? launch_oneshot_nt<__half, 4>(stream, g, nt) : launch_oneshot_nt<float, 4>(stream, g, nt);
