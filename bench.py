@@ -268,7 +268,7 @@ def main():
     tok_s = args.tokens * 1e3 / wall_ms
     launch_us = ms * 1e3 / dec.launches
     achieved = nbytes / dec.launches / launch_us / 1e3  # GB/s
-    kernel = {("int8", True): "gemv_int8_kernel", ("nf4", True): "gemv_nf4_kernel"}.get((args.quant, args.tokens < 16), "gemm_kernel")
+    kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_kernel<nf4>"}.get((args.quant, args.tokens == 1), "gemm_kernel")
     out = {
         "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
         "value": round(tok_s, 2),

@@ -1,0 +1,237 @@
+// Tests of the C++ host mirror (include/wrq.hpp).  `--cpu`: everything that needs no device
+// (token schedule against the literal expectations of src/runtime/infer/rnn.rs:362-569,
+// op-build shape errors).  Without flag: the same API driving the GPU, checked against a
+// float64 product on host-dequantised weights.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+
+#include "../../include/wrq.hpp"
+
+using namespace wrq;
+
+static int failures = 0;
+#define EXPECT(cond)                                                        \
+    do {                                                                    \
+        if (!(cond)) {                                                      \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);     \
+            failures++;                                                     \
+        }                                                                   \
+    } while (0)
+
+using Opt = std::optional<RnnOption>;
+static const Opt NONE = std::nullopt, LAST = RnnOption::Last, FULL = RnnOption::Full;
+
+static bool same(const RnnInfo &info, std::vector<std::pair<size_t, Opt>> want) {
+    if (info.batches.size() != want.size()) return false;
+    for (size_t i = 0; i < want.size(); i++)
+        if (info.batches[i].len != want[i].first || info.batches[i].option != want[i].second) return false;
+    return true;
+}
+
+static void test_run_iter() { // rnn.rs:362-454
+    RnnInput run({{139, RnnOption::Last}, {1, RnnOption::Last}, {0, RnnOption::Full}, {65, RnnOption::Full}}, 128);
+    auto it = run.iter();
+    EXPECT(same(it.next(), {{65, NONE}, {1, LAST}, {0, FULL}, {62, FULL}}));
+    EXPECT(same(it.next(), {{60, NONE}, {1, LAST}, {0, FULL}, {3, FULL}}));
+    EXPECT(same(it.next(), {{14, LAST}, {1, LAST}, {0, FULL}, {1, FULL}}));
+    EXPECT(same(it.next(), {{1, LAST}, {1, LAST}, {0, FULL}, {1, FULL}}));
+    EXPECT(same(it.next(), {{1, LAST}, {1, LAST}, {0, FULL}, {1, FULL}}));
+}
+
+static void test_advance() { // rnn.rs:456-507
+    RnnInput run({{139, RnnOption::Last}, {1, RnnOption::Last}, {0, RnnOption::Full}, {65, RnnOption::Full}}, 128);
+    run.step();
+    EXPECT(same(run.iter().next(), {{61, NONE}, {0, LAST}, {0, FULL}, {3, FULL}}));
+    RnnInput again({{61, RnnOption::Last}, {1, RnnOption::Last}, {0, RnnOption::Full}, {3, RnnOption::Full}}, 128);
+    EXPECT(same(again.iter().next(), {{60, NONE}, {1, LAST}, {0, FULL}, {3, FULL}}));
+}
+
+static void test_redirect() { // rnn.rs:509-569
+    RnnInput run({{61, RnnOption::Last}, {0, RnnOption::Last}, {0, RnnOption::Full}, {3, RnnOption::Full}}, 128);
+    auto r = run.iter().next().redirect();
+    EXPECT((r.headers == std::vector<size_t>{60, 61, 62, 63}));
+    EXPECT((r.inputs == std::vector<std::pair<size_t, size_t>>{{0, 61}, {61, 61}, {61, 61}, {61, 64}}));
+    EXPECT((r.outputs == std::vector<std::pair<size_t, size_t>>{{0, 1}, {1, 1}, {1, 1}, {1, 4}}));
+    std::vector<RnnInput::Batch> eight;
+    for (int rep = 0; rep < 2; rep++)
+        for (size_t n : {11, 8, 9, 4}) eight.push_back({n, RnnOption::Last});
+    RnnInput run2(eight, 32);
+    auto r2 = run2.iter().next().redirect();
+    EXPECT((r2.headers == std::vector<size_t>{15, 31}));
+    EXPECT((r2.inputs == std::vector<std::pair<size_t, size_t>>{{0, 4}, {4, 8}, {8, 12}, {12, 16}, {16, 20}, {20, 24}, {24, 28}, {28, 32}}));
+    EXPECT((r2.outputs == std::vector<std::pair<size_t, size_t>>{{0, 0}, {0, 0}, {0, 0}, {0, 1}, {1, 1}, {1, 1}, {1, 1}, {1, 2}}));
+}
+
+static void test_schedule_of_the_configs() {
+    // config 4: 512-token prompt in chunks of 128, then decode -> T = 128 x 4 (chunk kernels), then T = 1
+    RnnInput c4({{512, RnnOption::Last}}, 128);
+    for (int i = 0; i < 4; i++) {
+        auto info = c4.iter().next();
+        EXPECT(info.num_token() == 128 && turbo(info.num_token()));
+        c4.step();
+    }
+    EXPECT(c4.iter().next().num_token() == 0);
+    // token_chunk_size is rounded up to a multiple of 32 (rnn.rs:203-212); a 40-token prompt runs 32 + 8
+    RnnInput odd({{40, RnnOption::Last}}, 33);
+    EXPECT(odd.token_chunk_size() == 64);
+    EXPECT(odd.iter().next().num_token() == 32);
+    odd.step();
+    EXPECT(odd.iter().next().num_token() == 8 && !turbo(8));
+    EXPECT(turbo(32) && turbo(256) && !turbo(1) && !turbo(31));
+}
+
+static void test_build_time_errors() {
+    // op constructors fail like the reference's: TensorErrorKind::Shape(got, want)
+    const uint32_t K = 256, R = 8;
+    auto fake = reinterpret_cast<void *>(0x10000);
+    auto w = TensorGpu<uint8_t>::wrap(fake, Shape(K, R, 1, 1));
+    auto mm = TensorGpu<f16>::wrap(fake, Shape(2 * K * R / 128, 1, 1, 1));
+    auto x = TensorGpu<f16>::wrap(fake, Shape(K, 1, 1, 1));
+    auto out = TensorGpu<f16>::wrap(fake, Shape(R, 1, 1, 1));
+    bool threw = false;
+    try {
+        auto bad = TensorGpu<f16>::wrap(fake, Shape(7, 1, 1, 1));
+        TensorOp::matmul_vec_int8(w, bad, TensorGpuView<f16>(x), TensorGpuView<f16>(out), Activation::None, false);
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_SHAPE && std::string(e.what()) == "tensor shape not match: (7, 1, 1, 1) vs. (32, 1, 1, 1)";
+    }
+    EXPECT(threw);
+    threw = false;
+    try {
+        auto x2 = TensorGpu<f16>::wrap(fake, Shape(K, 2, 1, 1));
+        TensorOp::matmul_vec_int8(w, mm, TensorGpuView<f16>(x2), TensorGpuView<f16>(out), Activation::None, false);
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_SHAPE;
+    }
+    EXPECT(threw);
+    threw = false;
+    try {
+        view_of(x, {{{0, K}, {0, 2}, {0, 1}, {0, 1}}}); // slice past the parent
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_SHAPE;
+    }
+    EXPECT(threw);
+    // a well-formed op builds without touching a device
+    auto ok = TensorOp::matmul_vec_int8(w, mm, TensorGpuView<f16>(x), TensorGpuView<f16>(out), Activation::SquaredRelu, true);
+    EXPECT(ok.kind() == TensorOp::Kind::Atom);
+    EXPECT(TensorOp::INT8_BLOCK_SIZE == 128 && TensorOp::NF4_BLOCK_SIZE == 64);
+    EXPECT(float4_quant().size() == 16 && float4_quant()[7] == 0.0f);
+}
+
+// ------------------------------------------------------------------ GPU
+
+static uint16_t to_h(float f) { // round to nearest even, normal range only (test data)
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    int32_t e = (int32_t)((x >> 23) & 0xff) - 127 + 15;
+    uint32_t m = x & 0x7fffffu;
+    if (e <= 0) return (uint16_t)sign;
+    uint32_t r = ((uint32_t)e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) r++;
+    return (uint16_t)(sign | r);
+}
+static float from_h(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1f, m = h & 0x3ffu;
+    if (e == 0) return (sign ? -1.0f : 1.0f) * std::ldexp((float)m, -24);
+    uint32_t bits = sign | ((e + 112u) << 23) | (m << 13);
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+
+static void test_gpu_layer() {
+    check(wrq_init());
+    const uint32_t C = 512, H = 1024, T = 1;
+    std::mt19937 rng(42);
+    std::normal_distribution<float> nw(0.0f, 0.02f), nx(0.0f, 1.0f);
+    auto rand_h = [&](size_t n, std::normal_distribution<float> &d) {
+        std::vector<f16> v(n);
+        for (auto &e : v) e.bits = to_h(d(rng));
+        return v;
+    };
+    Queue queue;
+    // five [C, C] products reading slices of one [C, T, 5] tensor, as v6 does, plus ffn.key with squared ReLU
+    std::vector<std::vector<f16>> wh;
+    std::vector<Matrix> mats;
+    for (int j = 0; j < 4; j++) {
+        wh.push_back(rand_h((size_t)C * C, nw));
+        auto t = TensorGpu<f16>::from_data(Shape(C, C, 1, 1), wh.back());
+        mats.push_back(j % 2 ? Matrix::quant_nf4(t, queue) : Matrix::quant_u8(t, queue));
+    }
+    wh.push_back(rand_h((size_t)C * H, nw));
+    mats.push_back(Matrix::quant_u8(TensorGpu<f16>::from_data(Shape(C, H, 1, 1), wh.back()), queue));
+    auto sx_h = rand_h((size_t)C * T * 5, nx);
+    auto sx = TensorGpu<f16>::from_data(Shape(C, T, 5, 1), sx_h);
+    std::vector<TensorGpu<float>> outs;
+    std::vector<TensorOp> ops;
+    for (uint32_t j = 0; j < 4; j++) {
+        outs.push_back(TensorGpu<float>::init(Shape(C, T, 1, 1)));
+        ops.push_back(mats[j].matmul_op(view_of(sx, {{{0, C}, {0, T}, {j + 1, j + 2}, {0, 1}}}), TensorGpuView<float>(outs[j]),
+                                        Activation::None, turbo(T)));
+    }
+    auto ffn = TensorGpu<f16>::init(Shape(H, T, 1, 1));
+    ops.push_back(TensorOp::Sep());
+    ops.push_back(mats[4].matmul_op(view_of(sx, {{{0, C}, {0, T}, {0, 1}, {0, 1}}}), TensorGpuView<f16>(ffn), Activation::SquaredRelu,
+                                    turbo(T)));
+    queue.submit(TensorOp::List(ops));
+    queue.sync();
+
+    // host check: dequantise the packed bytes the device produced, multiply in double
+    auto close = [](double a, double b) { return std::fabs(a - b) <= std::max(2e-3, 2e-3 * std::max(std::fabs(a), std::fabs(b))); };
+    for (uint32_t j = 0; j < 5; j++) {
+        const uint32_t R = j < 4 ? C : H;
+        const auto wb = mats[j].w.back();
+        const auto sb = mats[j].m.back();
+        std::vector<double> got;
+        if (j < 4)
+            for (float v : outs[j].back()) got.push_back(v);
+        else
+            for (f16 v : ffn.back()) got.push_back(from_h(v.bits));
+        const uint32_t slice = j < 4 ? j + 1 : 0;
+        int bad = 0;
+        for (uint32_t r = 0; r < R; r++) {
+            double acc = 0;
+            for (uint32_t k = 0; k < C; k++) {
+                const size_t e = (size_t)r * C + k;
+                double wv;
+                if (mats[j].kind == Matrix::Kind::Int8) {
+                    const double mn = from_h(sb[2 * (e / 128)].bits), mx = from_h(sb[2 * (e / 128) + 1].bits);
+                    wv = wb[e] / 255.0 * (mx - mn) + mn;
+                } else {
+                    const uint8_t byte = wb[e / 2];
+                    const int nib = (e & 1) ? byte >> 4 : byte & 15;
+                    wv = (double)float4_quant()[nib] * from_h(sb[e / 64].bits);
+                }
+                acc += wv * from_h(sx_h[(size_t)slice * C * T + k].bits);
+                // the packed value stays close to the source weight
+                if (k == 0 && r == 0) EXPECT(std::fabs(wv - from_h(wh[j][e].bits)) < 0.02);
+            }
+            if (j == 4) acc = acc > 0 ? acc * acc : 0.0;
+            bad += !close(acc, got[r]);
+        }
+        EXPECT(bad == 0);
+    }
+}
+
+int main(int argc, char **argv) {
+    const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
+    test_run_iter();
+    test_advance();
+    test_redirect();
+    test_schedule_of_the_configs();
+    test_build_time_errors();
+    if (!cpu_only) {
+        try {
+            test_gpu_layer();
+        } catch (const TensorError &e) {
+            std::printf("FAIL: TensorError %d: %s\n", e.status, e.what());
+            failures++;
+        }
+    }
+    std::printf(failures ? "%d FAILED\n" : "host tests ok%.0d\n", failures);
+    return failures ? 1 : 0;
+}

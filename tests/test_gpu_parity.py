@@ -375,7 +375,7 @@ def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind):
     for j in range(len(shapes)):
         assert_close(host(group[j]), truths[j], EPS, f"group op {j} vs float64")
         # same arithmetic; only the lane count of the final reduction may differ with the group's shapes
-        assert_close(host(group[j]), host(single[j]), 1e-5, f"group op {j} vs the single call")
+        assert_close(host(group[j]), host(single[j]), 1e-3, f"group op {j} vs the single call")  # <= 1 f16 ulp
     # mixed token counts and a chunk-shaped op inside one list are split, not rejected
     x32 = gen_f16(rng, (32, C), 1.0)
     o32 = torch.empty((32, C), dtype=torch.float16, device="cuda")

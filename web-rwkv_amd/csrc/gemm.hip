@@ -4,26 +4,39 @@
 // out[t, r] = ACT( sum_k deq(W[r, k]) * x[t, k] )      (src/shaders/matmul_mat_int8.wgsl:62-153,
 //                                                        src/shaders/matmul_mat_nf4.wgsl:94-220)
 //
-// Layout of one workgroup (4 waves): 64 weight rows x (16 * NTILE) tokens, K walked in
-// steps of 128.  Wave w owns rows 16w..16w+15 as the MFMA "A" side.  Weight bytes go
-// from HBM straight into the A registers of the one wave that uses them (each byte is
-// read once and never shared, so an LDS tile for them would only add traffic); the
-// activation tile, shared by all four waves, is staged as f16 in double-buffered LDS
-// and read back as "B" operands with ds_read_b128.
+// The shapes of this path are skinny: 16..256 tokens against thousands of weight rows, so
+// even the chunk products are bound by streaming the packed weights once (below ~100
+// tokens) or sit close to that point.  The decomposition follows from it:
+//   * a workgroup (4 waves) owns 64*MRT weight rows x 16*NTILE tokens x one K range; wave w
+//     owns MRT row tiles of 16 as the MFMA "A" side.  Weight bytes go from HBM straight
+//     into the A registers of the one wave that uses them (each byte is read once and never
+//     shared, an LDS tile for them would only add traffic); the activation tile, shared by
+//     the four waves, is staged as f16 in double-buffered LDS and read back as "B" operands
+//     with ds_read_b128, each B operand serving MRT MFMAs;
+//   * weights are prefetched several K steps ahead through a ring of register buffers
+//     (a step is far shorter than HBM latency), activations two steps ahead; loads are
+//     issued activations first, weights after, because loads return in issue order;
+//   * K is split over workgroups (grid.y) until there are enough of them to fill 256 CUs;
+//     every split stores its partial tile to its own slice of an f32 scratch array and a
+//     second, tiny kernel sums the slices, applies the activation and stores the output
+//     type.  Without a split the first kernel stores directly.
 //
 // The scales never enter the matrix cores, which keeps the f16 operands exact:
-//   int8: A holds the codes as f16 (1024 + u, built with one v_perm_b32 per two
-//         weights); after each 128-block   out += s * D + (min - 1024 s) * sum_k x
-//         with s = (max - min) / 255, and sum_k x taken from the B registers.
+//   int8: A holds the codes as f16 (1024 + u, one v_perm_b32 per two weights); after each
+//         128-block   out += s * D + (min - 1024 s) * sum_k x,  s = (max - min) / 255,
+//         with sum_k x per token taken once per workgroup while the tile is staged.
 //   nf4:  A holds table values split into two f16 halves (hi + lo * 2^-11, exact to
-//         2^-22), fetched per byte (two weights) from a 256-entry LDS table; after
-//         each 64-block   out += absmax * (D_hi + 2^-11 D_lo).
+//         2^-22), fetched per byte (two weights) from a 256-entry LDS table; after each
+//         64-block   out += absmax * (D_hi + 2^-11 D_lo).
 #include "wrq_device.h"
 #include "wrq_host.h"
+
+#include <stdlib.h>
 
 namespace wrq {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
 union HalfPack {
@@ -34,38 +47,70 @@ union HalfPack {
 constexpr int kStep = 128;        // K elements per step
 constexpr int kPitch = kStep + 8; // f16 elements per LDS row: 272 B keeps 16-byte alignment and rotates banks
 
+// Partial tiles of split-K launches: [split][batch][token][row].  One array per process and
+// GPU: split-K calls that overlap in time on one GPU (different streams) would race on it,
+// calls on one stream cannot.  Nothing in it outlives a call.
+constexpr size_t kScratchFloats = 8u << 20; // 32 MiB: splits * R * T up to 8 Mi partial outputs
+__device__ __align__(256) float g_splitk_scratch[kScratchFloats];
+
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     return (uint32_t)f2h(a) | ((uint32_t)f2h(b) << 16);
 }
-
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float dot2_ones(uint32_t v, float acc) {
     // acc + lo(v) + hi(v) with f32 accumulation: v_dot2_f32_f16 against (1.0, 1.0)
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v), half2v{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
 }
 
-template <int NTILE>
-constexpr size_t gemm_lds_bytes(int quant) {
-    return (size_t)2 * 16 * NTILE * kPitch * sizeof(uint16_t) + (quant == kNf4 ? 256 * sizeof(uint2) : 0);
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xf, 0xf, true));
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xf, 0xf, true));
+    return v;
 }
 
-template <int QUANT, typename XT, int NTILE>
-__global__ __launch_bounds__(256) void gemm_kernel(const MatmulArgs a) {
+template <int NTILE>
+constexpr size_t gemm_lds_bytes(int quant) {
+    return (size_t)2 * 16 * NTILE * kPitch * sizeof(uint16_t) + (size_t)2 * 16 * NTILE * sizeof(float) +
+           (quant == kNf4 ? 256 * sizeof(uint2) : 0);
+}
+
+struct GemmArgs {
+    MatmulArgs m;
+    uint32_t k_per_split; // K range of one workgroup, a multiple of kStep
+    float *scratch;       // null: store directly
+};
+
+template <int QUANT, typename XT, int MRT, int NTILE>
+__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
+    const MatmulArgs &a = ga.m;
     constexpr int BN = 16 * NTILE;
+    constexpr int BM = 64 * MRT;
+    constexpr int NW = QUANT == kInt8 ? 2 : 1; // 16-byte weight registers per row tile and step
     extern __shared__ __align__(16) uint8_t smem[];
     uint16_t(*xs)[BN * kPitch] = reinterpret_cast<uint16_t(*)[BN * kPitch]>(smem);
-    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t));
+    float(*sxs)[BN] = reinterpret_cast<float(*)[BN]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t));
+    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BN * sizeof(float));
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r16 = lane & 15, g = lane >> 4;
-    const uint32_t b = blockIdx.z, t0 = blockIdx.y * BN;
+    const uint32_t tblocks = (a.T + BN - 1) / BN;
+    const uint32_t b = blockIdx.z / tblocks;
+    const uint32_t t0 = (blockIdx.z % tblocks) * BN;
     const uint32_t K = a.K;
-    const uint32_t row_base = blockIdx.x * 64 + wave * 16;
-    const uint32_t row = min(row_base + r16, a.R - 1);       // A-side row of this lane
-    const uint32_t frow = min(row_base + 4 * g, a.R - 4);    // first of the 4 D-side rows of this lane
-    const uint64_t e_row = ((uint64_t)b * a.R + row) * K;    // flat element index of (row, 0)
-    const uint64_t e_frow = ((uint64_t)b * a.R + frow) * K;
+    const uint32_t k_begin = blockIdx.y * ga.k_per_split;
+    const uint32_t k_end = min(K, k_begin + ga.k_per_split);
+    const uint32_t row_base = blockIdx.x * BM + wave * (16 * MRT);
+
+    uint64_t e_row[MRT], e_frow[MRT];
+#pragma unroll
+    for (int i = 0; i < MRT; i++) {
+        const uint32_t row = min(row_base + 16 * i + r16, a.R - 1);    // A-side row of this lane
+        const uint32_t frow = min(row_base + 16 * i + 4 * g, a.R - 4); // first of its 4 D-side rows
+        e_row[i] = ((uint64_t)b * a.R + row) * K; // flat element index of (row, 0)
+        e_frow[i] = ((uint64_t)b * a.R + frow) * K;
+    }
 
     if (QUANT == kNf4) {
         // entry for byte v: (hi(q[v & 15]), hi(q[v >> 4])), (lo(..), lo(..)); lo scaled by 2^11
@@ -74,7 +119,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const MatmulArgs a) {
         pair[tid] = make_uint2(pack_h2(q0, q1), pack_h2((q0 - h0) * 2048.0f, (q1 - h1) * 2048.0f));
     }
 
-    // activation tile staging: piece p of a tile is 8 consecutive k of one token
+    // activation tile staging: piece p of a tile is 8 consecutive k of one token; the 16 pieces
+    // of a token sit in 16 adjacent lanes, one DPP row
     constexpr int NPIECE = NTILE; // pieces per thread: BN * 16 / 256
     const XT *xbase = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
     uint4 xreg[NPIECE];
@@ -100,100 +146,116 @@ __global__ __launch_bounds__(256) void gemm_kernel(const MatmulArgs a) {
         for (int p = 0; p < NPIECE; p++) {
             const uint32_t piece = tid + 256 * p;
             *reinterpret_cast<uint4 *>(&xs[buf][(piece >> 4) * kPitch + ((piece & 15) << 3)]) = xreg[p];
+            if (QUANT == kInt8) {
+                float s = dot2_ones(xreg[p].x, 0.0f);
+                s = dot2_ones(xreg[p].y, s);
+                s = dot2_ones(xreg[p].z, s);
+                s = dot2_ones(xreg[p].w, s);
+                s = row16_sum(s);
+                if ((tid & 15) == 0) sxs[buf][piece >> 4] = s;
+            }
         }
     };
 
-    // packed weights of one step for this lane: int8 2 x 16 B, nf4 2 x 8 B
-    uint4 wreg[2];
-    auto load_w = [&](uint32_t kb) {
-        if (QUANT == kInt8) {
-            wreg[0] = load128_stream(a.w + e_row + kb + 16 * g);
-            wreg[1] = load128_stream(a.w + e_row + kb + 64 + 16 * g);
-        } else {
-            const uint8_t *p = a.w + ((e_row + kb) >> 1);
-            const uint2 v0 = load64_stream(p + 8 * g);
-            const uint2 v1 = load64_stream(p + 32 + 8 * g);
-            wreg[0] = make_uint4(v0.x, v0.y, v1.x, v1.y);
+    // packed weights and scale blocks of one step for this lane, per row tile: int8 2 x 16 B of
+    // codes + 4 (min, max) pairs (one per D-side row), nf4 2 x 8 B + 4 absmax pairs
+    struct StepRegs {
+        uint4 w[MRT][NW];
+        uint32_t sc[MRT][4];
+    };
+    auto load_w = [&](uint32_t kb, StepRegs &dst) {
+#pragma unroll
+        for (int i = 0; i < MRT; i++) {
+            if (QUANT == kInt8) {
+                dst.w[i][0] = load128_stream(a.w + e_row[i] + kb + 16 * g);
+                dst.w[i][NW - 1] = load128_stream(a.w + e_row[i] + kb + 64 + 16 * g);
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    dst.sc[i][d] = reinterpret_cast<const uint32_t *>(a.scale)[(e_frow[i] + (uint64_t)d * K + kb) >> 7];
+            } else {
+                const uint8_t *p = a.w + ((e_row[i] + kb) >> 1);
+                const uint2 v0 = load64_stream(p + 8 * g);
+                const uint2 v1 = load64_stream(p + 32 + 8 * g);
+                dst.w[i][0] = make_uint4(v0.x, v0.y, v1.x, v1.y);
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    dst.sc[i][d] = *reinterpret_cast<const uint32_t *>(&a.scale[(e_frow[i] + (uint64_t)d * K + kb) >> 6]);
+            }
         }
     };
 
-    float4v out[NTILE];
+    float4v out[MRT][NTILE];
 #pragma unroll
-    for (int n = 0; n < NTILE; n++) out[n] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MRT; i++)
+#pragma unroll
+        for (int n = 0; n < NTILE; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    load_tile(0);
-    load_w(0);
-    int buf = 0;
-    for (uint32_t kb = 0; kb < K; kb += kStep, buf ^= 1) {
-        store_tile(buf);
-        __syncthreads();
-        uint4 wcur[2] = {wreg[0], wreg[1]};
-        // scales of the 4 D-side rows for this step
-        float s_row[4], c_row[4], am_row[2][4];
-        if (QUANT == kInt8) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t mm = reinterpret_cast<const uint32_t *>(a.scale)[(e_frow + (uint64_t)i * K + kb) >> 7];
-                const float mn = h2f((uint16_t)(mm & 0xffffu)), mx = h2f((uint16_t)(mm >> 16));
-                s_row[i] = (mx - mn) * (1.0f / 255.0f);
-                c_row[i] = fmaf(-1024.0f, s_row[i], mn);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t am2 = *reinterpret_cast<const uint32_t *>(&a.scale[(e_frow + (uint64_t)i * K + kb) >> 6]);
-                am_row[0][i] = h2f((uint16_t)(am2 & 0xffffu));
-                am_row[1][i] = h2f((uint16_t)(am2 >> 16));
-            }
-        }
-        if (kb + kStep < K) {
-            load_tile(kb + kStep);
-            load_w(kb + kStep);
-        }
-
+    // one K step on the matrix cores: weights `cur` against the activation tile in LDS buffer `buf`
+    auto compute = [&](const StepRegs &cur, int buf) {
         const uint16_t *xt = xs[buf];
         if (QUANT == kInt8) {
-            HalfPack A[4];
-            const uint32_t w[8] = {wcur[0].x, wcur[0].y, wcur[0].z, wcur[0].w, wcur[1].x, wcur[1].y, wcur[1].z, wcur[1].w};
+            float s_row[MRT][4], c_row[MRT][4];
+            HalfPack A[MRT][4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                // 8 weights = dwords 2i, 2i+1 -> f16 codes 1024 + u
-                A[i].u[0] = __builtin_amdgcn_perm(0x64646464u, w[2 * i], 0x04010400u);
-                A[i].u[1] = __builtin_amdgcn_perm(0x64646464u, w[2 * i], 0x04030402u);
-                A[i].u[2] = __builtin_amdgcn_perm(0x64646464u, w[2 * i + 1], 0x04010400u);
-                A[i].u[3] = __builtin_amdgcn_perm(0x64646464u, w[2 * i + 1], 0x04030402u);
+            for (int i = 0; i < MRT; i++) {
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    const uint32_t mm = cur.sc[i][d];
+                    const float mn = h2f((uint16_t)(mm & 0xffffu)), mx = h2f((uint16_t)(mm >> 16));
+                    s_row[i][d] = (mx - mn) * (1.0f / 255.0f);
+                    c_row[i][d] = fmaf(-1024.0f, s_row[i][d], mn);
+                }
+                const uint32_t w[8] = {cur.w[i][0].x,      cur.w[i][0].y,      cur.w[i][0].z,      cur.w[i][0].w,
+                                       cur.w[i][NW - 1].x, cur.w[i][NW - 1].y, cur.w[i][NW - 1].z, cur.w[i][NW - 1].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    // 8 weights = dwords 2j, 2j+1 -> f16 codes 1024 + u
+                    A[i][j].u[0] = __builtin_amdgcn_perm(0x64646464u, w[2 * j], 0x04010400u);
+                    A[i][j].u[1] = __builtin_amdgcn_perm(0x64646464u, w[2 * j], 0x04030402u);
+                    A[i][j].u[2] = __builtin_amdgcn_perm(0x64646464u, w[2 * j + 1], 0x04010400u);
+                    A[i][j].u[3] = __builtin_amdgcn_perm(0x64646464u, w[2 * j + 1], 0x04030402u);
+                }
             }
 #pragma unroll
             for (int n = 0; n < NTILE; n++) {
-                float4v D = {0.f, 0.f, 0.f, 0.f};
-                float sx = 0.0f;
+                float4v D[MRT];
+#pragma unroll
+                for (int i = 0; i < MRT; i++) D[i] = float4v{0.f, 0.f, 0.f, 0.f};
                 const uint16_t *xrow = xt + (n * 16 + r16) * kPitch + 16 * g;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    // A[i] covers k = 64 (i / 2) + 16 g + 8 (i % 2) .. + 8
+                for (int j = 0; j < 4; j++) {
+                    // A[.][j] covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
                     HalfPack B;
-                    const uint4 v = *reinterpret_cast<const uint4 *>(xrow + 64 * (i >> 1) + 8 * (i & 1));
+                    const uint4 v = *reinterpret_cast<const uint4 *>(xrow + 64 * (j >> 1) + 8 * (j & 1));
                     B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
-                    sx = dot2_ones(v.x, sx); sx = dot2_ones(v.y, sx);
-                    sx = dot2_ones(v.z, sx); sx = dot2_ones(v.w, sx);
-                    D = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i].h, B.h, D, 0, 0, 0);
-                }
-                // sum over the four k-groups held by lanes l, l^16, l^32, l^48
-                sx += __shfl_xor(sx, 16);
-                sx += __shfl_xor(sx, 32);
 #pragma unroll
-                for (int i = 0; i < 4; i++) out[n][i] = fmaf(s_row[i], D[i], fmaf(c_row[i], sx, out[n][i]));
+                    for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, D[i], 0, 0, 0);
+                }
+                const float sx = sxs[buf][n * 16 + r16];
+#pragma unroll
+                for (int i = 0; i < MRT; i++)
+#pragma unroll
+                    for (int d = 0; d < 4; d++) out[i][n][d] = fmaf(s_row[i][d], D[i][d], fmaf(c_row[i][d], sx, out[i][n][d]));
             }
         } else {
-            const uint32_t w[4] = {wcur[0].x, wcur[0].y, wcur[0].z, wcur[0].w};
-            HalfPack Ah[4], Al[4];
+            HalfPack Ah[MRT][4], Al[MRT][4];
+            float am_row[MRT][2][4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < MRT; i++) {
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    am_row[i][0][d] = h2f((uint16_t)(cur.sc[i][d] & 0xffffu));
+                    am_row[i][1][d] = h2f((uint16_t)(cur.sc[i][d] >> 16));
+                }
+                const uint32_t w[4] = {cur.w[i][0].x, cur.w[i][0].y, cur.w[i][0].z, cur.w[i][0].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const uint2 e = pair[(w[i] >> (8 * j)) & 0xffu];
-                    Ah[i].u[j] = e.x;
-                    Al[i].u[j] = e.y;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const uint2 e = pair[(w[j] >> (8 * c)) & 0xffu];
+                        Ah[i][j].u[c] = e.x;
+                        Al[i][j].u[c] = e.y;
+                    }
                 }
             }
 #pragma unroll
@@ -201,70 +263,211 @@ __global__ __launch_bounds__(256) void gemm_kernel(const MatmulArgs a) {
                 const uint16_t *xrow = xt + (n * 16 + r16) * kPitch + 16 * g;
 #pragma unroll
                 for (int blk = 0; blk < 2; blk++) {
-                    float4v Dh = {0.f, 0.f, 0.f, 0.f}, Dl = {0.f, 0.f, 0.f, 0.f};
+                    float4v Dh[MRT], Dl[MRT];
+#pragma unroll
+                    for (int i = 0; i < MRT; i++) Dh[i] = Dl[i] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
                         // dword 2 blk + j covers k = 64 blk + 16 g + 8 j .. + 8
                         HalfPack B;
                         const uint4 v = *reinterpret_cast<const uint4 *>(xrow + 64 * blk + 8 * j);
                         B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
-                        Dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[2 * blk + j].h, B.h, Dh, 0, 0, 0);
-                        Dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[2 * blk + j].h, B.h, Dl, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < MRT; i++) {
+                            Dh[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[i][2 * blk + j].h, B.h, Dh[i], 0, 0, 0);
+                            Dl[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[i][2 * blk + j].h, B.h, Dl[i], 0, 0, 0);
+                        }
                     }
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        out[n][i] = fmaf(am_row[blk][i], fmaf(Dl[i], 1.0f / 2048.0f, Dh[i]), out[n][i]);
+                    for (int i = 0; i < MRT; i++)
+#pragma unroll
+                        for (int d = 0; d < 4; d++)
+                            out[i][n][d] = fmaf(am_row[i][blk][d], fmaf(Dl[i][d], 1.0f / 2048.0f, Dh[i][d]), out[i][n][d]);
                 }
+            }
+        }
+    };
+
+    // ring of NBUF weight steps in flight, activation tile two steps ahead; the step loop is
+    // unrolled by NBUF so that every ring slot is a fixed set of registers
+    constexpr int NBUF = MRT >= 4 ? 2 : 4;
+    const uint32_t nsteps = (k_end - k_begin) / kStep;
+    StepRegs ring[NBUF];
+    uint4 xring[2][NPIECE];
+    auto load_x = [&](uint32_t s, uint4(&dst)[NPIECE]) {
+        load_tile(k_begin + s * kStep);
+#pragma unroll
+        for (int p = 0; p < NPIECE; p++) dst[p] = xreg[p];
+    };
+    auto stage_x = [&](const uint4(&src)[NPIECE], int buf) {
+#pragma unroll
+        for (int p = 0; p < NPIECE; p++) xreg[p] = src[p];
+        store_tile(buf);
+    };
+    load_x(0, xring[0]);
+    if (nsteps > 1) load_x(1, xring[1]);
+#pragma unroll
+    for (int j = 0; j < NBUF; j++)
+        if ((uint32_t)j < nsteps) load_w(k_begin + j * kStep, ring[j]);
+    for (uint32_t base = 0; base < nsteps; base += NBUF) {
+#pragma unroll
+        for (int j = 0; j < NBUF; j++) {
+            const uint32_t s = base + j;
+            if (s < nsteps) {
+                stage_x(xring[j & 1], j & 1);
+                lds_barrier();
+                const StepRegs cur = ring[j];
+                // activations first, weights after: loads complete in issue order
+                if (s + 2 < nsteps) load_x(s + 2, xring[j & 1]);
+                if (s + NBUF < nsteps) load_w(k_begin + (s + NBUF) * kStep, ring[j]);
+                compute(cur, j & 1);
             }
         }
     }
 
-    // D layout of the 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
-    const uint32_t orow = row_base + 4 * g;
+    // D layout of a 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
 #pragma unroll
-    for (int n = 0; n < NTILE; n++) {
-        const uint32_t t = t0 + n * 16 + r16;
-        if (t < a.T && orow < a.R) {
-            const uint64_t idx = (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + orow;
-            float v[4];
+    for (int i = 0; i < MRT; i++) {
+        const uint32_t orow = row_base + 16 * i + 4 * g;
 #pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = act_apply(a.act, out[n][i]);
-            if (a.out_f16) {
-                *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) =
-                    make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
-            } else {
-                *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
+        for (int n = 0; n < NTILE; n++) {
+            const uint32_t t = t0 + n * 16 + r16;
+            if (t < a.T && orow < a.R) {
+                if (ga.scratch) {
+                    float *dst = ga.scratch + (((uint64_t)blockIdx.y * a.B + b) * a.T + t) * a.R + orow;
+                    *reinterpret_cast<float4 *>(dst) = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
+                } else {
+                    const uint64_t idx = (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + orow;
+                    float v[4];
+#pragma unroll
+                    for (int d = 0; d < 4; d++) v[d] = act_apply(a.act, out[i][n][d]);
+                    if (a.out_f16) {
+                        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) =
+                            make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
+                    } else {
+                        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+                }
             }
         }
+    }
+}
+
+// Second half of a split-K product: sum of the partial slices, activation, output type.
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits) {
+    const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x; // one quad of rows
+    const uint64_t quads_per_token = a.R / 4;
+    const uint64_t total = quads_per_token * a.T * a.B;
+    if (q >= total) return;
+    const uint64_t bt = q / quads_per_token, r = (q - bt * quads_per_token) * 4;
+    const uint64_t b = bt / a.T, t = bt - b * a.T;
+    const uint64_t slice = (uint64_t)a.B * a.T * a.R;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t k = 0; k < splits; k++) {
+        const float4 v = *reinterpret_cast<const float4 *>(scratch + k * slice + bt * a.R + r);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const float v[4] = {act_apply(a.act, s.x), act_apply(a.act, s.y), act_apply(a.act, s.z), act_apply(a.act, s.w)};
+    const uint64_t idx = b * a.out_batch_stride + t * a.out_token_stride + r;
+    if (a.out_f16) {
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
+    } else {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
     }
 }
 
 namespace {
 
-template <int QUANT, typename XT, int NTILE>
-void launch_one(hipStream_t stream, const MatmulArgs &a) {
-    dim3 grid((a.R + 63) / 64, (a.T + 16 * NTILE - 1) / (16 * NTILE), a.B);
+int env_int(const char *name, int fallback) {
+    const char *s = getenv(name);
+    return (s && *s) ? atoi(s) : fallback;
+}
+
+float *scratch_ptr() {
+    // the array's name is a host-side handle: resolve the device address once per device
+    static float *ptr[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_splitk_scratch)) != hipSuccess) return nullptr;
+        ptr[dev] = static_cast<float *>(p);
+    }
+    return ptr[dev];
+}
+
+template <int QUANT, typename XT, int MRT, int NTILE>
+int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
     constexpr size_t lds = gemm_lds_bytes<NTILE>(QUANT);
+    auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE>;
     if (lds > 48 * 1024) {
         // one-time opt-in to more than the default dynamic LDS limit
-        static const hipError_t once = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&gemm_kernel<QUANT, XT, NTILE>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         (void)once;
     }
-    hipLaunchKernelGGL((gemm_kernel<QUANT, XT, NTILE>), grid, dim3(256), lds, stream, a);
+    GemmArgs ga;
+    ga.m = a;
+    const uint32_t steps = a.K / kStep;
+    // the partial slices of all splits must fit the scratch array, whoever chose `ksplit`
+    const uint64_t outs = (uint64_t)a.R * a.T * a.B;
+    while (ksplit > 1 && outs * ksplit > kScratchFloats) ksplit /= 2;
+    if (ksplit > steps) ksplit = steps;
+    const uint32_t steps_per = (steps + ksplit - 1) / ksplit;
+    ga.k_per_split = steps_per * kStep;
+    const uint32_t splits = (steps + steps_per - 1) / steps_per;
+    ga.scratch = nullptr;
+    if (splits > 1) {
+        ga.scratch = scratch_ptr();
+        if (!ga.scratch) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+        if (outs * splits > kScratchFloats) return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(outs * splits), (unsigned long long)kScratchFloats);
+    }
+    const uint32_t tblocks = (a.T + 16 * NTILE - 1) / (16 * NTILE);
+    dim3 grid((a.R + 64 * MRT - 1) / (64 * MRT), splits, tblocks * a.B);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, ga);
+    int s = check_launch("matmul_mat");
+    if (s != WRQ_OK) return s;
+    if (splits > 1) {
+        const uint64_t quads = (uint64_t)a.R / 4 * a.T * a.B;
+        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((quads + 255) / 256)), dim3(256), 0, stream, a, ga.scratch, splits);
+        s = check_launch("matmul_mat (finish)");
+    }
+    return s;
 }
 
 template <int QUANT, typename XT>
-void launch_ntile(hipStream_t stream, const MatmulArgs &a) {
-    if (a.T <= 16)
-        launch_one<QUANT, XT, 1>(stream, a);
-    else if (a.T <= 32)
-        launch_one<QUANT, XT, 2>(stream, a);
-    else if (a.T <= 64)
-        launch_one<QUANT, XT, 4>(stream, a);
-    else
-        launch_one<QUANT, XT, 8>(stream, a);
+int launch_shape(hipStream_t stream, const MatmulArgs &a) {
+    // tokens per workgroup pass: up to 128; rows per workgroup: 64 * MRT.  More rows per
+    // workgroup re-read the activation tile less often; fewer give more workgroups.
+    const uint32_t T = a.T;
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? 4 : 8;
+    int mrt = T <= 32 ? 1 : 2;
+    if ((uint64_t)a.R * a.B >= 16384 && T > 16) mrt = 2;
+    if ((uint64_t)a.R * a.B >= 32768 && T > 64) mrt = 4;
+    mrt = env_int("WRQ_GEMM_MRT", mrt);
+    ntile = env_int("WRQ_GEMM_NTILE", ntile);
+    const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
+    const uint64_t wgs = (uint64_t)((a.R + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
+    // split K until ~2 workgroups per CU, keeping at least 4 steps per workgroup, the partial
+    // slices inside the scratch array and their traffic (8 B per output and split) small
+    // beside the packed weights
+    uint32_t ksplit = 1;
+    const uint32_t steps = a.K / kStep;
+    const uint64_t outs = (uint64_t)a.R * a.T * a.B;
+    const uint64_t wbytes = (uint64_t)a.R * a.K * a.B / (QUANT == kInt8 ? 1 : 2);
+    while (wgs * ksplit < 512 && ksplit * 2 <= steps / 4 && outs * ksplit * 2 <= kScratchFloats &&
+           outs * ksplit * 2 * 8 <= wbytes)
+        ksplit *= 2;
+    ksplit = (uint32_t)env_int("WRQ_GEMM_KSPLIT", (int)ksplit);
+    if (ksplit < 1) ksplit = 1;
+
+#define WRQ_CASE(M, N) \
+    if (mrt == M && ntile == N) return launch_one<QUANT, XT, M, N>(stream, a, ksplit);
+    WRQ_CASE(1, 1) WRQ_CASE(1, 2) WRQ_CASE(1, 4) WRQ_CASE(1, 8)
+    WRQ_CASE(2, 1) WRQ_CASE(2, 2) WRQ_CASE(2, 4) WRQ_CASE(2, 8)
+    WRQ_CASE(4, 2) WRQ_CASE(4, 4) WRQ_CASE(4, 8)
+#undef WRQ_CASE
+    return launch_one<QUANT, XT, 1, 2>(stream, a, ksplit);
 }
 
 } // namespace
@@ -273,19 +476,10 @@ void launch_ntile(hipStream_t stream, const MatmulArgs &a) {
 // activation rows and output rows of 4.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
     if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
-    if (a.B > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.B, 65535u);
-    if (quant == kInt8) {
-        if (in_f16)
-            launch_ntile<kInt8, __half>(stream, a);
-        else
-            launch_ntile<kInt8, float>(stream, a);
-    } else {
-        if (in_f16)
-            launch_ntile<kNf4, __half>(stream, a);
-        else
-            launch_ntile<kNf4, float>(stream, a);
-    }
-    return check_launch("matmul_mat");
+    if ((uint64_t)a.B * ((a.T + 15) / 16) > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.B, 65535u);
+    if (quant == kInt8)
+        return in_f16 ? launch_shape<kInt8, __half>(stream, a) : launch_shape<kInt8, float>(stream, a);
+    return in_f16 ? launch_shape<kNf4, __half>(stream, a) : launch_shape<kNf4, float>(stream, a);
 }
 
 } // namespace wrq
