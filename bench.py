@@ -169,6 +169,33 @@ def cpu_baseline(wrq, torch, layers, dec, quant, sample_layers):
     }
 
 
+def run_probe(torch):
+    """Plain copy and streaming read of 256 MiB with the probe kernels; returns their GB/s."""
+    import ctypes as C
+
+    L = C.CDLL(os.path.join(ROOT, "web-rwkv_amd", "libwrq_probe.so"))
+    L.wrq_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int]
+    L.wrq_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]
+    n = 256 << 20
+    src = torch.randint(0, 127, (4, n), dtype=torch.uint8, device="cuda")
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    it = [0]
+
+    def copy():
+        L.wrq_probe_copy(st, C.c_void_p(dst.data_ptr()), C.c_void_p(src[it[0] % 4].data_ptr()), n)
+        it[0] += 1
+
+    def read():
+        L.wrq_probe_read(st, C.c_void_p(src[it[0] % 4].data_ptr()), C.c_void_p(sink.data_ptr()), n, 2, 1)
+        it[0] += 1
+
+    ms_copy, _ = time_steps(torch, copy, 8, 2)
+    ms_read, _ = time_steps(torch, read, 8, 2)
+    return {"bytes": n, "copy_GBps": round(2 * n / ms_copy / 1e6, 1), "read_GBps": round(n / ms_read / 1e6, 1)}
+
+
 def sweep(wrq, torch, args):
     """Per-operator figures of configs 2 and 3: cold (rotating weight copies) GB/s per shape."""
     rows = []
@@ -226,6 +253,8 @@ def main():
     ap.add_argument("--no-group", action="store_true", help="one launch per product instead of grouped launches of independent products")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-layers", type=int, default=8)
+    ap.add_argument("--probe", action="store_true",
+                    help="also run the plain copy (256 MiB) and stream-read probes: the dispatches rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled against")
     ap.add_argument("--sweep", action="store_true", help="per-operator sweep (configs 2 and 3) instead of the decode step")
     ap.add_argument("--all-t", action="store_true", help="with --sweep: all token counts for int8 too")
     args = ap.parse_args()
@@ -242,6 +271,7 @@ def main():
     if args.sweep:
         sweep(wrq, torch, args)
         return
+    probe = run_probe(torch) if args.probe else None
 
     C, H = 4096, 14336
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
@@ -296,6 +326,8 @@ def main():
             "avg_launch_us": round(launch_us, 3), "bytes_per_launch": nbytes // dec.launches,
         },
     }
+    if probe:
+        out["probe"] = probe
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wrq, torch, layers, dec, args.quant, min(args.cpu_sample_layers, args.layers))
     print(json.dumps(out), flush=True)
