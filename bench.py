@@ -298,6 +298,12 @@ def main():
     tok_s = args.tokens * 1e3 / wall_ms
     launch_us = ms * 1e3 / dec.launches
     achieved = nbytes / dec.launches / launch_us / 1e3  # GB/s
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE (a counter run of its own,
+    # scaled by what the same counters read for a 256 MiB plain copy; summary under profiles/):
+    # 225.9 MB fetched + 0.2 MB written per layer of the grouped Int8 decode step, 4 launches
+    traffic = None
+    if args.quant == "int8" and args.tokens == 1 and grouped:
+        traffic = int((225.9e6 + 0.2e6) / 4)
     kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_kernel<nf4>"}.get((args.quant, args.tokens == 1), "gemm_kernel")
     out = {
         "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
@@ -321,7 +327,7 @@ def main():
         "bytes_per_step": nbytes,
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
             "kernel": kernel, "launches_per_step": dec.launches,
             "avg_launch_us": round(launch_us, 3), "bytes_per_launch": nbytes // dec.launches,
         },

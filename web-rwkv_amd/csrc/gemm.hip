@@ -9,25 +9,30 @@
 // tokens) or sit close to that point.  The decomposition follows from it:
 //   * a workgroup (4 waves) owns 64*MRT weight rows x 16*NTILE tokens x one K range; wave w
 //     owns MRT row tiles of 16 as the MFMA "A" side.  Weight bytes go from HBM straight
-//     into the A registers of the one wave that uses them (each byte is read once and never
+//     into registers of the one wave that uses them (each byte is read once and never
 //     shared, an LDS tile for them would only add traffic); the activation tile, shared by
 //     the four waves, is staged as f16 in double-buffered LDS and read back as "B" operands
 //     with ds_read_b128, each B operand serving MRT MFMAs;
-//   * weights are prefetched several K steps ahead through a ring of register buffers
-//     (a step is far shorter than HBM latency), activations two steps ahead; loads are
-//     issued activations first, weights after, because loads return in issue order;
+//   * weights are prefetched NBUF K steps ahead through a ring of register buffers,
+//     activations and scale words two steps ahead; loads are issued activations first,
+//     weights after, because loads return in issue order;
 //   * K is split over workgroups (grid.y) until there are enough of them to fill 256 CUs;
 //     every split stores its partial tile to its own slice of an f32 scratch array and a
 //     second, tiny kernel sums the slices, applies the activation and stores the output
 //     type.  Without a split the first kernel stores directly.
 //
-// The scales never enter the matrix cores, which keeps the f16 operands exact:
-//   int8: A holds the codes as f16 (1024 + u, one v_perm_b32 per two weights); after each
-//         128-block   out += s * D + (min - 1024 s) * sum_k x,  s = (max - min) / 255,
-//         with sum_k x per token taken once per workgroup while the tile is staged.
+// The scales never enter the matrix cores, which keeps the f16 operands exact (rounding a
+// dequantised weight to f16 would cost ~2^-11 of its block's range per weight, too much for
+// sums that cancel):
+//   int8: A holds the codes as f16 integers (1024 + u, one v_perm_b32 per two weights);
+//         after each 128-block   out += s * D + (min - 1024 s) * sum_k x,
+//         s = (max - min) / 255; (s, min - 1024 s) per row and sum_k x per token are staged
+//         in LDS next to the activation tile by the threads that load them.
 //   nf4:  A holds table values split into two f16 halves (hi + lo * 2^-11, exact to
 //         2^-22), fetched per byte (two weights) from a 256-entry LDS table; after each
 //         64-block   out += absmax * (D_hi + 2^-11 D_lo).
+// D is produced by MFMAs that start from a zero C operand, in ordinary vector registers,
+// so the only per-block work outside the matrix cores is one or two fmas per output.
 #include "wrq_device.h"
 #include "wrq_host.h"
 
@@ -57,6 +62,9 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     return (uint32_t)f2h(a) | ((uint32_t)f2h(b) << 16);
 }
 
+__device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
+__device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
+
 __device__ __forceinline__ float dot2_ones(uint32_t v, float acc) {
     // acc + lo(v) + hi(v) with f32 accumulation: v_dot2_f32_f16 against (1.0, 1.0)
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v), half2v{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
@@ -70,10 +78,11 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-template <int NTILE>
+// LDS: 2 x activation tile [BN][kPitch] f16 | 2 x row scales [BM] float2 | 2 x token sums [BN] f32 | nf4 pair table
+template <int MRT, int NTILE>
 constexpr size_t gemm_lds_bytes(int quant) {
-    return (size_t)2 * 16 * NTILE * kPitch * sizeof(uint16_t) + (size_t)2 * 16 * NTILE * sizeof(float) +
-           (quant == kNf4 ? 256 * sizeof(uint2) : 0);
+    return (size_t)2 * 16 * NTILE * kPitch * sizeof(uint16_t) + (size_t)2 * 64 * MRT * sizeof(float2) +
+           (size_t)2 * 16 * NTILE * sizeof(float) + (quant == kNf4 ? 256 * sizeof(uint2) : 0);
 }
 
 struct GemmArgs {
@@ -83,15 +92,18 @@ struct GemmArgs {
 };
 
 template <int QUANT, typename XT, int MRT, int NTILE>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
     const MatmulArgs &a = ga.m;
     constexpr int BN = 16 * NTILE;
     constexpr int BM = 64 * MRT;
-    constexpr int NW = QUANT == kInt8 ? 2 : 1; // 16-byte weight registers per row tile and step
+    constexpr int NW = QUANT == kInt8 ? 2 : 1;               // 16-byte weight registers per row tile and step
+    constexpr int WSTEP = QUANT == kInt8 ? kStep : kStep / 2; // packed bytes per row and step
     extern __shared__ __align__(16) uint8_t smem[];
     uint16_t(*xs)[BN * kPitch] = reinterpret_cast<uint16_t(*)[BN * kPitch]>(smem);
-    float(*sxs)[BN] = reinterpret_cast<float(*)[BN]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t));
-    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BN * sizeof(float));
+    float2(*scl)[BM] = reinterpret_cast<float2(*)[BM]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t));
+    float(*sxs)[BN] = reinterpret_cast<float(*)[BN]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BM * sizeof(float2));
+    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BM * sizeof(float2) +
+                                            (size_t)2 * BN * sizeof(float));
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r16 = lane & 15, g = lane >> 4;
@@ -101,15 +113,25 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
     const uint32_t K = a.K;
     const uint32_t k_begin = blockIdx.y * ga.k_per_split;
     const uint32_t k_end = min(K, k_begin + ga.k_per_split);
-    const uint32_t row_base = blockIdx.x * BM + wave * (16 * MRT);
+    const uint32_t nsteps = (k_end - k_begin) / kStep;
+    const uint32_t last = nsteps - 1;
+    const uint32_t row_local = wave * (16 * MRT); // first row of this wave inside the workgroup
+    const uint32_t row_base = blockIdx.x * BM + row_local;
 
-    uint64_t e_row[MRT], e_frow[MRT];
+    // this lane's A-side row of every row tile
+    const uint8_t *wp[MRT];
 #pragma unroll
     for (int i = 0; i < MRT; i++) {
-        const uint32_t row = min(row_base + 16 * i + r16, a.R - 1);    // A-side row of this lane
-        const uint32_t frow = min(row_base + 16 * i + 4 * g, a.R - 4); // first of its 4 D-side rows
-        e_row[i] = ((uint64_t)b * a.R + row) * K; // flat element index of (row, 0)
-        e_frow[i] = ((uint64_t)b * a.R + frow) * K;
+        const uint32_t row = min(row_base + 16 * i + r16, a.R - 1);
+        const uint64_t e = ((uint64_t)b * a.R + row) * K + k_begin; // flat element index of (row, k_begin)
+        wp[i] = QUANT == kInt8 ? a.w + e + 16 * g : a.w + (e >> 1) + 8 * g;
+    }
+    // scale words (one 32-bit word per row and step for both formats: a (min, max) pair, or the
+    // absmax of two 64-blocks): thread t < BM fetches those of workgroup row t
+    const uint32_t *sp;
+    {
+        const uint32_t row = min(blockIdx.x * BM + min(tid, (uint32_t)BM - 1), a.R - 1);
+        sp = reinterpret_cast<const uint32_t *>(a.scale) + ((((uint64_t)b * a.R + row) * K + k_begin) >> 7);
     }
 
     if (QUANT == kNf4) {
@@ -122,64 +144,73 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
     // activation tile staging: piece p of a tile is 8 consecutive k of one token; the 16 pieces
     // of a token sit in 16 adjacent lanes, one DPP row
     constexpr int NPIECE = NTILE; // pieces per thread: BN * 16 / 256
-    const XT *xbase = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
-    uint4 xreg[NPIECE];
-    auto load_tile = [&](uint32_t kb) {
+    struct Stage {
+        uint4 x[NPIECE];
+        uint32_t sc;
+    };
+    const XT *xp[NPIECE];
+#pragma unroll
+    for (int p = 0; p < NPIECE; p++) {
+        const uint32_t piece = tid + 256 * p;
+        const uint32_t tok = min(t0 + (piece >> 4), a.T - 1);
+        xp[p] = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride + (uint64_t)tok * a.x_token_stride + k_begin +
+                ((piece & 15) << 3);
+    }
+    auto load_stage = [&](uint32_t step, Stage &st) {
 #pragma unroll
         for (int p = 0; p < NPIECE; p++) {
-            const uint32_t piece = tid + 256 * p;
-            const uint32_t tok = min(t0 + (piece >> 4), a.T - 1);
-            const XT *src = xbase + (uint64_t)tok * a.x_token_stride + kb + ((piece & 15) << 3);
+            const XT *src = xp[p] + step * kStep;
             if constexpr (sizeof(XT) == 2) {
-                xreg[p] = load128(src);
+                st.x[p] = load128(src);
             } else {
                 const uint4 v0 = load128(src), v1 = load128(src + 4);
-                xreg[p] = make_uint4(pack_h2(__uint_as_float(v0.x), __uint_as_float(v0.y)),
+                st.x[p] = make_uint4(pack_h2(__uint_as_float(v0.x), __uint_as_float(v0.y)),
                                      pack_h2(__uint_as_float(v0.z), __uint_as_float(v0.w)),
                                      pack_h2(__uint_as_float(v1.x), __uint_as_float(v1.y)),
                                      pack_h2(__uint_as_float(v1.z), __uint_as_float(v1.w)));
             }
         }
+        st.sc = sp[step];
     };
-    auto store_tile = [&](int buf) {
+    auto store_stage = [&](const Stage &st, int buf) {
 #pragma unroll
         for (int p = 0; p < NPIECE; p++) {
             const uint32_t piece = tid + 256 * p;
-            *reinterpret_cast<uint4 *>(&xs[buf][(piece >> 4) * kPitch + ((piece & 15) << 3)]) = xreg[p];
+            *reinterpret_cast<uint4 *>(&xs[buf][(piece >> 4) * kPitch + ((piece & 15) << 3)]) = st.x[p];
             if (QUANT == kInt8) {
-                float s = dot2_ones(xreg[p].x, 0.0f);
-                s = dot2_ones(xreg[p].y, s);
-                s = dot2_ones(xreg[p].z, s);
-                s = dot2_ones(xreg[p].w, s);
+                float s = dot2_ones(st.x[p].x, 0.0f);
+                s = dot2_ones(st.x[p].y, s);
+                s = dot2_ones(st.x[p].z, s);
+                s = dot2_ones(st.x[p].w, s);
                 s = row16_sum(s);
                 if ((tid & 15) == 0) sxs[buf][piece >> 4] = s;
             }
         }
+        if (BM == 256 || tid < BM) {
+            const float lo = h2f((uint16_t)(st.sc & 0xffffu)), hi = h2f((uint16_t)(st.sc >> 16));
+            if (QUANT == kInt8) {
+                const float s = (hi - lo) * (1.0f / 255.0f); // (min, max) -> (s, min - 1024 s)
+                scl[buf][tid] = make_float2(s, fmaf(-1024.0f, s, lo));
+            } else {
+                scl[buf][tid] = make_float2(lo, hi); // absmax of the step's two 64-blocks
+            }
+        }
     };
 
-    // packed weights and scale blocks of one step for this lane, per row tile: int8 2 x 16 B of
-    // codes + 4 (min, max) pairs (one per D-side row), nf4 2 x 8 B + 4 absmax pairs
+    // packed weights of one step for this lane, per row tile: int8 2 x 16 B of codes, nf4 2 x 8 B
     struct StepRegs {
         uint4 w[MRT][NW];
-        uint32_t sc[MRT][4];
     };
-    auto load_w = [&](uint32_t kb, StepRegs &dst) {
+    auto load_w = [&](uint32_t step, StepRegs &dst) {
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
+            const uint8_t *p = wp[i] + step * WSTEP;
             if (QUANT == kInt8) {
-                dst.w[i][0] = load128_stream(a.w + e_row[i] + kb + 16 * g);
-                dst.w[i][NW - 1] = load128_stream(a.w + e_row[i] + kb + 64 + 16 * g);
-#pragma unroll
-                for (int d = 0; d < 4; d++)
-                    dst.sc[i][d] = reinterpret_cast<const uint32_t *>(a.scale)[(e_frow[i] + (uint64_t)d * K + kb) >> 7];
+                dst.w[i][0] = load128_stream(p);
+                dst.w[i][NW - 1] = load128_stream(p + 64);
             } else {
-                const uint8_t *p = a.w + ((e_row[i] + kb) >> 1);
-                const uint2 v0 = load64_stream(p + 8 * g);
-                const uint2 v1 = load64_stream(p + 32 + 8 * g);
+                const uint2 v0 = load64_stream(p), v1 = load64_stream(p + 32);
                 dst.w[i][0] = make_uint4(v0.x, v0.y, v1.x, v1.y);
-#pragma unroll
-                for (int d = 0; d < 4; d++)
-                    dst.sc[i][d] = *reinterpret_cast<const uint32_t *>(&a.scale[(e_frow[i] + (uint64_t)d * K + kb) >> 6]);
             }
         }
     };
@@ -189,64 +220,57 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
     for (int i = 0; i < MRT; i++)
 #pragma unroll
         for (int n = 0; n < NTILE; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
+    const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // one K step on the matrix cores: weights `cur` against the activation tile in LDS buffer `buf`
+    // one K step on the matrix cores: weights `cur` against the activation tile in LDS buffer `buf`.
+    // Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
     auto compute = [&](const StepRegs &cur, int buf) {
-        const uint16_t *xt = xs[buf];
+        const uint16_t *xt = xs[buf] + r16 * kPitch + 16 * g;
+        // scales of the 4 D-side rows of this lane, per row tile: (s, c) x 4 or (absmax0, absmax1) x 4
+        float4 sc0[MRT], sc1[MRT];
+#pragma unroll
+        for (int i = 0; i < MRT; i++) {
+            const float4 *q = reinterpret_cast<const float4 *>(&scl[buf][row_local + 16 * i + 4 * g]);
+            sc0[i] = q[0];
+            sc1[i] = q[1];
+        }
         if (QUANT == kInt8) {
-            float s_row[MRT][4], c_row[MRT][4];
             HalfPack A[MRT][4];
 #pragma unroll
             for (int i = 0; i < MRT; i++) {
-#pragma unroll
-                for (int d = 0; d < 4; d++) {
-                    const uint32_t mm = cur.sc[i][d];
-                    const float mn = h2f((uint16_t)(mm & 0xffffu)), mx = h2f((uint16_t)(mm >> 16));
-                    s_row[i][d] = (mx - mn) * (1.0f / 255.0f);
-                    c_row[i][d] = fmaf(-1024.0f, s_row[i][d], mn);
-                }
                 const uint32_t w[8] = {cur.w[i][0].x,      cur.w[i][0].y,      cur.w[i][0].z,      cur.w[i][0].w,
                                        cur.w[i][NW - 1].x, cur.w[i][NW - 1].y, cur.w[i][NW - 1].z, cur.w[i][NW - 1].w};
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    // 8 weights = dwords 2j, 2j+1 -> f16 codes 1024 + u
-                    A[i][j].u[0] = __builtin_amdgcn_perm(0x64646464u, w[2 * j], 0x04010400u);
-                    A[i][j].u[1] = __builtin_amdgcn_perm(0x64646464u, w[2 * j], 0x04030402u);
-                    A[i][j].u[2] = __builtin_amdgcn_perm(0x64646464u, w[2 * j + 1], 0x04010400u);
-                    A[i][j].u[3] = __builtin_amdgcn_perm(0x64646464u, w[2 * j + 1], 0x04030402u);
+                for (int d = 0; d < 8; d++) {
+                    // 4 codes of one dword -> f16 pairs 1024 + u
+                    A[i][d >> 1].u[2 * (d & 1)] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04010400u);
+                    A[i][d >> 1].u[2 * (d & 1) + 1] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04030402u);
                 }
             }
 #pragma unroll
             for (int n = 0; n < NTILE; n++) {
                 float4v D[MRT];
 #pragma unroll
-                for (int i = 0; i < MRT; i++) D[i] = float4v{0.f, 0.f, 0.f, 0.f};
-                const uint16_t *xrow = xt + (n * 16 + r16) * kPitch + 16 * g;
-#pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    // A[.][j] covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
                     HalfPack B;
-                    const uint4 v = *reinterpret_cast<const uint4 *>(xrow + 64 * (j >> 1) + 8 * (j & 1));
+                    const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * kPitch + 64 * (j >> 1) + 8 * (j & 1));
                     B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
 #pragma unroll
-                    for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, D[i], 0, 0, 0);
+                    for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, j == 0 ? zero4 : D[i], 0, 0, 0);
                 }
                 const float sx = sxs[buf][n * 16 + r16];
 #pragma unroll
-                for (int i = 0; i < MRT; i++)
-#pragma unroll
-                    for (int d = 0; d < 4; d++) out[i][n][d] = fmaf(s_row[i][d], D[i][d], fmaf(c_row[i][d], sx, out[i][n][d]));
+                for (int i = 0; i < MRT; i++) {
+                    out[i][n][0] = fmaf(sc0[i].x, D[i][0], fmaf(sc0[i].y, sx, out[i][n][0]));
+                    out[i][n][1] = fmaf(sc0[i].z, D[i][1], fmaf(sc0[i].w, sx, out[i][n][1]));
+                    out[i][n][2] = fmaf(sc1[i].x, D[i][2], fmaf(sc1[i].y, sx, out[i][n][2]));
+                    out[i][n][3] = fmaf(sc1[i].z, D[i][3], fmaf(sc1[i].w, sx, out[i][n][3]));
+                }
             }
         } else {
             HalfPack Ah[MRT][4], Al[MRT][4];
-            float am_row[MRT][2][4];
 #pragma unroll
             for (int i = 0; i < MRT; i++) {
-#pragma unroll
-                for (int d = 0; d < 4; d++) {
-                    am_row[i][0][d] = h2f((uint16_t)(cur.sc[i][d] & 0xffffu));
-                    am_row[i][1][d] = h2f((uint16_t)(cur.sc[i][d] >> 16));
-                }
                 const uint32_t w[4] = {cur.w[i][0].x, cur.w[i][0].y, cur.w[i][0].z, cur.w[i][0].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
@@ -260,87 +284,90 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
             }
 #pragma unroll
             for (int n = 0; n < NTILE; n++) {
-                const uint16_t *xrow = xt + (n * 16 + r16) * kPitch + 16 * g;
 #pragma unroll
                 for (int blk = 0; blk < 2; blk++) {
                     float4v Dh[MRT], Dl[MRT];
 #pragma unroll
-                    for (int i = 0; i < MRT; i++) Dh[i] = Dl[i] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
                     for (int j = 0; j < 2; j++) {
-                        // dword 2 blk + j covers k = 64 blk + 16 g + 8 j .. + 8
                         HalfPack B;
-                        const uint4 v = *reinterpret_cast<const uint4 *>(xrow + 64 * blk + 8 * j);
+                        const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * kPitch + 64 * blk + 8 * j);
                         B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
 #pragma unroll
                         for (int i = 0; i < MRT; i++) {
-                            Dh[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[i][2 * blk + j].h, B.h, Dh[i], 0, 0, 0);
-                            Dl[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[i][2 * blk + j].h, B.h, Dl[i], 0, 0, 0);
+                            Dh[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[i][2 * blk + j].h, B.h, j == 0 ? zero4 : Dh[i], 0, 0, 0);
+                            Dl[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[i][2 * blk + j].h, B.h, j == 0 ? zero4 : Dl[i], 0, 0, 0);
                         }
                     }
 #pragma unroll
-                    for (int i = 0; i < MRT; i++)
+                    for (int i = 0; i < MRT; i++) {
+                        const float am[4] = {blk ? sc0[i].y : sc0[i].x, blk ? sc0[i].w : sc0[i].z, blk ? sc1[i].y : sc1[i].x,
+                                             blk ? sc1[i].w : sc1[i].z};
 #pragma unroll
-                        for (int d = 0; d < 4; d++)
-                            out[i][n][d] = fmaf(am_row[i][blk][d], fmaf(Dl[i][d], 1.0f / 2048.0f, Dh[i][d]), out[i][n][d]);
+                        for (int d = 0; d < 4; d++) out[i][n][d] = fmaf(am[d], fmaf(Dl[i][d], 1.0f / 2048.0f, Dh[i][d]), out[i][n][d]);
+                    }
                 }
             }
         }
     };
 
-    // ring of NBUF weight steps in flight, activation tile two steps ahead; the step loop is
-    // unrolled by NBUF so that every ring slot is a fixed set of registers
-    constexpr int NBUF = MRT >= 4 ? 2 : 4;
-    const uint32_t nsteps = (k_end - k_begin) / kStep;
+    // ring of NBUF weight steps in flight, activation tile and scale words two steps ahead; the
+    // step loop is unrolled by NBUF so that every ring slot is a fixed set of registers.
+    // Refills past the K range re-read the last step (unconditional loads: the ring registers
+    // never pass through a control-flow join); only the compute part of such steps is skipped.
+    constexpr int NBUF = MRT * NTILE >= 8 ? 2 : 4;
     StepRegs ring[NBUF];
-    uint4 xring[2][NPIECE];
-    auto load_x = [&](uint32_t s, uint4(&dst)[NPIECE]) {
-        load_tile(k_begin + s * kStep);
+    Stage stage[2];
+    load_stage(0, stage[0]);
+    load_stage(min(1u, last), stage[1]);
 #pragma unroll
-        for (int p = 0; p < NPIECE; p++) dst[p] = xreg[p];
-    };
-    auto stage_x = [&](const uint4(&src)[NPIECE], int buf) {
-#pragma unroll
-        for (int p = 0; p < NPIECE; p++) xreg[p] = src[p];
-        store_tile(buf);
-    };
-    load_x(0, xring[0]);
-    if (nsteps > 1) load_x(1, xring[1]);
-#pragma unroll
-    for (int j = 0; j < NBUF; j++)
-        if ((uint32_t)j < nsteps) load_w(k_begin + j * kStep, ring[j]);
-    for (uint32_t base = 0; base < nsteps; base += NBUF) {
+    for (int j = 0; j < NBUF; j++) load_w(min((uint32_t)j, last), ring[j]);
+    for (uint32_t s0 = 0; s0 < nsteps; s0 += NBUF) {
 #pragma unroll
         for (int j = 0; j < NBUF; j++) {
-            const uint32_t s = base + j;
+            const uint32_t s = s0 + j;
+            __builtin_amdgcn_sched_barrier(0); // steps do not interleave: one set of operand registers
             if (s < nsteps) {
-                stage_x(xring[j & 1], j & 1);
+                store_stage(stage[j & 1], j & 1);
                 lds_barrier();
-                const StepRegs cur = ring[j];
-                // activations first, weights after: loads complete in issue order
-                if (s + 2 < nsteps) load_x(s + 2, xring[j & 1]);
-                if (s + NBUF < nsteps) load_w(k_begin + (s + NBUF) * kStep, ring[j]);
-                compute(cur, j & 1);
+                compute(ring[j], j & 1);
             }
+            // refill the slots just consumed; the scheduling barrier keeps the loads below the
+            // last use of the old values, so they can target the same registers
+            __builtin_amdgcn_sched_barrier(0);
+            load_stage(min(s + 2, last), stage[j & 1]);
+            load_w(min(s + NBUF, last), ring[j]);
         }
     }
 
     // D layout of a 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
+    if (ga.scratch) {
 #pragma unroll
-    for (int i = 0; i < MRT; i++) {
-        const uint32_t orow = row_base + 16 * i + 4 * g;
+        for (int i = 0; i < MRT; i++) {
+            const uint32_t orow = row_base + 16 * i + 4 * g;
 #pragma unroll
-        for (int n = 0; n < NTILE; n++) {
-            const uint32_t t = t0 + n * 16 + r16;
-            if (t < a.T && orow < a.R) {
-                if (ga.scratch) {
+            for (int n = 0; n < NTILE; n++) {
+                const uint32_t t = t0 + n * 16 + r16;
+                if (t < a.T && orow < a.R) {
                     float *dst = ga.scratch + (((uint64_t)blockIdx.y * a.B + b) * a.T + t) * a.R + orow;
                     *reinterpret_cast<float4 *>(dst) = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
-                } else {
+                }
+            }
+        }
+        return;
+    }
+    act_dispatch(a.act, [&](auto act_tag) {
+        constexpr int ACT = decltype(act_tag)::value;
+#pragma unroll
+        for (int i = 0; i < MRT; i++) {
+            const uint32_t orow = row_base + 16 * i + 4 * g;
+#pragma unroll
+            for (int n = 0; n < NTILE; n++) {
+                const uint32_t t = t0 + n * 16 + r16;
+                if (t < a.T && orow < a.R) {
                     const uint64_t idx = (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + orow;
                     float v[4];
 #pragma unroll
-                    for (int d = 0; d < 4; d++) v[d] = act_apply(a.act, out[i][n][d]);
+                    for (int d = 0; d < 4; d++) v[d] = act_one<ACT>(out[i][n][d]);
                     if (a.out_f16) {
                         *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) =
                             make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
@@ -350,7 +377,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs ga) {
                 }
             }
         }
-    }
+    });
 }
 
 // Second half of a split-K product: sum of the partial slices, activation, output type.
@@ -362,9 +389,18 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, co
     const uint64_t bt = q / quads_per_token, r = (q - bt * quads_per_token) * 4;
     const uint64_t b = bt / a.T, t = bt - b * a.T;
     const uint64_t slice = (uint64_t)a.B * a.T * a.R;
+    const float *src = scratch + bt * a.R + r;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t k = 0; k < splits; k++) {
-        const float4 v = *reinterpret_cast<const float4 *>(scratch + k * slice + bt * a.R + r);
+    uint32_t k = 0;
+    for (; k + 4 <= splits; k += 4) { // four slices in flight
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4 *>(src + (k + u) * slice);
+#pragma unroll
+        for (int u = 0; u < 4; u++) { s.x += v[u].x; s.y += v[u].y; s.z += v[u].z; s.w += v[u].w; }
+    }
+    for (; k < splits; k++) {
+        const float4 v = *reinterpret_cast<const float4 *>(src + k * slice);
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
     const float v[4] = {act_apply(a.act, s.x), act_apply(a.act, s.y), act_apply(a.act, s.z), act_apply(a.act, s.w)};
@@ -398,7 +434,7 @@ float *scratch_ptr() {
 
 template <int QUANT, typename XT, int MRT, int NTILE>
 int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
-    constexpr size_t lds = gemm_lds_bytes<NTILE>(QUANT);
+    constexpr size_t lds = gemm_lds_bytes<MRT, NTILE>(QUANT);
     auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE>;
     if (lds > 48 * 1024) {
         // one-time opt-in to more than the default dynamic LDS limit
@@ -443,7 +479,6 @@ int launch_shape(hipStream_t stream, const MatmulArgs &a) {
     int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? 4 : 8;
     int mrt = T <= 32 ? 1 : 2;
     if ((uint64_t)a.R * a.B >= 16384 && T > 16) mrt = 2;
-    if ((uint64_t)a.R * a.B >= 32768 && T > 64) mrt = 4;
     mrt = env_int("WRQ_GEMM_MRT", mrt);
     ntile = env_int("WRQ_GEMM_NTILE", ntile);
     const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
@@ -465,7 +500,6 @@ int launch_shape(hipStream_t stream, const MatmulArgs &a) {
     if (mrt == M && ntile == N) return launch_one<QUANT, XT, M, N>(stream, a, ksplit);
     WRQ_CASE(1, 1) WRQ_CASE(1, 2) WRQ_CASE(1, 4) WRQ_CASE(1, 8)
     WRQ_CASE(2, 1) WRQ_CASE(2, 2) WRQ_CASE(2, 4) WRQ_CASE(2, 8)
-    WRQ_CASE(4, 2) WRQ_CASE(4, 4) WRQ_CASE(4, 8)
 #undef WRQ_CASE
     return launch_one<QUANT, XT, 1, 2>(stream, a, ksplit);
 }

@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/wrq.h"
 
 namespace wrq {
@@ -26,27 +28,55 @@ struct MatmulArgs {
     int act;
 };
 
-__device__ __forceinline__ float act_apply(int act, float x) {
-    // src/tensor/ops.rs:205-235
-    switch (act) {
-    case WRQ_ACT_SQUARED_RELU: {
-        float p = fmaxf(x, 0.0f);
+// One activation, chosen at compile time (src/tensor/ops.rs:205-235).
+template <int ACT>
+__device__ __forceinline__ float act_one(float x) {
+    if constexpr (ACT == WRQ_ACT_SQUARED_RELU) {
+        const float p = fmaxf(x, 0.0f);
         return p * p;
-    }
-    case WRQ_ACT_TANH:
+    } else if constexpr (ACT == WRQ_ACT_TANH) {
         return x > 42.0f ? 1.0f : tanhf(x);
-    case WRQ_ACT_STABLE_EXP:
+    } else if constexpr (ACT == WRQ_ACT_STABLE_EXP) {
         return expf(-expf(x));
-    case WRQ_ACT_OPPOSITE_EXP:
+    } else if constexpr (ACT == WRQ_ACT_OPPOSITE_EXP) {
         return -expf(x);
-    case WRQ_ACT_SOFTPLUS:
+    } else if constexpr (ACT == WRQ_ACT_SOFTPLUS) {
         return logf(1.0f + expf(x));
-    case WRQ_ACT_SIGMOID:
+    } else if constexpr (ACT == WRQ_ACT_SIGMOID) {
         return 1.0f / (1.0f + expf(-x));
-    case WRQ_ACT_SILU:
+    } else if constexpr (ACT == WRQ_ACT_SILU) {
         return x / (1.0f + expf(-x));
-    default:
+    } else {
         return x;
+    }
+}
+
+__device__ __forceinline__ float act_apply(int act, float x) {
+    switch (act) {
+    case WRQ_ACT_SQUARED_RELU: return act_one<WRQ_ACT_SQUARED_RELU>(x);
+    case WRQ_ACT_TANH: return act_one<WRQ_ACT_TANH>(x);
+    case WRQ_ACT_STABLE_EXP: return act_one<WRQ_ACT_STABLE_EXP>(x);
+    case WRQ_ACT_OPPOSITE_EXP: return act_one<WRQ_ACT_OPPOSITE_EXP>(x);
+    case WRQ_ACT_SOFTPLUS: return act_one<WRQ_ACT_SOFTPLUS>(x);
+    case WRQ_ACT_SIGMOID: return act_one<WRQ_ACT_SIGMOID>(x);
+    case WRQ_ACT_SILU: return act_one<WRQ_ACT_SILU>(x);
+    default: return x;
+    }
+}
+
+// Calls f(std::integral_constant<int, ACT>) for the run-time activation: hoists the
+// choice out of element loops.
+template <typename F>
+__device__ __forceinline__ void act_dispatch(int act, F &&f) {
+    switch (act) {
+    case WRQ_ACT_SQUARED_RELU: f(std::integral_constant<int, WRQ_ACT_SQUARED_RELU>{}); break;
+    case WRQ_ACT_TANH: f(std::integral_constant<int, WRQ_ACT_TANH>{}); break;
+    case WRQ_ACT_STABLE_EXP: f(std::integral_constant<int, WRQ_ACT_STABLE_EXP>{}); break;
+    case WRQ_ACT_OPPOSITE_EXP: f(std::integral_constant<int, WRQ_ACT_OPPOSITE_EXP>{}); break;
+    case WRQ_ACT_SOFTPLUS: f(std::integral_constant<int, WRQ_ACT_SOFTPLUS>{}); break;
+    case WRQ_ACT_SIGMOID: f(std::integral_constant<int, WRQ_ACT_SIGMOID>{}); break;
+    case WRQ_ACT_SILU: f(std::integral_constant<int, WRQ_ACT_SILU>{}); break;
+    default: f(std::integral_constant<int, WRQ_ACT_NONE>{}); break;
     }
 }
 
