@@ -217,6 +217,31 @@ def test_gemm_against_truth(gpu, oracle, kind, K, R, T):
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("mrt,ntile", [(1, 1), (1, 2), (1, 4), (1, 8), (2, 1), (2, 2), (2, 4), (2, 8)], ids=str)
+def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, monkeypatch):
+    # every tile instantiation of the chunk kernel, with and without split K, on a shape that
+    # leaves ragged edges everywhere: 5 steps of K (a partial stage), rows and tokens that do
+    # not fill the tiles.  WRQ_GEMM_* are the library's tuning overrides, read at every launch.
+    announce("chunk tile variant", kind, mrt, ntile)
+    K, R, T = 640, 200, 40
+    rng = np.random.default_rng(SEED + 11 + mrt * 16 + ntile)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (T, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    monkeypatch.setenv("WRQ_GEMM_MRT", str(mrt))
+    monkeypatch.setenv("WRQ_GEMM_NTILE", str(ntile))
+    for ksplit in (1, 2, 5):
+        monkeypatch.setenv("WRQ_GEMM_KSPLIT", str(ksplit))
+        for out_dtype in (np.float16, np.float32):
+            got = run(gpu, m, x, R, "mat", out_dtype, act=1)
+            assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"{kind} tile ({mrt},{ntile}) ksplit {ksplit}")
+        got32 = run(gpu, m, x.astype(np.float32), R, "mat", np.float32)
+        assert_close(got32, truth, EPS, f"{kind} tile ({mrt},{ntile}) ksplit {ksplit} f32 in")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
 def test_reference_test_data_scale(gpu, oracle, kind):
     # the reference's unit tests draw weights/inputs of magnitude ~1..5, outputs ~100 (ops.rs:2929-2937, 3072-3093)
     announce("reference test scale", kind)

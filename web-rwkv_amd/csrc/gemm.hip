@@ -11,15 +11,18 @@
 //     owns MRT row tiles of 16 as the MFMA "A" side.  Weight bytes go from HBM straight
 //     into registers of the one wave that uses them (each byte is read once and never
 //     shared, an LDS tile for them would only add traffic); the activation tile, shared by
-//     the four waves, is staged as f16 in double-buffered LDS and read back as "B" operands
-//     with ds_read_b128, each B operand serving MRT MFMAs;
-//   * weights are prefetched NBUF K steps ahead through a ring of register buffers,
-//     activations and scale words two steps ahead; loads are issued activations first,
-//     weights after, because loads return in issue order;
-//   * K is split over workgroups (grid.y) until there are enough of them to fill 256 CUs;
-//     every split stores its partial tile to its own slice of an f32 scratch array and a
-//     second, tiny kernel sums the slices, applies the activation and stores the output
-//     type.  Without a split the first kernel stores directly.
+//     the four waves, is staged as f16 in double-buffered LDS, several K steps per barrier
+//     for narrow token tiles, and read back as "B" operands with ds_read_b128, each B
+//     operand serving MRT MFMAs;
+//   * weights are prefetched NBUF K steps ahead through a ring of register buffers, the
+//     next activation stage sits in registers while the current one is consumed from LDS;
+//   * the grid numbers workgroups so that the token blocks of one row tile run on one XCD
+//     (one L2) at about the same time: their weights cross HBM once;
+//   * K is split over workgroups (grid.y) only until there is about one workgroup per CU
+//     (small products) or a few (large ones); every split stores its partial tile, in the
+//     register layout of the tile (1 KiB per store instruction), to its own slice of an f32
+//     scratch array and a second, tiny kernel sums the slices, applies the activation and
+//     stores the output type.  Without a split the first kernel stores directly.
 //
 // The scales never enter the matrix cores, which keeps the f16 operands exact (rounding a
 // dequantised weight to f16 would cost ~2^-11 of its block's range per weight, too much for
@@ -49,10 +52,9 @@ union HalfPack {
     half8 h;
 };
 
-constexpr int kStep = 128;        // K elements per step
-constexpr int kPitch = kStep + 8; // f16 elements per LDS row: 272 B keeps 16-byte alignment and rotates banks
+constexpr int kStep = 128; // K elements per step
 
-// Partial tiles of split-K launches: [split][batch][token][row].  One array per process and
+// Partial tiles of split-K launches, in the tile order of the kernel.  One array per process and
 // GPU: split-K calls that overlap in time on one GPU (different streams) would race on it,
 // calls on one stream cannot.  Nothing in it outlives a call.
 constexpr size_t kScratchFloats = 8u << 20; // 32 MiB: splits * R * T up to 8 Mi partial outputs
@@ -78,45 +80,81 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// LDS: 2 x activation tile [BN][kPitch] f16 | 2 x row scales [BM] float2 | 2 x token sums [BN] f32 | nf4 pair table
+// Tile geometry of one instantiation.  A workgroup has 4 * KG waves: 4 row groups times KG
+// "k groups" that share the staged activations and take alternate K steps, so that a CU holds
+// two waves per SIMD even when the grid gives it one workgroup; their partial tiles are
+// added through LDS at the end.  A stage is what one barrier covers: KSUB steps of 128 k of
+// the activation tile, so that narrow token tiles do not pay a barrier per 128 k.
+constexpr int KG = 1; // measured: a second k group (8 waves) gains nothing on these shapes
 template <int MRT, int NTILE>
-constexpr size_t gemm_lds_bytes(int quant) {
-    return (size_t)2 * 16 * NTILE * kPitch * sizeof(uint16_t) + (size_t)2 * 64 * MRT * sizeof(float2) +
-           (size_t)2 * 16 * NTILE * sizeof(float) + (quant == kNf4 ? 256 * sizeof(uint2) : 0);
-}
+struct Geometry {
+    static constexpr int THREADS = 256 * KG;
+    static constexpr int BN = 16 * NTILE; // tokens per workgroup
+    static constexpr int BM = 64 * MRT;   // weight rows per workgroup
+    static constexpr int KSUB0 = (NTILE >= 8 ? 1 : NTILE == 4 ? 2 : 4) / MRT;
+    static constexpr int KSUB = KSUB0 > KG ? KSUB0 : KG;                   // steps per stage
+    static constexpr int LSUB = KSUB / KG;                                 // steps per stage and k group
+    static constexpr int PITCH = kStep * KSUB + 8;                         // f16 per LDS row: +16 B rotates the banks
+    static constexpr int NPIECE = NTILE * KSUB / KG;                       // 16-byte activation pieces per thread and stage
+    static constexpr int NBUF = (LSUB >= 2 || MRT >= 2) ? 2 * LSUB : 4;    // weight steps in flight per wave (an even number of stages)
+    static constexpr int TILE_FLOATS = 1024 * MRT * NTILE;                 // outputs of one workgroup
+    // LDS: 2 x activation tile [BN][PITCH] f16 | 2 x row scales [KSUB][BM] float2 | 2 x token sums [KSUB][BN] f32 | nf4 pair table
+    static constexpr size_t lds_bytes(int quant) {
+        return (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) + (size_t)2 * KSUB * BN * sizeof(float) +
+               (quant == kNf4 ? 256 * sizeof(uint2) : 0);
+    }
+    static_assert((size_t)4 * MRT * NTILE * 1024 <= (size_t)2 * BN * PITCH * sizeof(uint16_t), "partial tiles of a k group fit the activation buffers");
+};
 
 struct GemmArgs {
     MatmulArgs m;
     uint32_t k_per_split; // K range of one workgroup, a multiple of kStep
+    uint32_t row_tiles;   // ceil(R / BM)
+    uint32_t tblocks;     // ceil(T / BN)
     float *scratch;       // null: store directly
 };
 
+// blockIdx.x -> (row tile, token block).  Workgroups are dealt round-robin to the 8 XCDs, each
+// with its own L2: the token blocks of one row tile get ids that differ by multiples of 8 and
+// follow each other, so they run on one XCD at about the same time and the weights they share
+// cross HBM once.
+__device__ __forceinline__ void tile_of_block(uint32_t id, uint32_t tblocks, uint32_t &row_tile, uint32_t &tblock) {
+    const uint32_t xcd = id & 7u, slot = id >> 3;
+    tblock = slot % tblocks;
+    row_tile = (slot / tblocks) * 8u + xcd;
+}
+
 template <int QUANT, typename XT, int MRT, int NTILE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
+__global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
+    using G = Geometry<MRT, NTILE>;
     const MatmulArgs &a = ga.m;
-    constexpr int BN = 16 * NTILE;
-    constexpr int BM = 64 * MRT;
+    constexpr int BN = G::BN, BM = G::BM, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::NBUF, THREADS = G::THREADS;
     constexpr int NW = QUANT == kInt8 ? 2 : 1;               // 16-byte weight registers per row tile and step
     constexpr int WSTEP = QUANT == kInt8 ? kStep : kStep / 2; // packed bytes per row and step
     extern __shared__ __align__(16) uint8_t smem[];
-    uint16_t(*xs)[BN * kPitch] = reinterpret_cast<uint16_t(*)[BN * kPitch]>(smem);
-    float2(*scl)[BM] = reinterpret_cast<float2(*)[BM]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t));
-    float(*sxs)[BN] = reinterpret_cast<float(*)[BN]>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BM * sizeof(float2));
-    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * kPitch * sizeof(uint16_t) + (size_t)2 * BM * sizeof(float2) +
-                                            (size_t)2 * BN * sizeof(float));
+    uint16_t(*xs)[BN * PITCH] = reinterpret_cast<uint16_t(*)[BN * PITCH]>(smem);
+    float2(*scl)[KSUB][BM] = reinterpret_cast<float2(*)[KSUB][BM]>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t));
+    float(*sxs)[KSUB][BN] =
+        reinterpret_cast<float(*)[KSUB][BN]>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2));
+    uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) +
+                                            (size_t)2 * KSUB * BN * sizeof(float));
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t row_tile, tblock;
+    tile_of_block(blockIdx.x, ga.tblocks, row_tile, tblock);
+    if (row_tile >= ga.row_tiles) return; // padding of the XCD-aware grid
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (tid >> 6) & 3, kg = tid >> 8; // row group and k group of this wave
     const uint32_t r16 = lane & 15, g = lane >> 4;
-    const uint32_t tblocks = (a.T + BN - 1) / BN;
-    const uint32_t b = blockIdx.z / tblocks;
-    const uint32_t t0 = (blockIdx.z % tblocks) * BN;
+    const uint32_t b = blockIdx.z;
+    const uint32_t t0 = tblock * BN;
     const uint32_t K = a.K;
     const uint32_t k_begin = blockIdx.y * ga.k_per_split;
     const uint32_t k_end = min(K, k_begin + ga.k_per_split);
     const uint32_t nsteps = (k_end - k_begin) / kStep;
     const uint32_t last = nsteps - 1;
+    const uint32_t nstages = (nsteps + KSUB - 1) / KSUB;
     const uint32_t row_local = wave * (16 * MRT); // first row of this wave inside the workgroup
-    const uint32_t row_base = blockIdx.x * BM + row_local;
+    const uint32_t row_base = row_tile * BM + row_local;
 
     // this lane's A-side row of every row tile
     const uint8_t *wp[MRT];
@@ -130,36 +168,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // absmax of two 64-blocks): thread t < BM fetches those of workgroup row t
     const uint32_t *sp;
     {
-        const uint32_t row = min(blockIdx.x * BM + min(tid, (uint32_t)BM - 1), a.R - 1);
+        const uint32_t row = min(row_tile * BM + min(tid, (uint32_t)BM - 1), a.R - 1);
         sp = reinterpret_cast<const uint32_t *>(a.scale) + ((((uint64_t)b * a.R + row) * K + k_begin) >> 7);
     }
 
     if (QUANT == kNf4) {
         // entry for byte v: (hi(q[v & 15]), hi(q[v >> 4])), (lo(..), lo(..)); lo scaled by 2^11
-        const float q0 = a.quant[tid & 15], q1 = a.quant[tid >> 4];
+        const float q0 = a.quant[tid & 15], q1 = a.quant[(tid >> 4) & 15];
         const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
-        pair[tid] = make_uint2(pack_h2(q0, q1), pack_h2((q0 - h0) * 2048.0f, (q1 - h1) * 2048.0f));
+        if (tid < 256) pair[tid] = make_uint2(pack_h2(q0, q1), pack_h2((q0 - h0) * 2048.0f, (q1 - h1) * 2048.0f));
     }
 
-    // activation tile staging: piece p of a tile is 8 consecutive k of one token; the 16 pieces
-    // of a token sit in 16 adjacent lanes, one DPP row
-    constexpr int NPIECE = NTILE; // pieces per thread: BN * 16 / 256
+    // activation staging: piece p of a stage is 8 consecutive k of one token; the 16 pieces of a
+    // token and step sit in 16 adjacent lanes, one DPP row
     struct Stage {
         uint4 x[NPIECE];
-        uint32_t sc;
+        uint32_t sc[KSUB];
     };
-    const XT *xp[NPIECE];
+    const XT *xp[NPIECE]; // (token, k_begin + 8 * (piece & 15)) of each piece
 #pragma unroll
     for (int p = 0; p < NPIECE; p++) {
-        const uint32_t piece = tid + 256 * p;
-        const uint32_t tok = min(t0 + (piece >> 4), a.T - 1);
+        const uint32_t piece = tid + THREADS * p;
+        const uint32_t tok = min(t0 + piece / (16 * KSUB), a.T - 1);
         xp[p] = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride + (uint64_t)tok * a.x_token_stride + k_begin +
                 ((piece & 15) << 3);
     }
-    auto load_stage = [&](uint32_t step, Stage &st) {
+    // loads of a stage; steps past the K range re-read the last step (their data is not used)
+    auto load_stage = [&](uint32_t stage, Stage &st) {
 #pragma unroll
         for (int p = 0; p < NPIECE; p++) {
-            const XT *src = xp[p] + step * kStep;
+            const uint32_t sub = ((tid + THREADS * p) / 16) % KSUB;
+            const XT *src = xp[p] + min(stage * KSUB + sub, last) * kStep;
             if constexpr (sizeof(XT) == 2) {
                 st.x[p] = load128(src);
             } else {
@@ -170,29 +209,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                                      pack_h2(__uint_as_float(v1.z), __uint_as_float(v1.w)));
             }
         }
-        st.sc = sp[step];
+#pragma unroll
+        for (int u = 0; u < KSUB; u++) st.sc[u] = sp[min(stage * KSUB + u, last)];
     };
     auto store_stage = [&](const Stage &st, int buf) {
 #pragma unroll
         for (int p = 0; p < NPIECE; p++) {
-            const uint32_t piece = tid + 256 * p;
-            *reinterpret_cast<uint4 *>(&xs[buf][(piece >> 4) * kPitch + ((piece & 15) << 3)]) = st.x[p];
+            const uint32_t piece = tid + THREADS * p;
+            const uint32_t tok = piece / (16 * KSUB), c = piece % (16 * KSUB);
+            *reinterpret_cast<uint4 *>(&xs[buf][tok * PITCH + (c << 3)]) = st.x[p];
             if (QUANT == kInt8) {
                 float s = dot2_ones(st.x[p].x, 0.0f);
                 s = dot2_ones(st.x[p].y, s);
                 s = dot2_ones(st.x[p].z, s);
                 s = dot2_ones(st.x[p].w, s);
                 s = row16_sum(s);
-                if ((tid & 15) == 0) sxs[buf][piece >> 4] = s;
+                if ((tid & 15) == 0) sxs[buf][c >> 4][tok] = s;
             }
         }
-        if (BM == 256 || tid < BM) {
-            const float lo = h2f((uint16_t)(st.sc & 0xffffu)), hi = h2f((uint16_t)(st.sc >> 16));
-            if (QUANT == kInt8) {
-                const float s = (hi - lo) * (1.0f / 255.0f); // (min, max) -> (s, min - 1024 s)
-                scl[buf][tid] = make_float2(s, fmaf(-1024.0f, s, lo));
-            } else {
-                scl[buf][tid] = make_float2(lo, hi); // absmax of the step's two 64-blocks
+        if (tid < BM) {
+#pragma unroll
+            for (int u = 0; u < KSUB; u++) {
+                const float lo = h2f((uint16_t)(st.sc[u] & 0xffffu)), hi = h2f((uint16_t)(st.sc[u] >> 16));
+                if (QUANT == kInt8) {
+                    const float s = (hi - lo) * (1.0f / 255.0f); // (min, max) -> (s, min - 1024 s)
+                    scl[buf][u][tid] = make_float2(s, fmaf(-1024.0f, s, lo));
+                } else {
+                    scl[buf][u][tid] = make_float2(lo, hi); // absmax of the step's two 64-blocks
+                }
             }
         }
     };
@@ -201,7 +245,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     struct StepRegs {
         uint4 w[MRT][NW];
     };
-    auto load_w = [&](uint32_t step, StepRegs &dst) {
+    // k group `kg` owns the steps kg, kg + KG, ...: local step m is step m * KG + kg
+    const uint32_t nlocal = (nsteps + KG - 1 - kg) / KG;
+    auto load_w = [&](uint32_t m, StepRegs &dst) {
+        const uint32_t step = min(min(m, max(nlocal, 1u) - 1) * KG + kg, last); // clamped to the K range
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
             const uint8_t *p = wp[i] + step * WSTEP;
@@ -222,15 +269,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         for (int n = 0; n < NTILE; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // one K step on the matrix cores: weights `cur` against the activation tile in LDS buffer `buf`.
+    // one K step on the matrix cores: weights `cur` against step `sub` of the stage in LDS buffer `buf`.
     // Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
-    auto compute = [&](const StepRegs &cur, int buf) {
-        const uint16_t *xt = xs[buf] + r16 * kPitch + 16 * g;
+    auto compute = [&](const StepRegs &cur, int buf, uint32_t sub) {
+        const uint16_t *xt = xs[buf] + r16 * PITCH + sub * kStep + 16 * g;
         // scales of the 4 D-side rows of this lane, per row tile: (s, c) x 4 or (absmax0, absmax1) x 4
         float4 sc0[MRT], sc1[MRT];
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
-            const float4 *q = reinterpret_cast<const float4 *>(&scl[buf][row_local + 16 * i + 4 * g]);
+            const float4 *q = reinterpret_cast<const float4 *>(&scl[buf][sub][row_local + 16 * i + 4 * g]);
             sc0[i] = q[0];
             sc1[i] = q[1];
         }
@@ -253,12 +300,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     HalfPack B;
-                    const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * kPitch + 64 * (j >> 1) + 8 * (j & 1));
+                    const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * PITCH + 64 * (j >> 1) + 8 * (j & 1));
                     B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
 #pragma unroll
                     for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, j == 0 ? zero4 : D[i], 0, 0, 0);
                 }
-                const float sx = sxs[buf][n * 16 + r16];
+                const float sx = sxs[buf][sub][n * 16 + r16];
 #pragma unroll
                 for (int i = 0; i < MRT; i++) {
                     out[i][n][0] = fmaf(sc0[i].x, D[i][0], fmaf(sc0[i].y, sx, out[i][n][0]));
@@ -290,7 +337,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
                         HalfPack B;
-                        const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * kPitch + 64 * blk + 8 * j);
+                        const uint4 v = *reinterpret_cast<const uint4 *>(xt + n * 16 * PITCH + 64 * blk + 8 * j);
                         B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
 #pragma unroll
                         for (int i = 0; i < MRT; i++) {
@@ -310,49 +357,73 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
     };
 
-    // ring of NBUF weight steps in flight, activation tile and scale words two steps ahead; the
-    // step loop is unrolled by NBUF so that every ring slot is a fixed set of registers.
-    // Refills past the K range re-read the last step (unconditional loads: the ring registers
-    // never pass through a control-flow join); only the compute part of such steps is skipped.
-    constexpr int NBUF = MRT * NTILE >= 8 ? 2 : 4;
+    // Ring of NBUF weight steps in flight, the next activation stage in registers while the
+    // current one is consumed from LDS.  The loop is unrolled over NBUF steps (an even number of
+    // stages) so that every ring slot and LDS buffer is fixed at compile time.  Refills are
+    // unconditional and clamped to the K range, so the ring registers never pass through a
+    // control-flow join; only stores and matrix work of stages and steps past the range are
+    // skipped.
     StepRegs ring[NBUF];
-    Stage stage[2];
-    load_stage(0, stage[0]);
-    load_stage(min(1u, last), stage[1]);
+    Stage stage;
+    load_stage(0, stage);
 #pragma unroll
-    for (int j = 0; j < NBUF; j++) load_w(min((uint32_t)j, last), ring[j]);
-    for (uint32_t s0 = 0; s0 < nsteps; s0 += NBUF) {
+    for (int j = 0; j < NBUF; j++) load_w(j, ring[j]);
+    for (uint32_t S0 = 0; S0 < nstages; S0 += NBUF / LSUB) {
 #pragma unroll
-        for (int j = 0; j < NBUF; j++) {
-            const uint32_t s = s0 + j;
-            __builtin_amdgcn_sched_barrier(0); // steps do not interleave: one set of operand registers
-            if (s < nsteps) {
-                store_stage(stage[j & 1], j & 1);
-                lds_barrier();
-                compute(ring[j], j & 1);
-            }
-            // refill the slots just consumed; the scheduling barrier keeps the loads below the
-            // last use of the old values, so they can target the same registers
+        for (int q = 0; q < NBUF / LSUB; q++) {
+            const uint32_t S = S0 + q;
+            const int buf = q & 1;
             __builtin_amdgcn_sched_barrier(0);
-            load_stage(min(s + 2, last), stage[j & 1]);
-            load_w(min(s + NBUF, last), ring[j]);
+            if (S < nstages) store_stage(stage, buf);
+            __builtin_amdgcn_sched_barrier(0);
+            load_stage(min(S + 1, nstages - 1), stage);
+            if (S < nstages) lds_barrier();
+#pragma unroll
+            for (int u = 0; u < LSUB; u++) {
+                const int sub = u * KG; // + kg: step of the stage taken by this k group
+                __builtin_amdgcn_sched_barrier(0); // steps do not interleave: one set of operand registers
+                if (S * KSUB + sub + kg < nsteps) compute(ring[q * LSUB + u], buf, sub + kg);
+                // refill the slot just consumed; the scheduling barrier keeps the loads below the
+                // last use of the old values, so they can target the same registers
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(S * LSUB + u + NBUF, ring[q * LSUB + u]);
+            }
         }
+    }
+
+    // add the partial tiles of the k groups through LDS (the activation buffers are free now)
+    if constexpr (KG > 1) {
+        float4 *red = reinterpret_cast<float4 *>(smem);
+        lds_barrier();
+        if (kg != 0) {
+#pragma unroll
+            for (int i = 0; i < MRT; i++)
+#pragma unroll
+                for (int n = 0; n < NTILE; n++)
+                    red[((wave * MRT + i) * NTILE + n) * 64 + lane] = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
+        }
+        lds_barrier();
+        if (kg != 0) return;
+#pragma unroll
+        for (int i = 0; i < MRT; i++)
+#pragma unroll
+            for (int n = 0; n < NTILE; n++) {
+                const float4 v = red[((wave * MRT + i) * NTILE + n) * 64 + lane];
+                out[i][n][0] += v.x; out[i][n][1] += v.y; out[i][n][2] += v.z; out[i][n][3] += v.w;
+            }
     }
 
     // D layout of a 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
     if (ga.scratch) {
+        // partial tile of this split, stored tile-major so that every store instruction writes
+        // 1 KiB in one piece: [split][batch][workgroup][wave][i][n][lane][4]
+        const uint32_t wg = blockIdx.x, nwg = gridDim.x;
+        float *dst = ga.scratch + ((((uint64_t)blockIdx.y * a.B + b) * nwg + wg) * (4 * MRT * NTILE) + wave * (MRT * NTILE)) * 256 + lane * 4;
 #pragma unroll
-        for (int i = 0; i < MRT; i++) {
-            const uint32_t orow = row_base + 16 * i + 4 * g;
+        for (int i = 0; i < MRT; i++)
 #pragma unroll
-            for (int n = 0; n < NTILE; n++) {
-                const uint32_t t = t0 + n * 16 + r16;
-                if (t < a.T && orow < a.R) {
-                    float *dst = ga.scratch + (((uint64_t)blockIdx.y * a.B + b) * a.T + t) * a.R + orow;
-                    *reinterpret_cast<float4 *>(dst) = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
-                }
-            }
-        }
+            for (int n = 0; n < NTILE; n++)
+                *reinterpret_cast<float4 *>(dst + (i * NTILE + n) * 256) = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
         return;
     }
     act_dispatch(a.act, [&](auto act_tag) {
@@ -380,16 +451,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     });
 }
 
-// Second half of a split-K product: sum of the partial slices, activation, output type.
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits) {
-    const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x; // one quad of rows
-    const uint64_t quads_per_token = a.R / 4;
-    const uint64_t total = quads_per_token * a.T * a.B;
-    if (q >= total) return;
-    const uint64_t bt = q / quads_per_token, r = (q - bt * quads_per_token) * 4;
-    const uint64_t b = bt / a.T, t = bt - b * a.T;
-    const uint64_t slice = (uint64_t)a.B * a.T * a.R;
-    const float *src = scratch + bt * a.R + r;
+// Second half of a split-K product: sum of the partial tiles over the splits, activation,
+// output type.  One thread per lane slot of the first kernel's tiles (same decoding).
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits, uint32_t nwg,
+                                                          uint32_t tblocks, uint32_t row_tiles, uint32_t mrt, uint32_t ntile) {
+    const uint32_t per_wg = 4 * mrt * ntile * 64; // lane slots per workgroup tile
+    const uint64_t slots = (uint64_t)a.B * nwg * per_wg;
+    const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= slots) return;
+    const uint32_t lane = (uint32_t)(q & 63), r16 = lane & 15, g = lane >> 4;
+    const uint32_t tp = (uint32_t)((q >> 6) % (4 * mrt * ntile));
+    const uint64_t bw = q / per_wg;
+    const uint32_t wg = (uint32_t)(bw % nwg), b = (uint32_t)(bw / nwg);
+    const uint32_t n = tp % ntile, wi = tp / ntile; // wi = wave * mrt + i
+    uint32_t row_tile, tblock;
+    tile_of_block(wg, tblocks, row_tile, tblock);
+    if (row_tile >= row_tiles) return;
+    const uint32_t row = row_tile * 64 * mrt + wi * 16 + 4 * g;
+    const uint32_t t = tblock * 16 * ntile + n * 16 + r16;
+    if (t >= a.T || row >= a.R) return;
+    const float *src = scratch + q * 4;
+    const uint64_t slice = slots * 4;
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     uint32_t k = 0;
     for (; k + 4 <= splits; k += 4) { // four slices in flight
@@ -404,7 +486,7 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, co
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
     const float v[4] = {act_apply(a.act, s.x), act_apply(a.act, s.y), act_apply(a.act, s.z), act_apply(a.act, s.w)};
-    const uint64_t idx = b * a.out_batch_stride + t * a.out_token_stride + r;
+    const uint64_t idx = (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + row;
     if (a.out_f16) {
         *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
     } else {
@@ -434,7 +516,8 @@ float *scratch_ptr() {
 
 template <int QUANT, typename XT, int MRT, int NTILE>
 int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
-    constexpr size_t lds = gemm_lds_bytes<MRT, NTILE>(QUANT);
+    using G = Geometry<MRT, NTILE>;
+    constexpr size_t lds = G::lds_bytes(QUANT);
     auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE>;
     if (lds > 48 * 1024) {
         // one-time opt-in to more than the default dynamic LDS limit
@@ -444,11 +527,15 @@ int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
     }
     GemmArgs ga;
     ga.m = a;
+    ga.row_tiles = (a.R + G::BM - 1) / G::BM;
+    ga.tblocks = (a.T + G::BN - 1) / G::BN;
+    const uint32_t nwg = (ga.row_tiles + 7) / 8 * 8 * ga.tblocks; // grid.x, padded for the XCD-aware numbering
     const uint32_t steps = a.K / kStep;
-    // the partial slices of all splits must fit the scratch array, whoever chose `ksplit`
-    const uint64_t outs = (uint64_t)a.R * a.T * a.B;
-    while (ksplit > 1 && outs * ksplit > kScratchFloats) ksplit /= 2;
+    // the partial tiles of all splits must fit the scratch array, whoever chose `ksplit`
+    const uint64_t slice = (uint64_t)a.B * nwg * G::TILE_FLOATS;
+    while (ksplit > 1 && slice * ksplit > kScratchFloats) ksplit /= 2;
     if (ksplit > steps) ksplit = steps;
+    if (ksplit < 1) ksplit = 1;
     const uint32_t steps_per = (steps + ksplit - 1) / ksplit;
     ga.k_per_split = steps_per * kStep;
     const uint32_t splits = (steps + steps_per - 1) / steps_per;
@@ -456,16 +543,18 @@ int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
     if (splits > 1) {
         ga.scratch = scratch_ptr();
         if (!ga.scratch) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
-        if (outs * splits > kScratchFloats) return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(outs * splits), (unsigned long long)kScratchFloats);
+        if (slice * splits > kScratchFloats)
+            return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slice * splits), (unsigned long long)kScratchFloats);
     }
-    const uint32_t tblocks = (a.T + 16 * NTILE - 1) / (16 * NTILE);
-    dim3 grid((a.R + 64 * MRT - 1) / (64 * MRT), splits, tblocks * a.B);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, ga);
+    if (a.B > 65535u || splits > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.B > splits ? a.B : splits, 65535u);
+    dim3 grid(nwg, splits, a.B);
+    hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), lds, stream, ga);
     int s = check_launch("matmul_mat");
     if (s != WRQ_OK) return s;
     if (splits > 1) {
-        const uint64_t quads = (uint64_t)a.R / 4 * a.T * a.B;
-        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((quads + 255) / 256)), dim3(256), 0, stream, a, ga.scratch, splits);
+        const uint64_t slots = slice / 4;
+        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, a, ga.scratch, splits, nwg,
+                           ga.tblocks, ga.row_tiles, (uint32_t)MRT, (uint32_t)NTILE);
         s = check_launch("matmul_mat (finish)");
     }
     return s;
@@ -473,26 +562,25 @@ int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
 
 template <int QUANT, typename XT>
 int launch_shape(hipStream_t stream, const MatmulArgs &a) {
-    // tokens per workgroup pass: up to 128; rows per workgroup: 64 * MRT.  More rows per
-    // workgroup re-read the activation tile less often; fewer give more workgroups.
+    // Tile choice, from sweeps over the shapes of this path (rows 4096 .. 65536, K 2048 .. 14336,
+    // 16 .. 256 tokens).  Small products (rows x tokens up to 2^20) want many small tiles: 32
+    // tokens per workgroup (4 steps per barrier), as many rows per workgroup as still give
+    // about one workgroup per CU, and K split only up to that point.  Large ones want the
+    // widest token tile, 128 rows per workgroup and K split until 2-4 workgroups per CU.
     const uint32_t T = a.T;
-    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? 4 : 8;
-    int mrt = T <= 32 ? 1 : 2;
-    if ((uint64_t)a.R * a.B >= 16384 && T > 16) mrt = 2;
-    mrt = env_int("WRQ_GEMM_MRT", mrt);
+    const uint32_t steps = a.K / kStep;
+    const uint64_t rt = (uint64_t)a.R * a.B * T;
+    const bool small = rt <= (1u << 20);
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? (small ? 2 : 4) : (small && a.K <= 8192 ? 2 : 8);
     ntile = env_int("WRQ_GEMM_NTILE", ntile);
     const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
+    int mrt = 2;
+    if (ntile <= 2 && (uint64_t)((a.R + 63) / 64) * tblocks * a.B <= 256) mrt = 1;
+    mrt = env_int("WRQ_GEMM_MRT", mrt);
     const uint64_t wgs = (uint64_t)((a.R + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
-    // split K until ~2 workgroups per CU, keeping at least 4 steps per workgroup, the partial
-    // slices inside the scratch array and their traffic (8 B per output and split) small
-    // beside the packed weights
+    const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
     uint32_t ksplit = 1;
-    const uint32_t steps = a.K / kStep;
-    const uint64_t outs = (uint64_t)a.R * a.T * a.B;
-    const uint64_t wbytes = (uint64_t)a.R * a.K * a.B / (QUANT == kInt8 ? 1 : 2);
-    while (wgs * ksplit < 512 && ksplit * 2 <= steps / 4 && outs * ksplit * 2 <= kScratchFloats &&
-           outs * ksplit * 2 * 8 <= wbytes)
-        ksplit *= 2;
+    while (wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
     ksplit = (uint32_t)env_int("WRQ_GEMM_KSPLIT", (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
@@ -510,7 +598,6 @@ int launch_shape(hipStream_t stream, const MatmulArgs &a) {
 // activation rows and output rows of 4.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
     if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
-    if ((uint64_t)a.B * ((a.T + 15) / 16) > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.B, 65535u);
     if (quant == kInt8)
         return in_f16 ? launch_shape<kInt8, __half>(stream, a) : launch_shape<kInt8, float>(stream, a);
     return in_f16 ? launch_shape<kNf4, __half>(stream, a) : launch_shape<kNf4, float>(stream, a);
