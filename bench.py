@@ -304,7 +304,7 @@ def main():
     traffic = None
     if args.quant == "int8" and args.tokens == 1 and grouped:
         traffic = int((225.9e6 + 0.2e6) / 4)
-    kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_kernel<nf4>"}.get((args.quant, args.tokens == 1), "gemm_kernel")
+    kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_nf4_oneshot_kernel"}.get((args.quant, args.tokens == 1), "gemm_kernel")
     out = {
         "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
         "value": round(tok_s, 2),

@@ -419,6 +419,128 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     }
 }
 
+// nf4, one token: the same one-shot shape (one workgroup per task of ROWS rows, NT lanes along
+// K, every load of the task requested up front).  A lane holds 32 weights (16 packed bytes) of
+// each row and the 32 activations they meet.  A packed byte is two weights: a 256-entry LDS
+// table maps it to both table values at once,
+//   f16 activations: as two f16 pairs (hi, lo * 2^11) with hi + lo exact to 2^-22, so that a
+//                    byte costs one ds_read_b64 and two v_dot2_f32_f16 against the activation pair;
+//   f32 activations: as an f32 pair and two fmas.
+// The lookups, not HBM, bound this kernel: a CU sustains about 8 of them per clock.
+template <typename XT, int ROWS, int NT>
+__global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g) {
+    constexpr int NROW16 = NT / 16; // DPP rows per workgroup
+    constexpr bool F16 = sizeof(XT) == 2;
+    __shared__ float red[ROWS][NROW16];
+    __shared__ uint2 tab[256];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t task = blockIdx.x;
+    uint32_t pi = 0;
+    for (uint32_t i = 1; i < g.n; i++)
+        if (task >= g.p[i].task_begin) pi = i;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const GemvProblem &p = g.p[pi];
+    const uint32_t K = p.K, nchunk = K >> 5;
+    const uint32_t row0 = (task - p.task_begin) * ROWS;
+    const uint32_t rows_valid = min((uint32_t)ROWS, p.R - row0);
+    const uint64_t e0 = p.e_base + (uint64_t)row0 * K; // flat index of element (row0, 0)
+    const uint8_t *wbase = p.w + (((uint64_t)row0 * K) >> 1);
+    const XT *x = reinterpret_cast<const XT *>(p.x);
+
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+
+    bool table_ready = false;
+    for (uint32_t c = tid; c < nchunk || !table_ready; c += NT) {
+        const bool live = c < nchunk;
+        const uint32_t cc = live ? c : 0; // idle lanes of the first pass repeat chunk 0 and drop it
+        constexpr int NX = F16 ? 4 : 8;
+        uint4 xv[NX];
+#pragma unroll
+        for (int i = 0; i < NX; i++) xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)cc << 5)) + 16 * i);
+        uint4 wv[ROWS];
+        uint16_t sc[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const uint32_t rr = min((uint32_t)r, rows_valid - 1);
+            const uint64_t off = (uint64_t)rr * K + ((uint64_t)cc << 5);
+            wv[r] = load128_stream(wbase + (off >> 1));
+            sc[r] = p.scale[(e0 + off) >> 6];
+        }
+        if (!table_ready) {
+            // built once, behind the loads of the first pass
+            for (uint32_t v = tid; v < 256; v += NT) {
+                const float q0 = g.quant[v & 15], q1 = g.quant[v >> 4];
+                if constexpr (F16) {
+                    const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
+                    tab[v] = make_uint2((uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16),
+                                        (uint32_t)f2h((q0 - h0) * 2048.0f) | ((uint32_t)f2h((q1 - h1) * 2048.0f) << 16));
+                } else {
+                    tab[v] = make_uint2(__float_as_uint(q0), __float_as_uint(q1));
+                }
+            }
+            __syncthreads();
+            table_ready = true;
+        }
+        if (!live) continue;
+        if constexpr (F16) {
+            const uint32_t xd[16] = {xv[0].x, xv[0].y, xv[0].z, xv[0].w, xv[1].x, xv[1].y, xv[1].z, xv[1].w,
+                                     xv[2].x, xv[2].y, xv[2].z, xv[2].w, xv[3].x, xv[3].y, xv[3].z, xv[3].w};
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+                float ph = 0.0f, pl = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    const uint2 e = tab[(w[j >> 2] >> (8 * (j & 3))) & 0xffu];
+                    ph = dot2(e.x, xd[j], ph);
+                    pl = dot2(e.y, xd[j], pl);
+                }
+                acc[r] = fmaf(h2f(sc[r]), fmaf(pl, 1.0f / 2048.0f, ph), acc[r]);
+            }
+        } else {
+            float xf[32];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                xf[4 * i] = __uint_as_float(xv[i].x);
+                xf[4 * i + 1] = __uint_as_float(xv[i].y);
+                xf[4 * i + 2] = __uint_as_float(xv[i].z);
+                xf[4 * i + 3] = __uint_as_float(xv[i].w);
+            }
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+                float pr = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    const uint2 e = tab[(w[j >> 2] >> (8 * (j & 3))) & 0xffu];
+                    pr = fmaf(__uint_as_float(e.x), xf[2 * j], pr);
+                    pr = fmaf(__uint_as_float(e.y), xf[2 * j + 1], pr);
+                }
+                acc[r] = fmaf(h2f(sc[r]), pr, acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const float s = row_sum(acc[r]);
+        if ((tid & 15) == 0) red[r][tid >> 4] = s;
+    }
+    __syncthreads();
+    // NROW16 partials per output row: 16 lanes per row sum them, again with DPP
+    if (tid < ROWS * 16) {
+        const uint32_t r = tid >> 4, l = tid & 15;
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NROW16 / 16; i++) s += red[r][l + 16 * i];
+        if (NROW16 < 16) s = l < NROW16 ? red[r][l] : 0.0f;
+        s = row_sum(s);
+        const uint32_t row = row0 + r;
+        if (l == 0 && row < p.R) store_out(p.out, p.out_f16, row, act_apply(p.act, s));
+    }
+}
+
 // Any K the reference accepts (K % 4 for int8, K % 8 for nf4, with blocks that may
 // straddle rows): one wave per (row, token), scale looked up per group by flat index
 // exactly as the shaders do.  Slow path for odd shapes and unaligned views only.
@@ -520,6 +642,20 @@ int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
     return check_launch("matmul_vec_int8");
 }
 
+template <typename XT, int ROWS>
+int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+    const dim3 grid(g.total_tasks);
+    if (nt >= 512)
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 512>), grid, dim3(512), 0, stream, g);
+    else if (nt >= 256)
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, g);
+    else if (nt >= 128)
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 64>), grid, dim3(64), 0, stream, g);
+    return check_launch("matmul_vec_nf4");
+}
+
 bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
     const uint32_t chunk = quant == kInt8 ? 16 : 32;
     const size_t xs = in_f16 ? 2 : 4;
@@ -570,7 +706,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         for (int j = i; j < n; j++) rows_total += (uint64_t)args[j].R * args[j].B;
         // int8 at one token: the one-shot kernel (4 rows per workgroup; 8 once that still gives
         // every CU eight workgroups)
-        const bool oneshot = quant == kInt8 && T == 1 && env_int("WRQ_GEMV_ONESHOT", 1);
+        const bool oneshot = T == 1 && env_int("WRQ_GEMV_ONESHOT", 1);
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // chunks per lane: cover a whole row at once when it is short enough
@@ -581,6 +717,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         sl = env_int("WRQ_GEMV_SL", sl);
         if (tt > 1) rows = 4, sl = 1;
         if (oneshot && rows != 8) rows = 4;
+        // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
+        if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
         while (i < n && g.n < (uint32_t)kMaxGroup) {
             const MatmulArgs &a = args[i];
             if (a.R == 0 || a.T == 0 || a.B == 0) {
@@ -639,11 +777,26 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         }
         if (!g.n) continue;
         g.total_tasks = tasks;
+        if (oneshot && quant == kNf4) {
+            const uint32_t nchunk = g.p[0].K / 32;
+            int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk >= 128 ? 128 : 64;
+            nt = env_int("WRQ_GEMV_NT", nt);
+            if (nt > 512) nt = 512;
+            if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
+            int s1;
+            if (rows == 8 && nt >= 128)
+                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 8>(stream, g, nt) : launch_oneshot_nf4_nt<float, 8>(stream, g, nt);
+            else
+                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 4>(stream, g, nt) : launch_oneshot_nf4_nt<float, 4>(stream, g, nt);
+            if (s1 != WRQ_OK) return s1;
+            continue;
+        }
         if (oneshot) {
             const uint32_t nchunk = g.p[0].K / 16;
             // one lane per 16-byte chunk of a row where a workgroup can hold that many
             int nt = nchunk > 512 ? 1024 : nchunk > 256 ? 512 : nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
             nt = env_int("WRQ_GEMV_NT", nt);
+            if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;
             if (rows == 8 && nt >= 128) // the final reduction uses 16 lanes per output row
                 s1 = in_f16 ? launch_oneshot_nt<__half, 8>(stream, g, nt) : launch_oneshot_nt<float, 8>(stream, g, nt);
