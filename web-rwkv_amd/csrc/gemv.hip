@@ -709,6 +709,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         const bool oneshot = T == 1 && env_int("WRQ_GEMV_ONESHOT", 1);
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
+        // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
+        if (oneshot && quant == kInt8 && args[i].K / 16 > 512) rows = 8;
         // chunks per lane: cover a whole row at once when it is short enough
         const uint32_t groups = (args[i].K / (quant == kInt8 ? 16 : 32) + 63) / 64;
         int sl = groups >= 4 ? 4 : groups >= 2 ? 2 : 1;
@@ -794,7 +796,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (oneshot) {
             const uint32_t nchunk = g.p[0].K / 16;
             // one lane per 16-byte chunk of a row where a workgroup can hold that many
-            int nt = nchunk > 512 ? 1024 : nchunk > 256 ? 512 : nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
+            int nt = nchunk > 256 ? 512 : nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
             nt = env_int("WRQ_GEMV_NT", nt);
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;
