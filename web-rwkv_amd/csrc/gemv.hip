@@ -53,6 +53,9 @@ struct GemvProblem {
 };
 
 struct GemvGroup {
+    // first task of every product, unused entries 0xffffffff: one scalar load finds the product
+    // of a task, without a chain of dependent loads at the start of every workgroup
+    uint32_t task_begin[kMaxGroup];
     GemvProblem p[kMaxGroup];
     const float *quant;
     uint32_t n, T, total_tasks;
@@ -111,10 +114,11 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_kernel(const GemvGroup g) {
         TaskCtx c;
         c.task = task;
         uint32_t pi = 0;
-        for (uint32_t i = 1; i < g.n; i++)
-            if (task >= g.p[i].task_begin) pi = i;
+#pragma unroll
+        for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+            if (task >= g.task_begin[i]) pi = i;
         pi = __builtin_amdgcn_readfirstlane(pi); // uniform: the descriptor is read with scalar loads
-        const GemvProblem &p = g.p[pi];
+        const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
         c.K = p.K;
         c.R = p.R;
         c.x_lds = p.x_lds;
@@ -326,10 +330,11 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
-    for (uint32_t i = 1; i < g.n; i++)
-        if (task >= g.p[i].task_begin) pi = i;
+#pragma unroll
+    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+        if (task >= g.task_begin[i]) pi = i;
     pi = __builtin_amdgcn_readfirstlane(pi);
-    const GemvProblem &p = g.p[pi];
+    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
     const uint32_t K = p.K, nchunk = K >> 4;
     const uint32_t row0 = (task - p.task_begin) * ROWS;
     const uint32_t rows_valid = min((uint32_t)ROWS, p.R - row0);
@@ -436,10 +441,11 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
-    for (uint32_t i = 1; i < g.n; i++)
-        if (task >= g.p[i].task_begin) pi = i;
+#pragma unroll
+    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+        if (task >= g.task_begin[i]) pi = i;
     pi = __builtin_amdgcn_readfirstlane(pi);
-    const GemvProblem &p = g.p[pi];
+    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
     const uint32_t K = p.K, nchunk = K >> 5;
     const uint32_t row0 = (task - p.task_begin) * ROWS;
     const uint32_t rows_valid = min((uint32_t)ROWS, p.R - row0);
@@ -696,6 +702,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
     int i = 0;
     while (i < n) {
         GemvGroup g{};
+        for (int j = 0; j < kMaxGroup; j++) g.task_begin[j] = 0xffffffffu;
         g.quant = args[i].quant;
         g.T = T;
         size_t lds = lds_base;
@@ -753,6 +760,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 p.R = a.R;
                 p.x_lds = (uint32_t)(lds - lds_base);
                 p.task_begin = tasks;
+                g.task_begin[g.n - 1] = tasks;
                 p.out_f16 = a.out_f16;
                 p.act = a.act;
                 lds += need;
