@@ -86,8 +86,9 @@ typedef struct wrq_tensor_view {
  * NULL is the default stream. */
 typedef void *wrq_stream;
 
-/* Loads the code object on the current device and checks that it is a gfx950.
- * Optional: every entry point does this on first use. */
+/* Loads the code object on the current device, checks that it is a gfx950 and resolves the
+ * library's per-device scratch array.  Optional, but call it once per device before
+ * capturing entry points into a HIP graph: first use otherwise does the same lookups. */
 int wrq_init(void);
 
 int wrq_abi_version(void);

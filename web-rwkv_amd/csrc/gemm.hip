@@ -594,6 +594,10 @@ int launch_shape(hipStream_t stream, const MatmulArgs &a) {
 
 } // namespace
 
+int prepare_gemm_scratch() {
+    return scratch_ptr() ? WRQ_OK : fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+}
+
 // Preconditions (checked by the caller): K % 128 == 0, R % 4 == 0, 16-byte aligned
 // activation rows and output rows of 4.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {

@@ -246,7 +246,7 @@ int wrq_init(void) {
     if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "hipGetDeviceProperties: %s", hipGetErrorString(e));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(WRQ_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
-    return WRQ_OK;
+    return prepare_gemm_scratch();
 }
 
 int wrq_quantize_mat_int8(wrq_stream stream, const wrq_tensor *input, const wrq_tensor *minmax,

@@ -31,5 +31,8 @@ int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a
 int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
 // Chunk-shaped products (T >= 16): f16 MFMA.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+// Resolves the split-K scratch array of the current device (also done lazily by the first
+// chunk product; calling it from wrq_init keeps the lookup out of stream capture).
+int prepare_gemm_scratch();
 
 } // namespace wrq
