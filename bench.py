@@ -241,6 +241,111 @@ def sweep(wrq, torch, args):
     return rows
 
 
+MIN_TOKEN_CHUNK_SIZE = 32
+
+
+def rnn_iter_next(state, chunk):
+    """One RnnIter step (src/runtime/infer/rnn.rs:280-335): how many tokens of each slot enter
+    the next run.  `state` is a list of [generating, tokens_to_read]; updated in place."""
+    remains = [1 if gen else read for gen, read in state]
+    num_token = min(sum(remains), chunk)
+    if num_token > MIN_TOKEN_CHUNK_SIZE:
+        num_token -= num_token % MIN_TOKEN_CHUNK_SIZE
+    lens = [0] * len(state)
+    while num_token > 0:
+        live = [r for r in remains if r > 0]
+        if not live:
+            break
+        mid = min(live)
+        for i, r in enumerate(remains):
+            if r == 0:
+                continue
+            take = min(mid, num_token)
+            num_token -= take
+            lens[i] += take
+            remains[i] -= take
+    for i, n in enumerate(lens):
+        if n > 0:
+            state[i][0] = remains[i] == 0
+            state[i][1] = remains[i]
+    return lens
+
+
+def schedule(wrq, torch, args, layers, C, H):
+    """Config 5: a serving schedule instead of one step size.  `slots` requests with prompts of
+    16..1024 tokens arrive together, the reference's RnnIter cuts every run (chunk 256), every
+    request then decodes 128 tokens; a finished request leaves its slot empty.  The matrix path
+    of every run is replayed from a HIP graph per distinct run length T: chunk kernels for
+    T % 32 == 0, decode kernels otherwise (src/runtime/v6.rs:568-570)."""
+    rng = np.random.default_rng(SEED + 5)
+    slots, chunk, gen_len = args.slots, 256, 128
+    chunk = max(chunk, MIN_TOKEN_CHUNK_SIZE)
+    prompts = rng.integers(16, 1025, size=slots)
+    state = [[False, int(p)] for p in prompts]  # RnnIter state per slot
+    to_gen = [gen_len] * slots
+    runs = []  # tokens per run
+    while True:
+        if not any(read > 0 for _, read in state):
+            break
+        lens = rnn_iter_next(state, chunk)
+        T = sum(lens)
+        if T == 0:
+            break
+        runs.append(T)
+        for i in range(slots):
+            # every run starts from a fresh iterator over what is left to read (JobInput::step,
+            # rnn.rs:233-240); a slot whose input is exhausted emitted a token, which is fed back
+            # as its next input while the request lasts
+            state[i][0] = False
+            if lens[i] > 0 and state[i][1] == 0 and to_gen[i] > 0:
+                to_gen[i] -= 1
+                state[i][1] = 1 if to_gen[i] > 0 else 0
+    graphs = {}
+    for T in sorted(set(runs)):
+        dec = Decode(wrq, torch, layers, C, H, T)
+        step = dec.step_grouped if (not dec.turbo and T == 1) else dec.step
+        step()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            step()
+        graphs[T] = (g, dec)
+    for g, _ in graphs.values():
+        g.replay()
+    torch.cuda.synchronize()
+    phases = {"prefill (T = 256)": [0, 0.0], "mixed (32 < T < 256)": [0, 0.0], "all slots decoding (T = 32)": [0, 0.0], "tail (T < 32)": [0, 0.0]}
+    t0 = time.perf_counter()
+    evs = []
+    for T in runs:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graphs[T][0].replay()
+        e1.record()
+        evs.append((T, e0, e1))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    nbytes = 0
+    for T, e0, e1 in evs:
+        ms = e0.elapsed_time(e1)
+        key = "prefill (T = 256)" if T == 256 else "all slots decoding (T = 32)" if T == 32 else "tail (T < 32)" if T < 32 else "mixed (32 < T < 256)"
+        phases[key][0] += T
+        phases[key][1] += ms
+        nbytes += graphs[T][1].bytes_per_step(args.quant)
+    total_tokens = sum(runs)
+    gpu_ms = sum(v[1] for v in phases.values())
+    out = {
+        "metric": "config 5: serving schedule of the quantized matrix path, tokens/s over all runs",
+        "value": round(total_tokens / wall, 1), "unit": "tok/s", "n_gpus": 1,
+        "config": {"workload": f"config 5: RWKV-v6 7B-shape, {args.layers} layers {args.quant}, {slots} slots, prompts 16..1024 (seeded), chunk 256, "
+                               f"{gen_len} decode tokens per slot, runs cut by RnnIter", "runs": len(runs), "distinct_T": len(graphs)},
+        "tokens": total_tokens, "wall_ms": round(wall * 1e3, 2), "gpu_ms": round(gpu_ms, 2),
+        "packed_GBps": round(nbytes / gpu_ms / 1e6, 1),
+        "phases": {k: {"tokens": v[0], "ms": round(v[1], 2), "tok_per_s": round(v[0] / v[1] * 1e3, 1) if v[1] else None} for k, v in phases.items()},
+        "data": "synthetic",
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -257,6 +362,8 @@ def main():
                     help="also run the plain copy (256 MiB) and stream-read probes: the dispatches rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled against")
     ap.add_argument("--sweep", action="store_true", help="per-operator sweep (configs 2 and 3) instead of the decode step")
     ap.add_argument("--all-t", action="store_true", help="with --sweep: all token counts for int8 too")
+    ap.add_argument("--schedule", action="store_true", help="config 5: multi-slot serving schedule (use with --quant nf4) instead of one step size")
+    ap.add_argument("--slots", type=int, default=32)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported (the path shards by weight rows, see DESIGN.md)")
@@ -275,6 +382,9 @@ def main():
 
     C, H = 4096, 14336
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
+    if args.schedule:
+        schedule(wrq, torch, args, layers, C, H)
+        return
     dec = Decode(wrq, torch, layers, C, H, args.tokens)
 
     grouped = not args.no_group and not dec.turbo

@@ -186,6 +186,14 @@ def test_multi_token_vec_entry(gpu, oracle, kind, T):
     got = run(gpu, m, x, R, "vec", np.float32)
     assert_close(got, ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
     assert_close(got, truth_matmul(wdeq, x), EPS, "vs float64")
+    # K that is no multiple of 128 (blocks straddle rows) stays on the VALU kernels at every T
+    K2, R2 = 1056, 64
+    w2 = gen_f16(rng, (R2, K2), 0.02)
+    x2 = gen_f16(rng, (T, K2), 1.0)
+    wp2, scale2, wdeq2 = pack(oracle, kind, w2)
+    got2 = run(gpu, gpu_matrix(gpu, kind, wp2, scale2), x2, R2, "vec", np.float32)
+    assert_close(got2, ofn(wp2, scale2, x2, out_dtype=np.float32)[0], EPS, "K = 1056 vs oracle")
+    assert_close(got2, truth_matmul(wdeq2, x2), EPS, "K = 1056 vs float64")
 
 
 # (K, R, T) for the chunk kernels: config 3 (T in 32, 128, 256), config 4 (T = 128 at 7B), the
@@ -417,3 +425,58 @@ def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind):
     assert e.value.status == gpu.ERR_SHAPE
     torch.cuda.synchronize()
     assert (group[0] == 7.0).all()
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+def test_v5_shape_layer_sequence(gpu, oracle, kind):
+    # The quantized call sites of a v5-shape layer (768 wide, FFN 2688) in the order and with the
+    # kernel choice of the model builder (src/runtime/v5.rs: att k/v/r/g, att out, ffn key with
+    # SquaredRelu, ffn value on the sparse path, ffn receptance; chunk kernels iff T % 32 == 0):
+    # a 32-token prompt run, then single-token runs.  Every product is checked against the
+    # oracle on the inputs the GPU chain actually produced.
+    import torch
+
+    announce("v5-shape layer sequence", kind)
+    C, H, LAYERS = 768, 2688, 2
+    rng = np.random.default_rng(SEED + 1)
+    names = [("att_k", C, C), ("att_v", C, C), ("att_r", C, C), ("att_g", C, C), ("att_o", C, C),
+             ("ffn_k", C, H), ("ffn_v", H, C), ("ffn_r", C, C)]
+    layers = []
+    for _ in range(LAYERS):
+        L = {}
+        for name, K, R in names:
+            wp, scale, _ = pack(oracle, kind, gen_f16(rng, (R, K), 0.02))
+            L[name] = (wp, scale, gpu_matrix(gpu, kind, wp, scale))
+        layers.append(L)
+
+    def product(entry, name, xd, R, act=0, sparse=False, turbo=False):
+        wp, scale, m = entry[name]
+        T = xd.shape[0]
+        out = torch.full((T, R), float("nan"), dtype=torch.float16, device="cuda")
+        if sparse:
+            m.matmul_op_sparse(xd, out, act, turbo=turbo)
+        else:
+            m.matmul_op(xd, out, act, turbo=turbo)
+        x = host(xd)
+        if turbo:
+            ofn = oracle.matmul_mat_int8 if kind == "int8" else oracle.matmul_mat_nf4
+            want = ofn(wp, scale, x, act=act)[0]
+        else:
+            ofn = oracle.matmul_vec_int8 if kind == "int8" else oracle.matmul_vec_nf4
+            want = ofn(wp, scale, x, act=act, sparse=sparse)[0]
+        assert_close(host(out), want, EPS, f"{kind} {name} T={T}")
+        return out
+
+    for T in (32, 1, 1):
+        turbo = gpu.turbo(T)
+        x = dev(gen_f16(rng, (T, C), 1.0))
+        for L in layers:
+            k = product(L, "att_k", x, C, turbo=turbo)
+            v = product(L, "att_v", x, C, turbo=turbo)
+            r = product(L, "att_r", x, C, turbo=turbo)
+            g = product(L, "att_g", x, C, turbo=turbo)
+            mixed = (torch.sigmoid(r.float()) * (k.float() * v.float()) + g.float()).half()
+            x = (x.float() + product(L, "att_o", mixed, C, turbo=turbo).float()).half()
+            kk = product(L, "ffn_k", x, H, act=1, turbo=turbo)  # SquaredRelu
+            vv = product(L, "ffn_v", kk, C, sparse=True, turbo=turbo)
+            rr = product(L, "ffn_r", x, C, turbo=turbo)
+            x = (x.float() + torch.sigmoid(rr.float()) * vv.float()).half()

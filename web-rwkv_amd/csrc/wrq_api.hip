@@ -3,6 +3,8 @@
 #include "wrq_device.h"
 #include "wrq_host.h"
 
+#include <stdlib.h>
+
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -175,7 +177,14 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
                          ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0) &&
                          ((uintptr_t)a.out % (4 * osz) == 0) && ((a.out_token_stride * osz) % (4 * osz) == 0) &&
                          ((a.out_batch_stride * osz) % (4 * osz) == 0);
-    const bool chunk = entry == kMat ? true : n >= 16;
+    // decode entry point with several tokens: the VALU kernels re-stream the weights once per
+    // 4 tokens, the matrix-core kernel once per 16: measured at the 7B shapes it wins from 3
+    // tokens on (7B int8 step: 3.5 ms at T = 3..16 against 4.9..9.6 ms); WRQ_VEC_CHUNK_MIN_T overrides
+    static const uint64_t chunk_min_t = [] {
+        const char *e = getenv("WRQ_VEC_CHUNK_MIN_T");
+        return (uint64_t)((e && *e) ? atoi(e) : 3);
+    }();
+    const bool chunk = entry == kMat ? true : n >= chunk_min_t;
     out.in_f16 = in_f16;
     out.mfma = chunk && mfma_ok;
     return WRQ_OK;
