@@ -184,7 +184,9 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
         const char *e = getenv("WRQ_VEC_CHUNK_MIN_T");
         return (uint64_t)((e && *e) ? atoi(e) : 3);
     }();
-    const bool chunk = entry == kMat ? true : n >= chunk_min_t;
+    // f32 activations are rounded to f16 by the matrix-core kernel: keep them on the exact VALU
+    // kernels below 16 tokens
+    const bool chunk = entry == kMat ? true : n >= (in_f16 ? chunk_min_t : (uint64_t)16);
     out.in_f16 = in_f16;
     out.mfma = chunk && mfma_ok;
     return WRQ_OK;
