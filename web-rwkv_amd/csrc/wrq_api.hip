@@ -192,12 +192,17 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     return WRQ_OK;
 }
 
+int launch_chunk(hipStream_t stream, Quant quant, const Prepared &p) {
+    if (p.a.K == 0) return launch_gemv(stream, quant, p.in_f16, p.a); // nothing to stream: plain zeros through the generic kernel
+    return launch_gemm(stream, quant, p.in_f16, p.a);
+}
+
 int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Shape4 &mshape,
            const wrq_tensor *scale, const wrq_tensor *table, const wrq_tensor_view *input,
            const wrq_tensor_view *output, int act) {
     Prepared p;
     WRQ_TRY(prepare(entry, quant, w, mshape, scale, table, input, output, act, p));
-    if (p.mfma) return launch_gemm(stream, quant, p.in_f16, p.a);
+    if (p.mfma) return launch_chunk(stream, quant, p);
     return launch_gemv(stream, quant, p.in_f16, p.a);
 }
 
@@ -206,7 +211,7 @@ int dispatch_group(hipStream_t stream, Quant quant, const Prepared *ops, int n) 
     int i = 0;
     while (i < n) {
         if (ops[i].mfma) {
-            WRQ_TRY(launch_gemm(stream, quant, ops[i].in_f16, ops[i].a));
+            WRQ_TRY(launch_chunk(stream, quant, ops[i]));
             i++;
             continue;
         }
