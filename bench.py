@@ -37,6 +37,11 @@ def int8_bytes(K, R, T=1, out_size=2):
     return K * R + 4 * K * R // 128 + 2 * K * T + out_size * R * T
 
 
+def fp16_bytes(K, R, T=1, out_size=2):
+    """Plain f16 weights (head, low-rank matrices): 2 bytes per weight."""
+    return 2 * K * R + 2 * K * T + out_size * R * T
+
+
 def nf4_bytes(K, R, T=1, out_size=2):
     return K * R // 2 + 2 * K * R // 64 + 64 + 2 * K * T + out_size * R * T
 
@@ -201,15 +206,16 @@ def sweep(wrq, torch, args):
     rows = []
     g = torch.Generator(device="cuda").manual_seed(SEED + 2)
     shapes = [(2048, 2048), (2048, 7168), (7168, 2048), (2048, 65536), (4096, 4096), (4096, 14336), (14336, 4096)]
-    for quant in ("int8", "nf4"):
-        for K, R in shapes:
+    for quant in ("int8", "nf4", "fp16"):
+        for K, R in (shapes if quant != "fp16" else [(2048, 65536), (4096, 65536), (4096, 4096)]):
             w = (torch.randn((R, K), generator=g, device="cuda") * 0.02).half()
-            m0 = wrq.Matrix.quant_u8(w) if quant == "int8" else wrq.Matrix.quant_nf4(w)
+            m0 = wrq.Matrix.quant_u8(w) if quant == "int8" else wrq.Matrix.quant_nf4(w) if quant == "nf4" else wrq.Matrix.fp16(w)
             del w
-            ncopy = max(2, int(1.5e9 // m0.w.numel()) + 1)
+            wbytes = m0.w.numel() * m0.w.element_size()
+            ncopy = max(2, int(1.5e9 // wbytes) + 1)
             ncopy = min(ncopy, 64)
-            mats = [m0] + [wrq.Matrix(m0.kind, m0.w.clone(), m0.m.clone(), m0.q) for _ in range(ncopy - 1)]
-            for T in ([1] if quant == "int8" and not args.all_t else [1, 8, 32, 128, 256]):
+            mats = [m0] + [wrq.Matrix(m0.kind, m0.w.clone(), None if m0.m is None else m0.m.clone(), m0.q) for _ in range(ncopy - 1)]
+            for T in ([1] if quant != "nf4" and not args.all_t else [1, 8, 32, 128, 256]):
                 x = torch.randn((T, K), generator=g, device="cuda").half()
                 out = torch.empty((T, R), dtype=torch.float16, device="cuda")
                 turbo = wrq.turbo(T)
@@ -230,7 +236,7 @@ def sweep(wrq, torch, args):
                         fn()
                 ms, _ = time_steps(torch, graph.replay, 5, 2)
                 us = ms * 1e3 / reps
-                nbytes = (int8_bytes if quant == "int8" else nf4_bytes)(K, R, T)
+                nbytes = (int8_bytes if quant == "int8" else nf4_bytes if quant == "nf4" else fp16_bytes)(K, R, T)
                 flops = 2.0 * K * R * T
                 rows.append({"quant": quant, "K": K, "R": R, "T": T, "us": round(us, 2),
                              "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
@@ -362,6 +368,7 @@ def main():
                     help="also run the plain copy (256 MiB) and stream-read probes: the dispatches rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled against")
     ap.add_argument("--sweep", action="store_true", help="per-operator sweep (configs 2 and 3) instead of the decode step")
     ap.add_argument("--all-t", action="store_true", help="with --sweep: all token counts for int8 too")
+    ap.add_argument("--with-head", action="store_true", help="add the fp16 head (65536 x 4096, matmul_vec_fp16 / matmul_mat_fp16) to every step")
     ap.add_argument("--schedule", action="store_true", help="config 5: multi-slot serving schedule (use with --quant nf4) instead of one step size")
     ap.add_argument("--slots", type=int, default=32)
     args = ap.parse_args()
@@ -391,6 +398,22 @@ def main():
     step = dec.step_grouped if grouped else dec.step
     if grouped:
         dec.launches = 4 * len(layers)
+    head_bytes = 0
+    if args.with_head:
+        # the head of the model (src/runtime/v6.rs:982-987): plain f16, one product per step on
+        # the last token of the run (decode) -- here on all T tokens of the step
+        gh = torch.Generator(device="cuda").manual_seed(SEED + 6)
+        head = wrq.Matrix.fp16((torch.randn((65536, C), generator=gh, device="cuda") * 0.02).half())
+        head_x = torch.randn((args.tokens, C), generator=gh, device="cuda").half()
+        head_out = torch.empty((args.tokens, 65536), dtype=torch.float32, device="cuda")
+        body = step
+
+        def step():
+            body()
+            head.matmul_op(head_x, head_out, turbo=dec.turbo)
+
+        head_bytes = fp16_bytes(C, 65536, args.tokens, 4)
+        dec.launches += 1
     if args.no_graph:
         fn = step
     else:
@@ -404,7 +427,7 @@ def main():
         fn = graph.replay
 
     ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
-    nbytes = dec.bytes_per_step(args.quant)
+    nbytes = dec.bytes_per_step(args.quant) + head_bytes
     tok_s = args.tokens * 1e3 / wall_ms
     launch_us = ms * 1e3 / dec.launches
     achieved = nbytes / dec.launches / launch_us / 1e3  # GB/s
@@ -412,7 +435,7 @@ def main():
     # scaled by what the same counters read for a 256 MiB plain copy; summary under profiles/):
     # 225.9 MB fetched + 0.2 MB written per layer of the grouped Int8 decode step, 4 launches
     traffic = None
-    if args.quant == "int8" and args.tokens == 1 and grouped:
+    if args.quant == "int8" and args.tokens == 1 and grouped and not args.with_head:
         traffic = int((225.9e6 + 0.2e6) / 4)
     kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_nf4_oneshot_kernel"}.get((args.quant, args.tokens == 1), "gemm_kernel")
     out = {
@@ -432,6 +455,7 @@ def main():
             "workload": f"config 4: RWKV-v6 7B-shape ({args.layers} layers, d_model 4096, FFN 14336), all layers {args.quant}, "
                         f"batch 1, {args.tokens} token(s) per step, quantized-matrix path only (8 products per layer)",
             "quant": args.quant, "tokens_per_step": args.tokens, "hip_graph": not args.no_graph, "grouped_launches": grouped,
+            "fp16_head": bool(args.with_head),
         },
         "hbm_gbps": round(nbytes / (ms * 1e-3) / 1e9, 1),
         "bytes_per_step": nbytes,

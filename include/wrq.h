@@ -184,6 +184,20 @@ int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const w
                        const wrq_tensor *absmax, const wrq_tensor_view *input,
                        const wrq_tensor_view *output, int act);
 
+/*
+ * Plain f16 weights: the head and the low-rank matrices of a model, which the reference keeps
+ * unquantised behind the same Matrix interface (Matrix::Fp16, src/tensor/matrix.rs:29-44).
+ *
+ * TensorOp::matmul_vec_fp16(matrix, input, output, act, sparse)   src/tensor/ops.rs:697-784
+ *   matrix f16 [K, R, B, 1]; input view [K, T, B, 1]; output view [R, T, B, 1]; K % 4 == 0.
+ * TensorOp::matmul_mat_fp16(matrix, input, output, act)           src/tensor/ops.rs:999-1061
+ *   matrix: view of an f16 tensor covering its whole parent; K, R and T multiples of 4.
+ */
+int wrq_matmul_vec_fp16(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor_view *input,
+                        const wrq_tensor_view *output, int act, int sparse);
+int wrq_matmul_mat_fp16(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor_view *input,
+                        const wrq_tensor_view *output, int act);
+
 #ifdef __cplusplus
 }
 #endif

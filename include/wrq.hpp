@@ -327,6 +327,37 @@ class TensorOp {
         });
     }
 
+    // src/tensor/ops.rs:697-784: matrix f16 [K, R, B]
+    template <typename F0, typename F1>
+    static TensorOp matmul_vec_fp16(const TensorGpu<f16> &matrix, const TensorGpuView<F0> &input,
+                                    const TensorGpuView<F1> &output, Activation act, bool sparse) {
+        const Shape os = output.shape(), is = input.shape();
+        const uint32_t m = os[0], n = os[1], b = os[2], k = is[0];
+        matrix.check_shape(Shape(k, m, b, 1));
+        check_view_shape(input, Shape(k, n, b, 1));
+        check_view_shape(output, Shape(m, n, b, 1));
+        return atom([=](wrq_stream s) {
+            const wrq_tensor a = matrix.c();
+            const wrq_tensor_view i = input.c(), o = output.c();
+            return wrq_matmul_vec_fp16(s, &a, &i, &o, (int)act, sparse);
+        });
+    }
+
+    // src/tensor/ops.rs:999-1061
+    template <typename F0, typename F1>
+    static TensorOp matmul_mat_fp16(const TensorGpuView<f16> &matrix, const TensorGpuView<F0> &input,
+                                    const TensorGpuView<F1> &output, Activation act) {
+        const Shape os = output.shape(), is = input.shape();
+        const uint32_t m = os[0], n = os[1], b = os[2], k = is[0];
+        check_view_shape(matrix, Shape(k, m, b, 1));
+        check_view_shape(input, Shape(k, n, b, 1));
+        check_view_shape(output, Shape(m, n, b, 1));
+        return atom([=](wrq_stream s) {
+            const wrq_tensor_view a = matrix.c(), i = input.c(), o = output.c();
+            return wrq_matmul_mat_fp16(s, &a, &i, &o, (int)act);
+        });
+    }
+
     Kind kind() const { return kind_; }
     const std::vector<TensorOp> &list() const { return list_; }
     const Payload &payload() const { return payload_; }
@@ -463,12 +494,15 @@ inline std::vector<float> float4_quant() {
             1.0f};
 }
 
-// Matrix { Int8 { w, m }, Fp4 { q, w, m } } (src/tensor/matrix.rs:80-94).
+// Matrix { Fp16(w), Int8 { w, m }, Fp4 { q, w, m } } (src/tensor/matrix.rs:29-44, :80-94).
 struct Matrix {
-    enum class Kind { Int8, Fp4 } kind;
+    enum class Kind { Int8, Fp4, Fp16 } kind;
     TensorGpu<uint8_t> w;
     TensorGpu<f16> m;
     TensorGpu<float> q; // Fp4 only
+    TensorGpu<f16> h;   // Fp16 only: the weights as they are
+
+    static Matrix fp16(const TensorGpu<f16> &matrix) { return Matrix{Kind::Fp16, {}, {}, {}, matrix}; }
 
     // src/tensor/matrix.rs:162-178
     static Matrix quant_u8(const TensorGpu<f16> &matrix, Queue &queue) {
@@ -477,7 +511,7 @@ struct Matrix {
         auto m = TensorGpu<f16>::init(
             Shape((uint32_t)(((shape.len() << 1) + TensorOp::INT8_BLOCK_SIZE - 1) / TensorOp::INT8_BLOCK_SIZE), 1, 1, 1));
         queue.submit(TensorOp::quantize_mat_int8(matrix, m, w));
-        return Matrix{Kind::Int8, w, m, {}};
+        return Matrix{Kind::Int8, w, m, {}, {}};
     }
     // src/tensor/matrix.rs:180-200; `table` other than the default is quant_sf4's job (:202-222)
     static Matrix quant_nf4(const TensorGpu<f16> &matrix, Queue &queue, std::vector<float> table = float4_quant()) {
@@ -488,12 +522,13 @@ struct Matrix {
         auto w = TensorGpu<uint8_t>::init(matrix_shape);
         auto m = TensorGpu<f16>::init(absmax_shape);
         queue.submit(TensorOp::quantize_mat_nf4(matrix, q, m, w));
-        return Matrix{Kind::Fp4, w, m, q};
+        return Matrix{Kind::Fp4, w, m, q, {}};
     }
 
     template <typename F0, typename F1>
     TensorOp matmul_vec_op(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output, Activation act,
                            bool sparse = false) const {
+        if (kind == Kind::Fp16) return TensorOp::matmul_vec_fp16(h, input, output, act, sparse);
         return kind == Kind::Int8 ? TensorOp::matmul_vec_int8(w, m, input, output, act, sparse)
                                   : TensorOp::matmul_vec_nf4(w, q, m, input, output, act, sparse);
     }
@@ -503,6 +538,7 @@ struct Matrix {
     }
     template <typename F0, typename F1>
     TensorOp matmul_mat_op(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output, Activation act) const {
+        if (kind == Kind::Fp16) return TensorOp::matmul_mat_fp16(TensorGpuView<f16>(h), input, output, act);
         return kind == Kind::Int8 ? TensorOp::matmul_mat_int8(TensorGpuView<uint8_t>(w), m, input, output, act)
                                   : TensorOp::matmul_mat_nf4(TensorGpuView<uint8_t>(w), q, m, input, output, act);
     }

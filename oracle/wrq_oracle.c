@@ -30,6 +30,8 @@
  *     elements so that tests can report them.
  *   - products: pinned against f64 dequantise-then-matmul (numpy) and the
  *     reference tests' formulas (src/tensor/ops.rs:3004-3018, :3199-3211).
+ *   - fp16 matrices (matmul_vec_fp16 / matmul_mat_fp16): pinned against f64 matmul of
+ *     the same f16 values (numpy), the transposed-operand trap, views and activations.
  */
 #include <math.h>
 #include <stddef.h>
@@ -513,6 +515,80 @@ void wrq_oracle_matmul_mat_nf4(const uint8_t *matrix, const wrq_view *va, const 
                             load4(input, in_dtype, view_index(vb, batch, t, k + x, 3) * 2 + 1, xb);
                             acc[j] += dot4(m, xb);
                         }
+                    }
+                }
+                float out[4];
+                for (int j = 0; j < 4; j++) out[j] = activate(act, acc[j]);
+                store4(output, out_dtype, view_index(dst, batch, t, r4, 2), out);
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------- fp16 matrices */
+
+/*
+ * src/shaders/matmul_vec_fp16.wgsl:57-120 with src/tensor/ops.rs:697-784: matrix f16
+ * [K, R, B]; 128 lanes stride over groups of 4 elements, 4 rows per workgroup, tree reduce.
+ */
+void wrq_oracle_matmul_vec_fp16(const uint16_t *matrix, uint32_t K, uint32_t R, uint32_t B,
+                                const void *input, const wrq_view *src, int in_dtype, void *output,
+                                const wrq_view *dst, int out_dtype, int act, int sparse) {
+    uint32_t T = dst->shape[1];
+    size_t stride = K / 4;
+    for (uint32_t batch = 0; batch < B; batch++)
+        for (uint32_t token = 0; token < T; token++) {
+#pragma omp parallel for schedule(static)
+            for (uint32_t channel = 0; channel < R / 4; channel++) {
+                float sketch[WG][4];
+                size_t bb = view_index(src, batch, token, 0, 2);
+                size_t cb = (size_t)batch * R * stride + (size_t)channel * 4 * stride;
+                for (uint32_t lane = 0; lane < WG; lane++) {
+                    float local[4] = {0, 0, 0, 0};
+                    for (size_t i = lane; i < stride; i += WG) {
+                        float x[4];
+                        load4(input, in_dtype, bb + i, x);
+                        if (sparse && x[0] == 0.0f && x[1] == 0.0f && x[2] == 0.0f && x[3] == 0.0f)
+                            continue;
+                        for (int r = 0; r < 4; r++) {
+                            float m[4];
+                            load4(matrix, 0, cb + i + (size_t)r * stride, m);
+                            local[r] += dot4(m, x);
+                        }
+                    }
+                    memcpy(sketch[lane], local, sizeof(local));
+                }
+                tree_reduce(sketch);
+                float out[4];
+                for (int r = 0; r < 4; r++) out[r] = activate(act, sketch[0][r]);
+                store4(output, out_dtype, view_index(dst, batch, token, channel, 2), out);
+            }
+        }
+}
+
+/*
+ * src/shaders/matmul_mat_fp16.wgsl:57-140 with src/tensor/ops.rs:999-1061: matrix view
+ * [K, R, B] f16; k runs in groups of 4 elements, 8 groups per tile step, in order.
+ */
+void wrq_oracle_matmul_mat_fp16(const uint16_t *matrix, const wrq_view *va, const void *input,
+                                const wrq_view *vb, int in_dtype, void *output, const wrq_view *dst,
+                                int out_dtype, int act) {
+    uint32_t K4a = va->shape[0] / 4, R = va->shape[1];
+    uint32_t K4b = vb->shape[0] / 4, T = vb->shape[1];
+    uint32_t B = dst->shape[2];
+    uint32_t stride = K4a < K4b ? K4a : K4b;
+    for (uint32_t batch = 0; batch < B; batch++) {
+#pragma omp parallel for schedule(static)
+        for (uint32_t r4 = 0; r4 < R / 4; r4++) {
+            for (uint32_t t = 0; t < T; t++) {
+                float acc[4] = {0, 0, 0, 0};
+                for (uint32_t k = 0; k < stride; k++) {
+                    float xb[4];
+                    load4(input, in_dtype, view_index(vb, batch, t, k, 2), xb);
+                    for (int j = 0; j < 4; j++) {
+                        float m[4];
+                        load4(matrix, 0, view_index(va, batch, r4 * 4 + j, k, 2), m);
+                        acc[j] += dot4(m, xb);
                     }
                 }
                 float out[4];

@@ -99,6 +99,10 @@ def lib():
         L.wrq_oracle_matmul_mat_int8.restype = None
         L.wrq_oracle_matmul_mat_nf4.argtypes = [vp, VP, vp, vp, vp, VP, i32, vp, VP, i32, i32]
         L.wrq_oracle_matmul_mat_nf4.restype = None
+        L.wrq_oracle_matmul_vec_fp16.argtypes = [vp, u32, u32, u32, vp, VP, i32, vp, VP, i32, i32, i32]
+        L.wrq_oracle_matmul_vec_fp16.restype = None
+        L.wrq_oracle_matmul_mat_fp16.argtypes = [vp, VP, vp, VP, i32, vp, VP, i32, i32]
+        L.wrq_oracle_matmul_mat_fp16.restype = None
         L.wrq_oracle_f32_to_f16.argtypes = [vp, vp, sz]
         L.wrq_oracle_f16_to_f32.argtypes = [vp, vp, sz]
         _lib = L
@@ -224,5 +228,35 @@ def matmul_mat_nf4(w, absmax, x, quant=NF4_QUANT, out_dtype=np.float16, act=0, v
     out, dst = _mk_out(va.shape[1], src.shape[1], va.shape[2], out_dtype, out, dst)
     lib().wrq_oracle_matmul_mat_nf4(
         _p(w), C.byref(va), _p(quant), _p(absmax), _p(x), C.byref(src), _dt(x), _p(out), C.byref(dst), _dt(out), _act(act)
+    )
+    return out
+
+
+def matmul_vec_fp16(w, x, out_dtype=np.float16, act=0, sparse=False, src=None, out=None, dst=None):
+    """matmul_vec_fp16: `w` f16 (B, R, K) or (R, K)."""
+    K, R, B = _shape3(w)
+    w = np.ascontiguousarray(w, dtype=np.float16)
+    x = np.ascontiguousarray(x)
+    if src is None:
+        src = View.full(*_shape3(x))
+    T = src.shape[1]
+    out, dst = _mk_out(R, T, B, out_dtype, out, dst)
+    lib().wrq_oracle_matmul_vec_fp16(
+        _p(w), K, R, B, _p(x), C.byref(src), _dt(x), _p(out), C.byref(dst), _dt(out), _act(act), int(sparse)
+    )
+    return out
+
+
+def matmul_mat_fp16(w, x, out_dtype=np.float16, act=0, va=None, src=None, out=None, dst=None):
+    K, R, B = _shape3(w)
+    w = np.ascontiguousarray(w, dtype=np.float16)
+    x = np.ascontiguousarray(x)
+    if va is None:
+        va = View.full(K, R, B)
+    if src is None:
+        src = View.full(*_shape3(x))
+    out, dst = _mk_out(va.shape[1], src.shape[1], va.shape[2], out_dtype, out, dst)
+    lib().wrq_oracle_matmul_mat_fp16(
+        _p(w), C.byref(va), _p(x), C.byref(src), _dt(x), _p(out), C.byref(dst), _dt(out), _act(act)
     )
     return out

@@ -217,6 +217,39 @@ static void test_gpu_layer() {
     }
 }
 
+// The head (src/runtime/v6.rs:982-987): an f16 matrix behind the same Matrix interface, one token.
+static void test_gpu_head() {
+    check(wrq_init());
+    const uint32_t C = 512, V = 2048;
+    std::mt19937 rng(7);
+    std::normal_distribution<float> nw(0.0f, 0.02f), nx(0.0f, 1.0f);
+    std::vector<f16> wh((size_t)C * V), xh(C);
+    for (auto &e : wh) e.bits = to_h(nw(rng));
+    for (auto &e : xh) e.bits = to_h(nx(rng));
+    Queue queue;
+    const Matrix head = Matrix::fp16(TensorGpu<f16>::from_data(Shape(C, V, 1, 1), wh));
+    auto x = TensorGpu<f16>::from_data(Shape(C, 1, 1, 1), xh);
+    auto out = TensorGpu<float>::init(Shape(V, 1, 1, 1));
+    queue.submit(head.matmul_op(TensorGpuView<f16>(x), TensorGpuView<float>(out), Activation::None, turbo(1)));
+    queue.sync();
+    const auto got = out.back();
+    int bad = 0;
+    for (uint32_t r = 0; r < V; r++) {
+        double acc = 0;
+        for (uint32_t k = 0; k < C; k++) acc += (double)from_h(wh[(size_t)r * C + k].bits) * from_h(xh[k].bits);
+        bad += std::fabs(acc - got[r]) > std::max(2e-3, 2e-3 * std::fabs(acc));
+    }
+    EXPECT(bad == 0);
+    bool threw = false;
+    try {
+        auto wrong = TensorGpu<float>::init(Shape(V + 4, 1, 1, 1));
+        head.matmul_op(TensorGpuView<f16>(x), TensorGpuView<float>(wrong), Activation::None, false);
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_SHAPE;
+    }
+    EXPECT(threw);
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     test_run_iter();
@@ -227,6 +260,7 @@ int main(int argc, char **argv) {
     if (!cpu_only) {
         try {
             test_gpu_layer();
+            test_gpu_head();
         } catch (const TensorError &e) {
             std::printf("FAIL: TensorError %d: %s\n", e.status, e.what());
             failures++;

@@ -480,3 +480,35 @@ def test_v5_shape_layer_sequence(gpu, oracle, kind):
             vv = product(L, "ffn_v", kk, C, sparse=True, turbo=turbo)
             rr = product(L, "ffn_r", x, C, turbo=turbo)
             x = (x.float() + torch.sigmoid(rr.float()) * vv.float()).half()
+
+
+# ---------------------------------------------------------------- plain f16 weights
+
+
+FP16_CASES = [(2048, 512, 1), (2048, 512, 2), (4096, 1024, 1), (324, 64, 5), (1056, 64, 3), (2048, 512, 17),
+              (2048, 2048, 32), (2560, 2048, 64), (4096, 4096, 128), (2048, 65536, 1), (2048, 65536, 32)]
+
+
+@pytest.mark.parametrize("K,R,T", FP16_CASES, ids=str)
+def test_fp16_matrix_products(gpu, oracle, K, R, T):
+    # matmul_vec_fp16 / matmul_mat_fp16 (head and low-rank matrices): one-token kernel, generic
+    # kernel (K % 8 != 0), per-token fallback (K % 128 != 0) and the matrix-core kernel
+    import torch
+
+    announce("fp16 matrix", K, R, T)
+    rng = np.random.default_rng(SEED + 13 + K + R + T)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (T, K), 1.0)
+    m = gpu.Matrix.fp16(dev(w))
+    truth = x.astype(np.float64) @ w.astype(np.float64).T
+    for entry in (["vec", "mat"] if T % 4 == 0 else ["vec"]):
+        for out_dtype in (np.float16, np.float32):
+            got = run(gpu, m, x, R, entry, out_dtype)
+            assert_close(got, truth, EPS, f"fp16 {K}x{R}x{T} {entry} vs float64")
+        assert_close(got, truth, 2e-4, "f32 output vs float64")
+    if R * T * K <= 2048 * 2048 * 32:
+        assert_close(got, oracle.matmul_vec_fp16(w, x, out_dtype=np.float32)[0], EPS, "vs oracle")
+        xf = x.astype(np.float32) * np.float32(1.0009765625)  # f32 activations that are not f16 values
+        got32 = run(gpu, m, xf, R, "vec", np.float32, act=1)
+        want = np.square(np.maximum(xf.astype(np.float64) @ w.astype(np.float64).T, 0.0))
+        assert_close(got32, want, EPS, "f32 activations, squared relu")

@@ -155,3 +155,47 @@ def test_row_permutation_permutes_outputs(oracle):
     a = oracle.matmul_vec_int8(u8, mm, x, out_dtype=np.float32)[0]
     b = oracle.matmul_vec_int8(u8p, mmp, x, out_dtype=np.float32)[0]
     assert np.array_equal(a[:, perm], b)
+
+
+# ------------------------------------------------------------ plain f16 weights (matmul_*_fp16)
+
+
+@pytest.mark.parametrize("K,R,T", [(320, 64, 320), (2560, 96, 4), (512, 128, 1), (36, 8, 5)], ids=str)
+def test_fp16_products_against_float64(oracle, K, R, T):
+    rng = np.random.default_rng(23 + K + R + T)
+    w = gen_f16(rng, (R, K), 0.05)
+    x = gen_f16(rng, (T, K), 1.0)
+    truth = x.astype(np.float64) @ w.astype(np.float64).T
+    assert_close(oracle.matmul_vec_fp16(w, x, out_dtype=np.float32)[0], truth, 1e-5, "vec f32 out")
+    assert_close(oracle.matmul_vec_fp16(w, x)[0], truth, 1e-3, "vec f16 out")
+    if T % 4 == 0:
+        assert_close(oracle.matmul_mat_fp16(w, x, out_dtype=np.float32)[0], truth, 1e-5, "mat f32 out")
+    # a transposed or row-shuffled weight operand must not pass
+    wrong = x.astype(np.float64) @ np.roll(w, 1, axis=0).astype(np.float64).T
+    assert not np.allclose(oracle.matmul_vec_fp16(w, x, out_dtype=np.float32)[0], wrong, atol=1e-3)
+
+
+def test_fp16_views_batch_activation_and_f32_input(oracle):
+    rng = np.random.default_rng(29)
+    K, R, T, B = 256, 16, 4, 2
+    w = gen_f16(rng, (B, R, K), 0.05)
+    x = rng.standard_normal((B, T, K), dtype=np.float32)
+    truth = np.einsum("btk,brk->btr", x.astype(np.float64), w.astype(np.float64))
+    for act, fn in ACTS.items():
+        assert_close(oracle.matmul_vec_fp16(w, x, out_dtype=np.float32, act=act), fn(truth), 2e-5, f"vec act {act}")
+        assert_close(oracle.matmul_mat_fp16(w, x, out_dtype=np.float32, act=act), fn(truth), 2e-5, f"mat act {act}")
+    # offset views, as the att_sx call sites use them (src/runtime/v6.rs:806-829)
+    parent = gen_f16(rng, (5, T, K), 1.0)
+    outp = np.full((3, T + 2, R), -7.0, dtype=np.float32)
+    src = oracle.View.make((K, T, 1), (K, T, 5), (0, 0, 3))
+    dst = oracle.View.make((R, T, 1), (R, T + 2, 3), (0, 1, 2))
+    for fn in (oracle.matmul_vec_fp16, oracle.matmul_mat_fp16):
+        outp[:] = -7.0
+        fn(w[0], parent, out_dtype=np.float32, src=src, out=outp, dst=dst)
+        want = fn(w[0], np.ascontiguousarray(parent[3]), out_dtype=np.float32)[0]
+        assert np.array_equal(outp[2, 1:1 + T], want)
+        rest = outp.copy(); rest[2, 1:1 + T] = -7.0
+        assert (rest == -7.0).all()
+    # sparse flag: skipping all-zero groups changes nothing
+    xs = gen_f16(rng, (T, K), 1.0); xs[:, 64:192] = 0
+    assert np.array_equal(oracle.matmul_vec_fp16(w[0], xs, sparse=True), oracle.matmul_vec_fp16(w[0], xs, sparse=False))

@@ -40,6 +40,7 @@ EXPORTS = [
     "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
     "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
+    "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
 ]
 MAX_GROUP = 8
 
@@ -109,6 +110,8 @@ def lib():
         L.wrq_matmul_vec_nf4.argtypes = [vp, T, T, T, V, V, i, i]
         L.wrq_matmul_mat_int8.argtypes = [vp, V, T, V, V, i]
         L.wrq_matmul_mat_nf4.argtypes = [vp, V, T, T, V, V, i]
+        L.wrq_matmul_vec_fp16.argtypes = [vp, T, V, V, i, i]
+        L.wrq_matmul_mat_fp16.argtypes = [vp, V, V, V, i]
         L.wrq_matmul_vec_int8_group.argtypes = [vp, C.POINTER(CVecInt8Op), i]
         L.wrq_matmul_vec_nf4_group.argtypes = [vp, C.POINTER(CVecNf4Op), i]
         for name in EXPORTS[4:]:
@@ -196,6 +199,16 @@ class TensorOp:
         _check(lib().wrq_matmul_mat_nf4(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(quant)), C.byref(as_tensor(absmax)),
                                         C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
 
+    @staticmethod
+    def matmul_vec_fp16(matrix, input, output, act=ACT_NONE, sparse=False, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_vec_fp16(_stream(), C.byref(as_tensor(matrix)), C.byref(as_view(input, input_view)),
+                                         C.byref(as_view(output, output_view)), act, int(sparse)))
+
+    @staticmethod
+    def matmul_mat_fp16(matrix, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_mat_fp16(_stream(), C.byref(as_view(matrix, matrix_view)), C.byref(as_view(input, input_view)),
+                                         C.byref(as_view(output, output_view)), act))
+
 
 def matmul_vec_group(ops):
     """Independent decode products in shared launches (``wrq_matmul_vec_*_group``).
@@ -225,7 +238,7 @@ def matmul_vec_group(ops):
 
 
 class Matrix:
-    """``Matrix::{Int8, Fp4}`` (src/tensor/matrix.rs:80-94): packed weights plus scales."""
+    """``Matrix::{Fp16, Int8, Fp4}`` (src/tensor/matrix.rs:29-44, :80-94): weights plus scales."""
 
     def __init__(self, kind, w, m, q=None):
         self.kind, self.w, self.m, self.q = kind, w, m, q
@@ -253,14 +266,23 @@ class Matrix:
         TensorOp.quantize_mat_nf4(matrix, q, m, w)
         return Matrix("Fp4", w, m, q)
 
+    @staticmethod
+    def fp16(matrix):
+        """Matrix::Fp16: the f16 tensor as it is."""
+        return Matrix("Fp16", matrix, None)
+
     def matmul_vec_op(self, input, output, act=ACT_NONE, sparse=False, **views):
-        if self.kind == "Int8":
+        if self.kind == "Fp16":
+            TensorOp.matmul_vec_fp16(self.w, input, output, act, sparse, **views)
+        elif self.kind == "Int8":
             TensorOp.matmul_vec_int8(self.w, self.m, input, output, act, sparse, **views)
         else:
             TensorOp.matmul_vec_nf4(self.w, self.q, self.m, input, output, act, sparse, **views)
 
     def matmul_mat_op(self, input, output, act=ACT_NONE, **views):
-        if self.kind == "Int8":
+        if self.kind == "Fp16":
+            TensorOp.matmul_mat_fp16(self.w, input, output, act, **views)
+        elif self.kind == "Int8":
             TensorOp.matmul_mat_int8(self.w, self.m, input, output, act, **views)
         else:
             TensorOp.matmul_mat_nf4(self.w, self.q, self.m, input, output, act, **views)

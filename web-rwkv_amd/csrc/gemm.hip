@@ -53,6 +53,10 @@ union HalfPack {
 };
 
 constexpr int kStep = 128; // K elements per step
+#ifndef WRQ_UNROLL_STAGES
+#define WRQ_UNROLL_STAGES 2
+#endif
+constexpr int kUnrollStages = WRQ_UNROLL_STAGES; // even
 
 // Partial tiles of split-K launches, in the tile order of the kernel.  One array per process and
 // GPU: split-K calls that overlap in time on one GPU (different streams) would race on it,
@@ -96,7 +100,11 @@ struct Geometry {
     static constexpr int LSUB = KSUB / KG;                                 // steps per stage and k group
     static constexpr int PITCH = kStep * KSUB + 8;                         // f16 per LDS row: +16 B rotates the banks
     static constexpr int NPIECE = NTILE * KSUB / KG;                       // 16-byte activation pieces per thread and stage
-    static constexpr int NBUF = (LSUB >= 2 || MRT >= 2) ? 2 * LSUB : 4;    // weight steps in flight per wave (an even number of stages)
+    // weight steps in flight per wave: two stages (an even number of them), one for plain f16
+    // weights, whose steps take twice the registers
+    static constexpr int NBUFQ = (LSUB >= 2 || MRT >= 2) ? 2 * LSUB : 4;
+    static constexpr int NBUFH = LSUB >= 2 ? LSUB : 2;
+    static constexpr int nbuf(int quant) { return quant == kFp16 ? NBUFH : NBUFQ; }
     static constexpr int TILE_FLOATS = 1024 * MRT * NTILE;                 // outputs of one workgroup
     // LDS: 2 x activation tile [BN][PITCH] f16 | 2 x row scales [KSUB][BM] float2 | 2 x token sums [KSUB][BN] f32 | nf4 pair table
     static constexpr size_t lds_bytes(int quant) {
@@ -128,9 +136,9 @@ template <int QUANT, typename XT, int MRT, int NTILE>
 __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
     using G = Geometry<MRT, NTILE>;
     const MatmulArgs &a = ga.m;
-    constexpr int BN = G::BN, BM = G::BM, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::NBUF, THREADS = G::THREADS;
-    constexpr int NW = QUANT == kInt8 ? 2 : 1;               // 16-byte weight registers per row tile and step
-    constexpr int WSTEP = QUANT == kInt8 ? kStep : kStep / 2; // packed bytes per row and step
+    constexpr int BN = G::BN, BM = G::BM, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::nbuf(QUANT), THREADS = G::THREADS;
+    constexpr int NW = QUANT == kFp16 ? 4 : QUANT == kInt8 ? 2 : 1;                        // 16-byte weight registers per row tile and step
+    constexpr int WSTEP = QUANT == kFp16 ? 2 * kStep : QUANT == kInt8 ? kStep : kStep / 2; // weight bytes per row and step
     extern __shared__ __align__(16) uint8_t smem[];
     uint16_t(*xs)[BN * PITCH] = reinterpret_cast<uint16_t(*)[BN * PITCH]>(smem);
     float2(*scl)[KSUB][BM] = reinterpret_cast<float2(*)[KSUB][BM]>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t));
@@ -143,7 +151,8 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     tile_of_block(blockIdx.x, ga.tblocks, row_tile, tblock);
     if (row_tile >= ga.row_tiles) return; // padding of the XCD-aware grid
     const uint32_t tid = threadIdx.x, lane = tid & 63;
-    const uint32_t wave = (tid >> 6) & 3, kg = tid >> 8; // row group and k group of this wave
+    const uint32_t wave = (tid >> 6) & 3;                                        // row group of this wave
+    const uint32_t kg = KG == 1 ? 0u : __builtin_amdgcn_readfirstlane(tid >> 8); // its k group
     const uint32_t r16 = lane & 15, g = lane >> 4;
     const uint32_t b = blockIdx.z;
     const uint32_t t0 = tblock * BN;
@@ -162,14 +171,14 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     for (int i = 0; i < MRT; i++) {
         const uint32_t row = min(row_base + 16 * i + r16, a.R - 1);
         const uint64_t e = ((uint64_t)b * a.R + row) * K + k_begin; // flat element index of (row, k_begin)
-        wp[i] = QUANT == kInt8 ? a.w + e + 16 * g : a.w + (e >> 1) + 8 * g;
+        wp[i] = QUANT == kFp16 ? a.w + 2 * e + 16 * g : QUANT == kInt8 ? a.w + e + 16 * g : a.w + (e >> 1) + 8 * g;
     }
     // scale words (one 32-bit word per row and step for both formats: a (min, max) pair, or the
     // absmax of two 64-blocks): thread t < BM fetches those of workgroup row t
     const uint32_t *sp;
     {
         const uint32_t row = min(row_tile * BM + min(tid, (uint32_t)BM - 1), a.R - 1);
-        sp = reinterpret_cast<const uint32_t *>(a.scale) + ((((uint64_t)b * a.R + row) * K + k_begin) >> 7);
+        sp = QUANT == kFp16 ? nullptr : reinterpret_cast<const uint32_t *>(a.scale) + ((((uint64_t)b * a.R + row) * K + k_begin) >> 7);
     }
 
     if (QUANT == kNf4) {
@@ -210,7 +219,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
             }
         }
 #pragma unroll
-        for (int u = 0; u < KSUB; u++) st.sc[u] = sp[min(stage * KSUB + u, last)];
+        for (int u = 0; u < KSUB; u++) st.sc[u] = QUANT == kFp16 ? 0u : sp[min(stage * KSUB + u, last)];
     };
     auto store_stage = [&](const Stage &st, int buf) {
 #pragma unroll
@@ -227,7 +236,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
                 if ((tid & 15) == 0) sxs[buf][c >> 4][tok] = s;
             }
         }
-        if (tid < BM) {
+        if (QUANT != kFp16 && tid < BM) {
 #pragma unroll
             for (int u = 0; u < KSUB; u++) {
                 const float lo = h2f((uint16_t)(st.sc[u] & 0xffffu)), hi = h2f((uint16_t)(st.sc[u] >> 16));
@@ -252,7 +261,10 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
             const uint8_t *p = wp[i] + step * WSTEP;
-            if (QUANT == kInt8) {
+            if (QUANT == kFp16) {
+#pragma unroll
+                for (int j = 0; j < NW; j++) dst.w[i][j] = load128_stream(p + 64 * j); // operand j: k = 32 j + 8 g .. + 8
+            } else if (QUANT == kInt8) {
                 dst.w[i][0] = load128_stream(p);
                 dst.w[i][NW - 1] = load128_stream(p + 64);
             } else {
@@ -272,6 +284,27 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     // one K step on the matrix cores: weights `cur` against step `sub` of the stage in LDS buffer `buf`.
     // Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
     auto compute = [&](const StepRegs &cur, int buf, uint32_t sub) {
+        if constexpr (QUANT == kFp16) {
+            // plain f16 weights are the A operands as loaded; the accumulators stay in the matrix cores
+            const uint16_t *xh = xs[buf] + r16 * PITCH + sub * kStep + 8 * g;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+#pragma unroll
+                for (int n = 0; n < NTILE; n++) {
+                    HalfPack B;
+                    const uint4 v = *reinterpret_cast<const uint4 *>(xh + n * 16 * PITCH + 32 * j);
+                    B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
+#pragma unroll
+                    for (int i = 0; i < MRT; i++) {
+                        HalfPack A;
+                        const uint4 &wv = cur.w[i][j < NW ? j : 0];
+                        A.u[0] = wv.x; A.u[1] = wv.y; A.u[2] = wv.z; A.u[3] = wv.w;
+                        out[i][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.h, B.h, out[i][n], 0, 0, 0);
+                    }
+                }
+            }
+            return;
+        }
         const uint16_t *xt = xs[buf] + r16 * PITCH + sub * kStep + 16 * g;
         // scales of the 4 D-side rows of this lane, per row tile: (s, c) x 4 or (absmax0, absmax1) x 4
         float4 sc0[MRT], sc1[MRT];
@@ -368,9 +401,10 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     load_stage(0, stage);
 #pragma unroll
     for (int j = 0; j < NBUF; j++) load_w(j, ring[j]);
-    for (uint32_t S0 = 0; S0 < nstages; S0 += NBUF / LSUB) {
+    constexpr int STAGES = kUnrollStages > NBUF / LSUB ? kUnrollStages : NBUF / LSUB; // stages per loop iteration
+    for (uint32_t S0 = 0; S0 < nstages; S0 += STAGES) {
 #pragma unroll
-        for (int q = 0; q < NBUF / LSUB; q++) {
+        for (int q = 0; q < STAGES; q++) {
             const uint32_t S = S0 + q;
             const int buf = q & 1;
             __builtin_amdgcn_sched_barrier(0);
@@ -381,12 +415,13 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
             for (int u = 0; u < LSUB; u++) {
                 const int sub = u * KG; // + kg: step of the stage taken by this k group
+                const int slot = (q * LSUB + u) % NBUF;
                 __builtin_amdgcn_sched_barrier(0); // steps do not interleave: one set of operand registers
-                if (S * KSUB + sub + kg < nsteps) compute(ring[q * LSUB + u], buf, sub + kg);
+                if (S * KSUB + sub + kg < nsteps) compute(ring[slot], buf, sub + kg);
                 // refill the slot just consumed; the scheduling barrier keeps the loads below the
                 // last use of the old values, so they can target the same registers
                 __builtin_amdgcn_sched_barrier(0);
-                load_w(S * LSUB + u + NBUF, ring[q * LSUB + u]);
+                load_w(S * LSUB + u + NBUF, ring[slot]);
             }
         }
     }
@@ -604,6 +639,8 @@ int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a
     if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
     if (quant == kInt8)
         return in_f16 ? launch_shape<kInt8, __half>(stream, a) : launch_shape<kInt8, float>(stream, a);
+    if (quant == kFp16)
+        return in_f16 ? launch_shape<kFp16, __half>(stream, a) : launch_shape<kFp16, float>(stream, a);
     return in_f16 ? launch_shape<kNf4, __half>(stream, a) : launch_shape<kNf4, float>(stream, a);
 }
 

@@ -120,7 +120,9 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     const Shape4 os = shape_of(output->view.shape), is = shape_of(input->view.shape);
     const uint64_t m = os.d[0], n = os.d[1], b = os.d[2], k = is.d[0];
     // src/tensor/ops.rs:805-813 (int8), :907-916 (nf4), :1094-1103, :1172-1181
-    if (quant == kInt8) {
+    if (quant == kFp16) {
+        WRQ_TRY(check_shape(mshape, Shape4{{k, m, b, 1}})); // src/tensor/ops.rs:713-720, :1015-1022
+    } else if (quant == kInt8) {
         const uint64_t len = mshape.len();
         WRQ_TRY(check_shape(shape_of(scale->shape), Shape4{{div_ceil(len << 1, WRQ_INT8_BLOCK_SIZE), 1, 1, 1}}));
         WRQ_TRY(check_shape(mshape, Shape4{{k, m, b, 1}}));
@@ -134,8 +136,8 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     WRQ_TRY(check_shape(os, Shape4{{m, n, b, 1}}));
 
     // preconditions the reference leaves to the caller
-    const uint64_t block = quant == kInt8 ? WRQ_INT8_BLOCK_SIZE : WRQ_NF4_BLOCK_SIZE;
-    const uint64_t group = quant == kInt8 ? 4 : 8; // elements per u32 of packed weights
+    const uint64_t block = quant == kFp16 ? 1 : quant == kInt8 ? WRQ_INT8_BLOCK_SIZE : WRQ_NF4_BLOCK_SIZE;
+    const uint64_t group = quant == kNf4 ? 8 : 4; // elements per load unit of the shaders (vec4 / 8 nibbles)
     if ((k * m * b) % block)
         return fail(WRQ_ERR_ALIGNMENT, "matrix size %llu is not a multiple of the %llu-element block",
                     (unsigned long long)(k * m * b), (unsigned long long)block);
@@ -145,13 +147,13 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
         return fail(WRQ_ERR_ALIGNMENT, "input view offset/stride along x not a multiple of %llu", (unsigned long long)group);
     if (output->view.offset[0] % 4 || output->view.stride[0] % 4)
         return fail(WRQ_ERR_ALIGNMENT, "output view offset/stride along x not a multiple of 4");
-    if ((uintptr_t)w % 4 || (uintptr_t)scale->data % 4 || (uintptr_t)input->data % 16 || (uintptr_t)output->data % 16)
+    if ((uintptr_t)w % (quant == kFp16 ? 8 : 4) || (scale && (uintptr_t)scale->data % 4) || (uintptr_t)input->data % 16 || (uintptr_t)output->data % 16)
         return fail(WRQ_ERR_ALIGNMENT, "device pointers must be 16-byte aligned");
     if (entry == kMat) {
         // src/tensor/ops.rs:1068-1070, :1146-1149; the k-step of the shaders fetches one
         // scale per 32 (int8) / 64 (nf4) columns
         if (n % 4) return fail(WRQ_ERR_ALIGNMENT, "tokens %llu not a multiple of 4", (unsigned long long)n);
-        const uint64_t kstep = quant == kInt8 ? 32 : 64;
+        const uint64_t kstep = quant == kFp16 ? 4 : quant == kInt8 ? 32 : 64;
         if (k % kstep) return fail(WRQ_ERR_ALIGNMENT, "input columns %llu not a multiple of %llu", (unsigned long long)k, (unsigned long long)kstep);
     }
     if (m > 0xffffffffull || n > 0xffffffffull || k > 0xffffffffull) return fail(WRQ_ERR_SIZE, "data size not match");
@@ -159,7 +161,7 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     MatmulArgs &a = out.a;
     a = MatmulArgs{};
     a.w = static_cast<const uint8_t *>(w);
-    a.scale = static_cast<const uint16_t *>(scale->data);
+    a.scale = scale ? static_cast<const uint16_t *>(scale->data) : nullptr;
     a.quant = table ? static_cast<const float *>(table->data) : nullptr;
     a.K = (uint32_t)k;
     a.R = (uint32_t)m;
@@ -192,8 +194,12 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     return WRQ_OK;
 }
 
+int launch_vec(hipStream_t stream, Quant quant, const Prepared &p) {
+    return quant == kFp16 ? launch_gemv_fp16(stream, p.in_f16, p.a) : launch_gemv(stream, quant, p.in_f16, p.a);
+}
+
 int launch_chunk(hipStream_t stream, Quant quant, const Prepared &p) {
-    if (p.a.K == 0) return launch_gemv(stream, quant, p.in_f16, p.a); // nothing to stream: plain zeros through the generic kernel
+    if (p.a.K == 0) return launch_vec(stream, quant, p); // nothing to stream: plain zeros through the generic kernel
     return launch_gemm(stream, quant, p.in_f16, p.a);
 }
 
@@ -203,7 +209,7 @@ int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Sh
     Prepared p;
     WRQ_TRY(prepare(entry, quant, w, mshape, scale, table, input, output, act, p));
     if (p.mfma) return launch_chunk(stream, quant, p);
-    return launch_gemv(stream, quant, p.in_f16, p.a);
+    return launch_vec(stream, quant, p);
 }
 
 // Runs of consecutive decode-shaped ops with one input type and token count share launches.
@@ -383,6 +389,28 @@ int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const w
     if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
     return matmul(static_cast<hipStream_t>(stream), kMat, kNf4, matrix->data, shape_of(matrix->view.shape), absmax,
                   quant, input, output, act);
+}
+
+/* plain f16 weights */
+
+int wrq_matmul_vec_fp16(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor_view *input,
+                        const wrq_tensor_view *output, int act, int sparse) {
+    (void)sparse;
+    WRQ_TRY(need_tensor(matrix, "matrix"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    return matmul(static_cast<hipStream_t>(stream), kVec, kFp16, matrix->data, shape_of(matrix->shape), nullptr, nullptr,
+                  input, output, act);
+}
+
+int wrq_matmul_mat_fp16(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor_view *input,
+                        const wrq_tensor_view *output, int act) {
+    WRQ_TRY(need_view(matrix, "matrix", false));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    return matmul(static_cast<hipStream_t>(stream), kMat, kFp16, matrix->data, shape_of(matrix->view.shape), nullptr,
+                  nullptr, input, output, act);
 }
 
 } // extern "C"

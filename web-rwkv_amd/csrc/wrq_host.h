@@ -20,7 +20,7 @@ int launch_quant_int8(hipStream_t stream, const void *in, void *minmax, void *ou
 int launch_quant_nf4(hipStream_t stream, const void *in, const void *quant, void *absmax, void *out,
                      uint64_t len);
 
-enum Quant { kInt8 = 0, kNf4 = 1 };
+enum Quant { kInt8 = 0, kNf4 = 1, kFp16 = 2 }; // kFp16: plain f16 weights (matmul_*_fp16), no scales
 
 constexpr int kMaxGroup = 8; // products per grouped decode launch
 
@@ -29,7 +29,9 @@ int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a
 // The same for `n` independent products of one quantisation, input type and token count,
 // in as few launches as their activations fit in LDS together.
 int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
-// Chunk-shaped products (T >= 16): f16 MFMA.
+// Decode-shaped products on plain f16 weights (matmul_vec_fp16).
+int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &args);
+// Chunk-shaped products: f16 MFMA.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
 // Resolves the split-K scratch array of the current device (also done lazily by the first
 // chunk product; calling it from wrq_init keeps the lookup out of stream capture).
