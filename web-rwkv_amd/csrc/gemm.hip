@@ -36,6 +36,8 @@
 //         64-block   out += absmax * (D_hi + 2^-11 D_lo).
 // D is produced by MFMAs that start from a zero C operand, in ordinary vector registers,
 // so the only per-block work outside the matrix cores is one or two fmas per output.
+// Plain f16 weights (matmul_mat_fp16, src/shaders/matmul_mat_fp16.wgsl:57-140) take the same
+// kernel: they are A operands as loaded and accumulate in the matrix cores over the whole K.
 #include "wrq_device.h"
 #include "wrq_host.h"
 
