@@ -97,16 +97,16 @@ class Decode:
 
     def step_grouped(self):
         """The same products with the independent ones of a layer sharing launches: {k, v, r, g},
-        then output, then {ffn.key, ffn.receptance}, then ffn.value (decode only)."""
+        then output, then {ffn.key, ffn.receptance}, then ffn.value."""
         wrq, C, T = self.wrq, self.C, self.T
         sq, no = wrq.ACT_SQUARED_RELU, wrq.ACT_NONE
         for L in self.layers:
             wrq.matmul_vec_group([
                 (m, self.att_sx, out, no, False, dict(input_view=((C, T, 1), (C, T, 5), (0, 0, i))))
                 for i, (m, out) in enumerate(((L.att_k, self.att_k), (L.att_v, self.att_v), (L.att_r, self.att_r), (L.att_g, self.att_g)), 1)])
-            L.att_o.matmul_op(self.att_x, self.att_o, turbo=False)
+            L.att_o.matmul_op(self.att_x, self.att_o, turbo=self.turbo)
             wrq.matmul_vec_group([(L.ffn_k, self.ffn_kx, self.ffn_k, sq, False, {}), (L.ffn_r, self.ffn_rx, self.ffn_r, no, False, {})])
-            L.ffn_v.matmul_op_sparse(self.ffn_k, self.ffn_v, turbo=False)
+            L.ffn_v.matmul_op_sparse(self.ffn_k, self.ffn_v, turbo=self.turbo)
 
     def step(self):
         wrq, C, T, turbo = self.wrq, self.C, self.T, self.turbo
@@ -309,7 +309,7 @@ def schedule(wrq, torch, args, layers, C, H):
     graphs = {}
     for T in sorted(set(runs)):
         dec = Decode(wrq, torch, layers, C, H, T)
-        step = dec.step_grouped if (not dec.turbo and T == 1) else dec.step
+        step = dec.step_grouped
         step()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
@@ -394,7 +394,7 @@ def main():
         return
     dec = Decode(wrq, torch, layers, C, H, args.tokens)
 
-    grouped = not args.no_group and not dec.turbo
+    grouped = not args.no_group
     step = dec.step_grouped if grouped else dec.step
     if grouped:
         dec.launches = 4 * len(layers)

@@ -371,14 +371,17 @@ def test_full_size_properties(gpu, oracle, kind):
     assert_close(host(om), host(ov), 2e-4, "mat vs vec")
 
 
+@pytest.mark.parametrize("T", [1, 5, 32])
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
-def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind):
-    # the independent products of a layer in shared launches: same results as one call each
+def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind, T):
+    # the independent products of a layer in shared launches: same results as one call each;
+    # one token on the decode kernels, several on the matrix-core kernel (products of one K
+    # share a launch there as well)
     import torch
 
-    announce("grouped", kind)
-    C, H, T = 1024, 3584, 1
-    rng = np.random.default_rng(SEED + 23)
+    announce("grouped", kind, T)
+    C, H = 1024, 3584
+    rng = np.random.default_rng(SEED + 23 + T)
     shapes = [(C, C), (C, C), (C, C), (C, C), (C, H), (H, C)]  # (K, R); the last two differ in K
     mats, truths = [], []
     att_sx = gen_f16(rng, (5, T, C), 1.0)

@@ -116,12 +116,16 @@ struct Geometry {
     static_assert((size_t)4 * MRT * NTILE * 1024 <= (size_t)2 * BN * PITCH * sizeof(uint16_t), "partial tiles of a k group fit the activation buffers");
 };
 
+// One launch serves up to kMaxGroup independent products with the same K, token count and
+// types (the attention projections of a layer, or ffn.key + ffn.receptance): together they
+// fill the CUs without a split of K, where each alone would need one plus its finish kernel.
 struct GemmArgs {
-    MatmulArgs m;
-    uint32_t k_per_split; // K range of one workgroup, a multiple of kStep
-    uint32_t row_tiles;   // ceil(R / BM)
-    uint32_t tblocks;     // ceil(T / BN)
-    float *scratch;       // null: store directly
+    uint32_t tile_begin[kMaxGroup]; // first blockIdx.x of every product, unused entries 0xffffffff
+    uint32_t row_tiles[kMaxGroup];  // ceil(R / BM) of every product
+    MatmulArgs m[kMaxGroup];
+    float *scratch[kMaxGroup]; // partial tiles of every product; null: store directly
+    uint32_t k_per_split;      // K range of one workgroup, a multiple of kStep
+    uint32_t tblocks;          // ceil(T / BN)
 };
 
 // blockIdx.x -> (row tile, token block).  Workgroups are dealt round-robin to the 8 XCDs, each
@@ -137,7 +141,16 @@ __device__ __forceinline__ void tile_of_block(uint32_t id, uint32_t tblocks, uin
 template <int QUANT, typename XT, int MRT, int NTILE>
 __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
     using G = Geometry<MRT, NTILE>;
-    const MatmulArgs &a = ga.m;
+    // the product of this workgroup: one scalar load of the tile starts, then its descriptor
+    uint32_t pi = 0;
+#pragma unroll
+    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+        if (blockIdx.x >= ga.tile_begin[i]) pi = i;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const MatmulArgs a = ga.m[pi];
+    const uint32_t tile_id = blockIdx.x - ga.tile_begin[pi];
+    const uint32_t my_row_tiles = ga.row_tiles[pi];
+    float *const my_scratch = ga.scratch[pi];
     constexpr int BN = G::BN, BM = G::BM, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::nbuf(QUANT), THREADS = G::THREADS;
     constexpr int NW = QUANT == kFp16 ? 4 : QUANT == kInt8 ? 2 : 1;                        // 16-byte weight registers per row tile and step
     constexpr int WSTEP = QUANT == kFp16 ? 2 * kStep : QUANT == kInt8 ? kStep : kStep / 2; // weight bytes per row and step
@@ -150,8 +163,8 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
                                             (size_t)2 * KSUB * BN * sizeof(float));
 
     uint32_t row_tile, tblock;
-    tile_of_block(blockIdx.x, ga.tblocks, row_tile, tblock);
-    if (row_tile >= ga.row_tiles) return; // padding of the XCD-aware grid
+    tile_of_block(tile_id, ga.tblocks, row_tile, tblock);
+    if (row_tile >= my_row_tiles) return; // padding of the XCD-aware grid
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (tid >> 6) & 3;                                        // row group of this wave
     const uint32_t kg = KG == 1 ? 0u : __builtin_amdgcn_readfirstlane(tid >> 8); // its k group
@@ -451,11 +464,11 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     }
 
     // D layout of a 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
-    if (ga.scratch) {
+    if (my_scratch) {
         // partial tile of this split, stored tile-major so that every store instruction writes
         // 1 KiB in one piece: [split][batch][workgroup][wave][i][n][lane][4]
-        const uint32_t wg = blockIdx.x, nwg = gridDim.x;
-        float *dst = ga.scratch + ((((uint64_t)blockIdx.y * a.B + b) * nwg + wg) * (4 * MRT * NTILE) + wave * (MRT * NTILE)) * 256 + lane * 4;
+        const uint32_t wg = tile_id, nwg = (my_row_tiles + 7) / 8 * 8 * ga.tblocks;
+        float *dst = my_scratch + ((((uint64_t)blockIdx.y * a.B + b) * nwg + wg) * (4 * MRT * NTILE) + wave * (MRT * NTILE)) * 256 + lane * 4;
 #pragma unroll
         for (int i = 0; i < MRT; i++)
 #pragma unroll
@@ -552,7 +565,7 @@ float *scratch_ptr() {
 }
 
 template <int QUANT, typename XT, int MRT, int NTILE>
-int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
+int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t ksplit) {
     using G = Geometry<MRT, NTILE>;
     constexpr size_t lds = G::lds_bytes(QUANT);
     auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE>;
@@ -563,58 +576,84 @@ int launch_one(hipStream_t stream, const MatmulArgs &a, uint32_t ksplit) {
         (void)once;
     }
     GemmArgs ga;
-    ga.m = a;
-    ga.row_tiles = (a.R + G::BM - 1) / G::BM;
-    ga.tblocks = (a.T + G::BN - 1) / G::BN;
-    const uint32_t nwg = (ga.row_tiles + 7) / 8 * 8 * ga.tblocks; // grid.x, padded for the XCD-aware numbering
-    const uint32_t steps = a.K / kStep;
+    const MatmulArgs &a0 = args[0];
+    ga.tblocks = (a0.T + G::BN - 1) / G::BN;
+    uint32_t nwg[kMaxGroup], total = 0;
+    uint64_t slice[kMaxGroup], slices = 0; // partial-tile floats of one split, per product
+    for (int i = 0; i < kMaxGroup; i++) {
+        ga.tile_begin[i] = 0xffffffffu;
+        ga.row_tiles[i] = 0;
+        ga.scratch[i] = nullptr;
+        if (i >= n) continue;
+        ga.m[i] = args[i];
+        ga.row_tiles[i] = (args[i].R + G::BM - 1) / G::BM;
+        nwg[i] = (ga.row_tiles[i] + 7) / 8 * 8 * ga.tblocks; // padded for the XCD-aware numbering
+        ga.tile_begin[i] = total;
+        total += nwg[i];
+        slice[i] = (uint64_t)args[i].B * nwg[i] * G::TILE_FLOATS;
+        slices += slice[i];
+    }
+    const uint32_t steps = a0.K / kStep;
     // the partial tiles of all splits must fit the scratch array, whoever chose `ksplit`
-    const uint64_t slice = (uint64_t)a.B * nwg * G::TILE_FLOATS;
-    while (ksplit > 1 && slice * ksplit > kScratchFloats) ksplit /= 2;
+    while (ksplit > 1 && slices * ksplit > kScratchFloats) ksplit /= 2;
     if (ksplit > steps) ksplit = steps;
     if (ksplit < 1) ksplit = 1;
     const uint32_t steps_per = (steps + ksplit - 1) / ksplit;
     ga.k_per_split = steps_per * kStep;
     const uint32_t splits = (steps + steps_per - 1) / steps_per;
-    ga.scratch = nullptr;
     if (splits > 1) {
-        ga.scratch = scratch_ptr();
-        if (!ga.scratch) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
-        if (slice * splits > kScratchFloats)
-            return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slice * splits), (unsigned long long)kScratchFloats);
+        float *base = scratch_ptr();
+        if (!base) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+        if (slices * splits > kScratchFloats)
+            return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slices * splits), (unsigned long long)kScratchFloats);
+        uint64_t off = 0;
+        for (int i = 0; i < n; i++) {
+            ga.scratch[i] = base + off;
+            off += slice[i] * splits;
+        }
     }
-    if (a.B > 65535u || splits > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.B > splits ? a.B : splits, 65535u);
-    dim3 grid(nwg, splits, a.B);
+    if (a0.B > 65535u || splits > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a0.B > splits ? a0.B : splits, 65535u);
+    dim3 grid(total, splits, a0.B);
     hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), lds, stream, ga);
     int s = check_launch("matmul_mat");
     if (s != WRQ_OK) return s;
     if (splits > 1) {
-        const uint64_t slots = slice / 4;
-        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, a, ga.scratch, splits, nwg,
-                           ga.tblocks, ga.row_tiles, (uint32_t)MRT, (uint32_t)NTILE);
+        for (int i = 0; i < n; i++) {
+            const uint64_t slots = slice[i] / 4;
+            hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, args[i], ga.scratch[i], splits,
+                               nwg[i], ga.tblocks, ga.row_tiles[i], (uint32_t)MRT, (uint32_t)NTILE);
+        }
         s = check_launch("matmul_mat (finish)");
     }
     return s;
 }
 
+// `n` products with one K, token count and batch count (the caller groups them so).
 template <int QUANT, typename XT>
-int launch_shape(hipStream_t stream, const MatmulArgs &a) {
+int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
     // Tile choice, from sweeps over the shapes of this path (rows 4096 .. 65536, K 2048 .. 14336,
     // 16 .. 256 tokens).  Small products (rows x tokens up to 2^20) want many small tiles: 32
     // tokens per workgroup (4 steps per barrier), as many rows per workgroup as still give
     // about one workgroup per CU, and K split only up to that point.  Large ones want the
     // widest token tile, 128 rows per workgroup and K split until 2-4 workgroups per CU.
+    // A group counts as one product with the rows of all its members.
+    const MatmulArgs &a = args[0];
     const uint32_t T = a.T;
     const uint32_t steps = a.K / kStep;
-    const uint64_t rt = (uint64_t)a.R * a.B * T;
+    uint64_t rows = 0, rows_max = 0;
+    for (int i = 0; i < n; i++) {
+        rows += args[i].R;
+        rows_max = args[i].R > rows_max ? args[i].R : rows_max;
+    }
+    const uint64_t rt = rows_max * a.B * T;
     const bool small = rt <= (1u << 20);
     int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? (small ? 2 : 4) : (small && a.K <= 8192 ? 2 : 8);
     ntile = env_int("WRQ_GEMM_NTILE", ntile);
     const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
     int mrt = 2;
-    if (ntile <= 2 && (uint64_t)((a.R + 63) / 64) * tblocks * a.B <= 256) mrt = 1;
+    if (ntile <= 2 && (uint64_t)((rows + 63) / 64) * tblocks * a.B <= 256) mrt = 1;
     mrt = env_int("WRQ_GEMM_MRT", mrt);
-    const uint64_t wgs = (uint64_t)((a.R + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
+    const uint64_t wgs = (uint64_t)((rows + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
     const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
     uint32_t ksplit = 1;
     while (wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
@@ -622,11 +661,11 @@ int launch_shape(hipStream_t stream, const MatmulArgs &a) {
     if (ksplit < 1) ksplit = 1;
 
 #define WRQ_CASE(M, N) \
-    if (mrt == M && ntile == N) return launch_one<QUANT, XT, M, N>(stream, a, ksplit);
+    if (mrt == M && ntile == N) return launch_one<QUANT, XT, M, N>(stream, args, n, ksplit);
     WRQ_CASE(1, 1) WRQ_CASE(1, 2) WRQ_CASE(1, 4) WRQ_CASE(1, 8)
     WRQ_CASE(2, 1) WRQ_CASE(2, 2) WRQ_CASE(2, 4) WRQ_CASE(2, 8)
 #undef WRQ_CASE
-    return launch_one<QUANT, XT, 1, 2>(stream, a, ksplit);
+    return launch_one<QUANT, XT, 1, 2>(stream, args, n, ksplit);
 }
 
 } // namespace
@@ -638,12 +677,34 @@ int prepare_gemm_scratch() {
 // Preconditions (checked by the caller): K % 128 == 0, R % 4 == 0, 16-byte aligned
 // activation rows and output rows of 4.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
-    if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
-    if (quant == kInt8)
-        return in_f16 ? launch_shape<kInt8, __half>(stream, a) : launch_shape<kInt8, float>(stream, a);
-    if (quant == kFp16)
-        return in_f16 ? launch_shape<kFp16, __half>(stream, a) : launch_shape<kFp16, float>(stream, a);
-    return in_f16 ? launch_shape<kNf4, __half>(stream, a) : launch_shape<kNf4, float>(stream, a);
+    return launch_gemm_group(stream, quant, in_f16, &a, 1);
+}
+
+// `n` <= kMaxGroup independent products of one quantisation and input type; those that share K,
+// T and B = 1 go into one launch, the others are launched one by one.
+int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n) {
+    int i = 0;
+    while (i < n) {
+        if (args[i].R == 0 || args[i].T == 0 || args[i].B == 0) {
+            i++;
+            continue;
+        }
+        int m = 1;
+        if (args[i].B == 1)
+            while (i + m < n && m < kMaxGroup && args[i + m].B == 1 && args[i + m].R > 0 && args[i + m].K == args[i].K &&
+                   args[i + m].T == args[i].T)
+                m++;
+        int s;
+        if (quant == kInt8)
+            s = in_f16 ? launch_shape<kInt8, __half>(stream, args + i, m) : launch_shape<kInt8, float>(stream, args + i, m);
+        else if (quant == kFp16)
+            s = in_f16 ? launch_shape<kFp16, __half>(stream, args + i, m) : launch_shape<kFp16, float>(stream, args + i, m);
+        else
+            s = in_f16 ? launch_shape<kNf4, __half>(stream, args + i, m) : launch_shape<kNf4, float>(stream, args + i, m);
+        if (s != WRQ_OK) return s;
+        i += m;
+    }
+    return WRQ_OK;
 }
 
 } // namespace wrq

@@ -216,19 +216,18 @@ int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Sh
 int dispatch_group(hipStream_t stream, Quant quant, const Prepared *ops, int n) {
     int i = 0;
     while (i < n) {
-        if (ops[i].mfma) {
-            WRQ_TRY(launch_chunk(stream, quant, ops[i]));
-            i++;
-            continue;
-        }
+        // a run of ops of one kernel family, input type and token count
         MatmulArgs run[kMaxGroup];
         int m = 0;
-        while (i + m < n && m < kMaxGroup && !ops[i + m].mfma && ops[i + m].in_f16 == ops[i].in_f16 &&
+        while (i + m < n && m < kMaxGroup && ops[i + m].mfma == ops[i].mfma && ops[i + m].in_f16 == ops[i].in_f16 &&
                ops[i + m].a.T == ops[i].a.T && ops[i + m].a.quant == ops[i].a.quant) {
             run[m] = ops[i + m].a;
             m++;
         }
-        WRQ_TRY(launch_gemv_group(stream, quant, ops[i].in_f16, run, m));
+        if (ops[i].mfma && ops[i].a.K != 0)
+            WRQ_TRY(launch_gemm_group(stream, quant, ops[i].in_f16, run, m));
+        else
+            WRQ_TRY(launch_gemv_group(stream, quant, ops[i].in_f16, run, m));
         i += m;
     }
     return WRQ_OK;

@@ -33,6 +33,9 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
 int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &args);
 // Chunk-shaped products: f16 MFMA.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+// The same for `n` independent products of one quantisation and input type: those with one K
+// and token count share a launch (and then rarely need a split of K).
+int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
 // Resolves the split-K scratch array of the current device (also done lazily by the first
 // chunk product; calling it from wrq_init keeps the lookup out of stream capture).
 int prepare_gemm_scratch();
