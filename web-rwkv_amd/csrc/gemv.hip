@@ -323,17 +323,21 @@ __device__ __forceinline__ float row_sum(float v) {
 //     sum_j (u_j s + m) x_j = s * sum_j (1024 + u_j) x_j + (m - 1024 s) * sum_j x_j
 // -- one VALU op per weight.  f32 activations keep v_cvt_f32_ubyteN + FMA.
 // Lanes reduce inside DPP rows; rows and waves meet once in LDS.
-template <typename XT, int ROWS, int NT>
+// SINGLE: the launch holds one product; its descriptor sits at a fixed place in the kernel
+// arguments and is read in the first round of scalar loads.
+template <typename XT, int ROWS, int NT, bool SINGLE>
 __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g) {
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     __shared__ float red[ROWS][NROW16];
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
+    if constexpr (!SINGLE) {
 #pragma unroll
-    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-        if (task >= g.task_begin[i]) pi = i;
-    pi = __builtin_amdgcn_readfirstlane(pi);
+        for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+            if (task >= g.task_begin[i]) pi = i;
+        pi = __builtin_amdgcn_readfirstlane(pi);
+    }
     const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
     const uint32_t K = p.K, nchunk = K >> 4;
     const uint32_t row0 = (task - p.task_begin) * ROWS;
@@ -432,7 +436,7 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
 //                    byte costs one ds_read_b64 and two v_dot2_f32_f16 against the activation pair;
 //   f32 activations: as an f32 pair and two fmas.
 // The lookups, not HBM, bound this kernel: a CU sustains about 8 of them per clock.
-template <typename XT, int ROWS, int NT>
+template <typename XT, int ROWS, int NT, bool SINGLE>
 __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g) {
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     constexpr bool F16 = sizeof(XT) == 2;
@@ -441,10 +445,12 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
+    if constexpr (!SINGLE) {
 #pragma unroll
-    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-        if (task >= g.task_begin[i]) pi = i;
-    pi = __builtin_amdgcn_readfirstlane(pi);
+        for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
+            if (task >= g.task_begin[i]) pi = i;
+        pi = __builtin_amdgcn_readfirstlane(pi);
+    }
     const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
     const uint32_t K = p.K, nchunk = K >> 5;
     const uint32_t row0 = (task - p.task_begin) * ROWS;
@@ -722,34 +728,44 @@ int launch_group_xt(hipStream_t stream, const GemvGroup &g, int rows, int sl, in
     return launch_group_rt<QUANT, XT, 4, 1, 1>(stream, g, grid_x, grid_y, lds);
 }
 
-template <typename XT, int ROWS>
-int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+template <typename XT, int ROWS, bool SINGLE>
+int launch_oneshot_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
     if (nt >= 1024)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024>), grid, dim3(1024), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024, SINGLE>), grid, dim3(1024), 0, stream, g);
     else if (nt >= 512)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512>), grid, dim3(512), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512, SINGLE>), grid, dim3(512), 0, stream, g);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256, SINGLE>), grid, dim3(256), 0, stream, g);
     else if (nt >= 128)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128, SINGLE>), grid, dim3(128), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64>), grid, dim3(64), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64, SINGLE>), grid, dim3(64), 0, stream, g);
     return check_launch("matmul_vec_int8");
 }
 
 template <typename XT, int ROWS>
-int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+    return g.n == 1 ? launch_oneshot_nt_n<XT, ROWS, true>(stream, g, nt) : launch_oneshot_nt_n<XT, ROWS, false>(stream, g, nt);
+}
+
+template <typename XT, int ROWS, bool SINGLE>
+int launch_oneshot_nf4_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
     if (nt >= 512)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 512>), grid, dim3(512), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 512, SINGLE>), grid, dim3(512), 0, stream, g);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 256, SINGLE>), grid, dim3(256), 0, stream, g);
     else if (nt >= 128)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 128, SINGLE>), grid, dim3(128), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 64>), grid, dim3(64), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 64, SINGLE>), grid, dim3(64), 0, stream, g);
     return check_launch("matmul_vec_nf4");
+}
+
+template <typename XT, int ROWS>
+int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt) {
+    return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false>(stream, g, nt);
 }
 
 bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
