@@ -13,8 +13,11 @@ Weights are random-init f16 ~ N(0, 0.02) (att.output and ffn.value pre-multiplie
 2^-(layer / 6), src/runtime/loader.rs:734-762) packed on the GPU by the library itself;
 inputs are resident in HBM before the timed region.
 
-Prints one JSON line; see README/DESIGN for the fields.  `--sweep` prints the per-operator
-figures of configs 2 and 3 instead.
+Prints one JSON line: metric / value (tok/s of the path) / unit / n_gpus / steps / warmup /
+ms_per_step / dtype / config, `roofline` (algorithmic bytes per launch over the average launch
+duration against 8 TB/s, measured HBM traffic) and `cpu_baseline` (the CPU restatement on the
+host cores).  `--sweep` prints per-operator figures instead, `--schedule` a multi-slot serving
+schedule, `--tokens N` steps of N tokens, `--with-head` adds the f16 head.
 """
 import argparse
 import importlib
@@ -373,7 +376,7 @@ def main():
     ap.add_argument("--slots", type=int, default=32)
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported (the path shards by weight rows, see DESIGN.md)")
+        sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
 
     import torch
 
