@@ -13,6 +13,7 @@
 // on each other share launches.
 #pragma once
 
+#include <cmath>
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -494,6 +495,77 @@ inline std::vector<float> float4_quant() {
             1.0f};
 }
 
+// Float4Quant::new_student / quantile_student (src/tensor/matrix.rs:29-44): 16 quantiles of
+// Student's t with `nu` degrees of freedom at the probabilities delta + i (0.5 - delta) / 7
+// (i < 7) and 0.5 + i (0.5 - delta) / 8 (i < 9), delta = (1/32 + 1/30) / 2, divided by the
+// largest.  The reference takes the quantile from the `statrs` crate (0.18, not vendored);
+// here the t CDF is the regularised incomplete beta function (Lentz continued fraction) and
+// is inverted by bisection in double precision, which agrees with statrs far inside f32.
+namespace detail {
+inline double betacf(double a, double b, double x) {
+    const double tiny = 1e-300;
+    double qab = a + b, qap = a + 1.0, qam = a - 1.0, c = 1.0, d = 1.0 - qab * x / qap;
+    if (std::fabs(d) < tiny) d = tiny;
+    d = 1.0 / d;
+    double h = d;
+    for (int m = 1; m <= 400; m++) {
+        const int m2 = 2 * m;
+        double aa = m * (b - m) * x / ((qam + m2) * (a + m2));
+        d = 1.0 + aa * d;
+        if (std::fabs(d) < tiny) d = tiny;
+        c = 1.0 + aa / c;
+        if (std::fabs(c) < tiny) c = tiny;
+        d = 1.0 / d;
+        h *= d * c;
+        aa = -(a + m) * (qab + m) * x / ((a + m2) * (qap + m2));
+        d = 1.0 + aa * d;
+        if (std::fabs(d) < tiny) d = tiny;
+        c = 1.0 + aa / c;
+        if (std::fabs(c) < tiny) c = tiny;
+        d = 1.0 / d;
+        const double del = d * c;
+        h *= del;
+        if (std::fabs(del - 1.0) < 1e-16) break;
+    }
+    return h;
+}
+inline double betai(double a, double b, double x) { // regularised incomplete beta I_x(a, b)
+    if (x <= 0.0) return 0.0;
+    if (x >= 1.0) return 1.0;
+    const double bt = std::exp(std::lgamma(a + b) - std::lgamma(a) - std::lgamma(b) + a * std::log(x) + b * std::log(1.0 - x));
+    return x < (a + 1.0) / (a + b + 2.0) ? bt * betacf(a, b, x) / a : 1.0 - bt * betacf(b, a, 1.0 - x) / b;
+}
+inline double student_cdf(double t, double nu) {
+    const double tail = 0.5 * betai(0.5 * nu, 0.5, nu / (nu + t * t));
+    return t > 0 ? 1.0 - tail : tail;
+}
+inline double student_quantile(double p, double nu) {
+    if (p == 0.5) return 0.0; // the median, exactly (table entry 7)
+    double lo = -1e6, hi = 1e6;
+    for (int i = 0; i < 200; i++) {
+        const double mid = 0.5 * (lo + hi);
+        (student_cdf(mid, nu) < p ? lo : hi) = mid;
+    }
+    return 0.5 * (lo + hi);
+}
+} // namespace detail
+
+inline std::vector<float> float4_quant_student(double nu) {
+    const double delta = (1.0 / 32.0 + 1.0 / 30.0) / 2.0;
+    std::vector<double> p;
+    for (int i = 0; i < 7; i++) p.push_back(delta + (0.5 - delta) / 7.0 * i);
+    for (int i = 0; i < 9; i++) p.push_back(0.5 + (1.0 - delta - 0.5) / 8.0 * i);
+    std::vector<double> q;
+    double most = -1e300;
+    for (double v : p) {
+        q.push_back(detail::student_quantile(v, nu));
+        most = std::max(most, q.back());
+    }
+    std::vector<float> out;
+    for (double v : q) out.push_back((float)(v / most));
+    return out;
+}
+
 // Matrix { Fp16(w), Int8 { w, m }, Fp4 { q, w, m } } (src/tensor/matrix.rs:29-44, :80-94).
 struct Matrix {
     enum class Kind { Int8, Fp4, Fp16 } kind;
@@ -523,6 +595,11 @@ struct Matrix {
         auto m = TensorGpu<f16>::init(absmax_shape);
         queue.submit(TensorOp::quantize_mat_nf4(matrix, q, m, w));
         return Matrix{Kind::Fp4, w, m, q, {}};
+    }
+
+    // src/tensor/matrix.rs:202-222
+    static Matrix quant_sf4(const TensorGpu<f16> &matrix, Queue &queue, double nu) {
+        return quant_nf4(matrix, queue, float4_quant_student(nu));
     }
 
     template <typename F0, typename F1>

@@ -118,6 +118,12 @@ static void test_build_time_errors() {
     EXPECT(ok.kind() == TensorOp::Kind::Atom);
     EXPECT(TensorOp::INT8_BLOCK_SIZE == 128 && TensorOp::NF4_BLOCK_SIZE == 64);
     EXPECT(float4_quant().size() == 16 && float4_quant()[7] == 0.0f);
+    {   // SF4 table (src/tensor/matrix.rs:29-44): nu = 5, values from scipy.stats.t.ppf
+        const auto sf4 = float4_quant_student(5.0);
+        EXPECT(sf4.size() == 16 && sf4[0] == -1.0f && sf4[7] == 0.0f && sf4[15] == 1.0f);
+        EXPECT(std::fabs(sf4[1] - -0.62778056f) < 2e-7 && std::fabs(sf4[2] - -0.454736f) < 2e-7);
+        for (int i = 1; i < 16; i++) EXPECT(sf4[i] > sf4[i - 1]);
+    }
 }
 
 // ------------------------------------------------------------------ GPU

@@ -122,3 +122,24 @@ def test_missing_library_fails_loudly(wrq, monkeypatch, tmp_path):
     monkeypatch.setattr(wrq, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(FileNotFoundError, match="no CPU or eager fallback"):
         wrq.lib()
+
+
+def test_sf4_table_matches_student_quantiles():
+    # Float4Quant::new_student (src/tensor/matrix.rs:29-44).  The reference takes the quantile from
+    # the statrs crate, which is not available here: the table is checked against scipy's
+    # Student-t quantile instead (equal far inside f32) -- bit parity with statrs is unpinned.
+    import importlib
+
+    import numpy as np
+    from scipy import stats
+
+    wrq = importlib.import_module("web-rwkv_amd")
+    delta = (1 / 32 + 1 / 30) / 2
+    probs = [delta + (0.5 - delta) / 7 * i for i in range(7)] + [0.5 + (0.5 - delta) / 8 * i for i in range(9)]
+    for nu in (1.0, 2.5, 5.0, 30.0):
+        q = np.array(wrq.quantile_student(nu), dtype=np.float32)
+        ref = stats.t.ppf(probs, nu)
+        ref = (ref / ref.max()).astype(np.float32)
+        assert q.shape == (16,) and q[0] == -1.0 and q[7] == 0.0 and q[15] == 1.0
+        assert (np.diff(q) > 0).all()
+        assert np.abs(q.astype(np.float64) - ref.astype(np.float64)).max() <= 1.2e-7

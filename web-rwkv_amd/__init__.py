@@ -45,6 +45,73 @@ EXPORTS = [
 MAX_GROUP = 8
 
 
+def quantile_student(nu):
+    """Float4Quant::new_student (src/tensor/matrix.rs:29-44): the 16-entry SF4 table.
+
+    Quantiles of Student's t at delta + i (0.5 - delta) / 7 (i < 7) and 0.5 + i (0.5 - delta) / 8
+    (i < 9), delta = (1/32 + 1/30) / 2, divided by the largest.  The reference uses the `statrs`
+    crate's inverse CDF; here the CDF (regularised incomplete beta, continued fraction) is
+    inverted by bisection in double precision.
+    """
+    import math
+
+    def betacf(a, b, x):
+        tiny = 1e-300
+        qab, qap, qam = a + b, a + 1.0, a - 1.0
+        c, d = 1.0, 1.0 - qab * x / qap
+        d = 1.0 / (d if abs(d) > tiny else tiny)
+        h = d
+        for m in range(1, 401):
+            m2 = 2 * m
+            aa = m * (b - m) * x / ((qam + m2) * (a + m2))
+            d = 1.0 + aa * d
+            d = 1.0 / (d if abs(d) > tiny else tiny)
+            c = 1.0 + aa / c
+            c = c if abs(c) > tiny else tiny
+            h *= d * c
+            aa = -(a + m) * (qab + m) * x / ((a + m2) * (qap + m2))
+            d = 1.0 + aa * d
+            d = 1.0 / (d if abs(d) > tiny else tiny)
+            c = 1.0 + aa / c
+            c = c if abs(c) > tiny else tiny
+            h *= d * c
+            if abs(d * c - 1.0) < 1e-16:
+                break
+        return h
+
+    def betai(a, b, x):
+        if x <= 0.0:
+            return 0.0
+        if x >= 1.0:
+            return 1.0
+        bt = math.exp(math.lgamma(a + b) - math.lgamma(a) - math.lgamma(b) + a * math.log(x) + b * math.log(1.0 - x))
+        return bt * betacf(a, b, x) / a if x < (a + 1.0) / (a + b + 2.0) else 1.0 - bt * betacf(b, a, 1.0 - x) / b
+
+    def cdf(t):
+        tail = 0.5 * betai(0.5 * nu, 0.5, nu / (nu + t * t))
+        return 1.0 - tail if t > 0 else tail
+
+    def quantile(p):
+        if p == 0.5:
+            return 0.0  # the median, exactly (table entry 7)
+        lo, hi = -1e6, 1e6
+        for _ in range(200):
+            mid = 0.5 * (lo + hi)
+            if cdf(mid) < p:
+                lo = mid
+            else:
+                hi = mid
+        return 0.5 * (lo + hi)
+
+    delta = (1.0 / 32.0 + 1.0 / 30.0) / 2.0
+    probs = [delta + (0.5 - delta) / 7.0 * i for i in range(7)] + [0.5 + (1.0 - delta - 0.5) / 8.0 * i for i in range(9)]
+    q = [quantile(p) for p in probs]
+    most = max(q)
+    import numpy as np
+
+    return [float(np.float32(v / most)) for v in q]
+
+
 class TensorError(RuntimeError):
     """A failed op constructor; ``status`` is the wrq_status code."""
 
@@ -270,6 +337,11 @@ class Matrix:
     def fp16(matrix):
         """Matrix::Fp16: the f16 tensor as it is."""
         return Matrix("Fp16", matrix, None)
+
+    @staticmethod
+    def quant_sf4(matrix, nu):
+        """Matrix::quant_sf4, src/tensor/matrix.rs:202-222."""
+        return Matrix.quant_nf4(matrix, quantile_student(nu))
 
     def matmul_vec_op(self, input, output, act=ACT_NONE, sparse=False, **views):
         if self.kind == "Fp16":
