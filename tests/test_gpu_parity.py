@@ -515,3 +515,58 @@ def test_fp16_matrix_products(gpu, oracle, K, R, T):
         got32 = run(gpu, m, xf, R, "vec", np.float32, act=1)
         want = np.square(np.maximum(xf.astype(np.float64) @ w.astype(np.float64).T, 0.0))
         assert_close(got32, want, EPS, "f32 activations, squared relu")
+
+
+def test_entry_points_from_several_threads(gpu, oracle):
+    # ops are built on worker threads in the reference (src/runtime/mod.rs:138-166): the entry
+    # points keep no shared mutable state (errors are per thread); every thread drives its own
+    # stream and its own decode products here
+    import threading
+
+    import torch
+
+    announce("threads")
+    K, R = 2048, 512
+    rng = np.random.default_rng(SEED + 31)
+    cases = []
+    for j in range(4):
+        kind = "int8" if j % 2 == 0 else "nf4"
+        w = gen_f16(rng, (R, K), 0.02)
+        x = gen_f16(rng, (1, K), 1.0)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        cases.append((gpu_matrix(gpu, kind, wp, scale), dev(x), truth_matmul(wdeq, x)))
+    torch.cuda.synchronize()
+    results, errors = [None] * 4, []
+
+    def work(j):
+        try:
+            m, xd, _ = cases[j]
+            stream = torch.cuda.Stream()
+            outs = []
+            with torch.cuda.stream(stream):
+                for _ in range(50):
+                    out = torch.empty((1, R), dtype=torch.float32, device="cuda")
+                    m.matmul_vec_op(xd, out)
+                    outs.append(out)
+                # a failing call on this thread reports this thread's message
+                bad = torch.empty((1, R + 4), dtype=torch.float32, device="cuda")
+                try:
+                    m.matmul_vec_op(xd, bad)
+                    errors.append((j, "shape error not raised"))
+                except gpu.TensorError as e:
+                    if e.status != gpu.ERR_SHAPE or str(R + 4) not in str(e):
+                        errors.append((j, str(e)))
+            stream.synchronize()
+            results[j] = [o.cpu().numpy() for o in outs]
+        except Exception as e:  # noqa: BLE001
+            errors.append((j, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for j in range(4):
+        for o in results[j]:
+            assert_close(o, cases[j][2], EPS, f"thread {j}")
