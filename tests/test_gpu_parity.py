@@ -115,6 +115,76 @@ def test_quant_every_f16_value(gpu, oracle):
         assert np.array_equal(host(m4.w), w4) and np.array_equal(host(m4.m).view(np.uint16), s4.view(np.uint16))
 
 
+def test_quant_int8_hard_divisions(gpu, oracle):
+    """Blocks whose range max - min is the f32 just below a power of two (all-ones mantissa): the
+    reciprocal of such a divisor sits next to a rounding boundary, the hard case of any division
+    built from a reciprocal.  Dividends: powers of two, their neighbours and random values."""
+    announce("quant_int8 hard divisions")
+    rng = np.random.default_rng(SEED + 50)
+    rows = []
+    for k in range(0, 16):
+        mx, mn = np.float16(2.0 ** k), np.float16(2.0 ** (k - 24))
+        assert np.float32(mx) - np.float32(mn) == np.nextafter(np.float32(mx), np.float32(0))
+        for _ in range(4):
+            blk = (rng.random(128) * float(mx)).astype(np.float16)
+            p2 = np.float16(2.0) ** rng.integers(k - 24, k, 48)
+            blk[:48] = p2.astype(np.float16)
+            blk[48:64] = np.nextafter(p2[:16].astype(np.float16), np.float16(0))
+            blk[64:80] = np.nextafter(p2[16:32].astype(np.float16), np.float16(65504))
+            blk = np.clip(blk, mn, mx)
+            blk[rng.integers(0, 128)] = mx
+            blk[(np.argmax(blk == mx) + 1) % 128] = mn
+            rows.append(blk if rng.random() < 0.5 else -blk)
+    w = np.stack(rows).astype(np.float16)
+    m = gpu.Matrix.quant_u8(dev(w))
+    want_w, want_m, _ = oracle.quant_int8(w)
+    assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+    got = host(m.w)
+    assert np.array_equal(got, want_w), f"{(got != want_w).sum()} bytes differ"
+
+
+@pytest.mark.parametrize("table", ["eighths", "sf4", "reversed", "shuffled", "duplicates", "narrow", "close_pair"])
+def test_quant_nf4_tables(gpu, oracle, table):
+    """Tables on both sides of the packer's choice between threshold search and literal scan.
+    `eighths` puts every decision threshold on an f16 value, and blocks holding 1.0 present those
+    values unscaled: exact ties, which the scan gives to the later entry."""
+    announce("quant_nf4 table", table)
+    rng = np.random.default_rng(SEED + 60)
+    q = {
+        "eighths": np.arange(-8, 8) / 8.0,
+        "sf4": np.array(gpu.quantile_student(5.0)),
+        "reversed": NF4_QUANT[::-1],
+        "shuffled": rng.permutation(NF4_QUANT),
+        "duplicates": np.repeat(NF4_QUANT[::2], 2),
+        "narrow": NF4_QUANT * 0.2 - 0.7,  # all entries in [-0.9, -0.5]: x above 0.5 is further than the scan's initial bound
+        "close_pair": np.concatenate([NF4_QUANT[:8], [NF4_QUANT[8] * 0 + 1e-7], NF4_QUANT[9:]]),
+    }[table].astype(np.float32)
+    w = gen_f16(rng, (256, 1024), 0.02)
+    w[:64] = (rng.integers(-16, 17, (64, 1024)) / 16.0).astype(np.float16)  # thresholds of `eighths` and entries
+    w[:64, ::64] = 1.0
+    w[64:96] = (rng.random((32, 1024)) * 2 - 1).astype(np.float16)
+    w[96:128] = gen_f16(rng, (32, 1024), 30.0)
+    m = gpu.Matrix.quant_nf4(dev(w), q.tolist())
+    want_w, want_m = oracle.quant_nf4(w, q)
+    assert np.array_equal(host(m.m).view(np.uint16), want_m.view(np.uint16))
+    got = host(m.w)
+    assert np.array_equal(got, want_w), f"{(got != want_w).sum()} bytes differ"
+
+
+def test_quant_full_size_random_scales(gpu, oracle):
+    """A 4096 x 4096 matrix whose blocks span many magnitudes: x = v / absmax then takes f32 values
+    all over [-1, 1], next to the nf4 decision thresholds included."""
+    announce("quant 4096x4096 mixed scales")
+    rng = np.random.default_rng(SEED + 70)
+    scale = np.exp2(rng.integers(-20, 12, (4096, 64))).repeat(64, axis=1)
+    w = (rng.standard_normal((4096, 4096)) * scale).astype(np.float16)
+    m8, m4 = gpu.Matrix.quant_u8(dev(w)), gpu.Matrix.quant_nf4(dev(w))
+    w8, s8, _ = oracle.quant_int8(w)
+    w4, s4 = oracle.quant_nf4(w)
+    assert np.array_equal(host(m8.w), w8) and np.array_equal(host(m8.m).view(np.uint16), s8.view(np.uint16))
+    assert np.array_equal(host(m4.w), w4) and np.array_equal(host(m4.m).view(np.uint16), s4.view(np.uint16))
+
+
 # --------------------------------------------------------------- products
 
 
