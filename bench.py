@@ -204,6 +204,36 @@ def run_probe(torch):
     return {"bytes": n, "copy_GBps": round(2 * n / ms_copy / 1e6, 1), "read_GBps": round(n / ms_read / 1e6, 1)}
 
 
+def sweep_pack(wrq, torch, quant, w):
+    """Packing one f16 matrix (quant_mat_int8 / quant_mat_nf4): microseconds and HBM bytes per
+    second, 2 B read + 1 or 0.5 B written per element plus the scale blocks; inputs rotate so
+    that none is still cached."""
+    R, K = w.shape
+    nin = min(16, max(2, int(1.0e9 // (w.numel() * 2)) + 1))
+    ins = [w] + [w.clone() for _ in range(nin - 1)]
+    if quant == "int8":
+        out = torch.empty((R, K), dtype=torch.uint8, device="cuda")
+        scale = torch.empty(2 * R * K // wrq.INT8_BLOCK_SIZE, dtype=torch.float16, device="cuda")
+        calls = [lambda x=x: wrq.TensorOp.quantize_mat_int8(x, scale, out) for x in ins]
+    else:
+        out = torch.empty((R, K // 2), dtype=torch.uint8, device="cuda")
+        scale = torch.empty(R * K // wrq.NF4_BLOCK_SIZE, dtype=torch.float16, device="cuda")
+        table = torch.tensor(wrq.NF4_QUANT, dtype=torch.float32, device="cuda")
+        calls = [lambda x=x: wrq.TensorOp.quantize_mat_nf4(x, table, scale, out) for x in ins]
+    reps = max(nin, 24)
+    calls[0]()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(reps):
+            calls[i % nin]()
+    ms, _ = time_steps(torch, graph.replay, 5, 2)
+    us = ms * 1e3 / reps
+    nbytes = w.numel() * 2 + out.numel() + scale.numel() * 2
+    return {"op": "pack", "quant": quant, "K": K, "R": R, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+            "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3), "copies": nin}
+
+
 def sweep(wrq, torch, args):
     """Per-operator figures of configs 2 and 3: cold (rotating weight copies) GB/s per shape."""
     rows = []
@@ -212,6 +242,9 @@ def sweep(wrq, torch, args):
     for quant in ("int8", "nf4", "fp16"):
         for K, R in (shapes if quant != "fp16" else [(2048, 65536), (4096, 65536), (4096, 4096)]):
             w = (torch.randn((R, K), generator=g, device="cuda") * 0.02).half()
+            if quant != "fp16":
+                rows.append(sweep_pack(wrq, torch, quant, w))
+                print(json.dumps(rows[-1]), flush=True)
             m0 = wrq.Matrix.quant_u8(w) if quant == "int8" else wrq.Matrix.quant_nf4(w) if quant == "nf4" else wrq.Matrix.fp16(w)
             del w
             wbytes = m0.w.numel() * m0.w.element_size()

@@ -441,7 +441,26 @@ def test_full_size_properties(gpu, oracle, kind):
     assert_close(host(om), host(ov), 2e-4, "mat vs vec")
 
 
-@pytest.mark.parametrize("T", [1, 5, 32])
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("T", [2, 3, 4])
+@pytest.mark.parametrize("K,R", [(14336, 516), (4096, 2060), (2048, 16388)], ids=str)
+def test_short_runs_on_decode_kernels(gpu, oracle, kind, K, R, T):
+    # 2 - 4 tokens share one pass of the decode kernels: long rows (two chunks per lane), row
+    # counts that leave a partial task, enough rows for 8 per task, f16 output with an activation
+    announce("short run", kind, K, R, T)
+    rng = np.random.default_rng(SEED + 29 + T + K)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (T, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    got = run(gpu, m, x, R, "vec", np.float16, act=gpu.ACT_SILU)
+    assert got.shape == (T, R)
+    assert_close(got, truth_matmul(wdeq, x, "silu"), EPS, "vs float64")
+    one = np.concatenate([run(gpu, m, x[t:t + 1], R, "vec", np.float16, act=gpu.ACT_SILU) for t in range(T)])
+    assert_close(got, one, 1e-3, "vs one call per token")  # same arithmetic up to the last f16 ulp
+
+
+@pytest.mark.parametrize("T", [1, 2, 4, 5, 32])
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
 def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind, T):
     # the independent products of a layer in shared launches: same results as one call each;

@@ -312,6 +312,33 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
+// End of a one-shot task: lanes reduce inside DPP rows, the NT / 16 row partials of every
+// (output row, token) meet in LDS and 16 lanes sum them, again with DPP.
+template <int ROWS, int NT, int TT>
+__device__ __forceinline__ void oneshot_reduce_store(float (&acc)[ROWS][TT], float (&red)[ROWS * TT][NT / 16], const GemvProblem &p,
+                                                     uint32_t row0, uint32_t T) {
+    constexpr int NROW16 = NT / 16;
+    const uint32_t tid = threadIdx.x;
+#pragma unroll
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float s = row_sum(acc[r][t]);
+            if ((tid & 15) == 0) red[r * TT + t][tid >> 4] = s;
+        }
+    __syncthreads();
+    const uint32_t l = tid & 15;
+    for (uint32_t o = tid >> 4; o < (uint32_t)(ROWS * TT); o += NROW16) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NROW16 / 16; i++) s += red[o][l + 16 * i];
+        if (NROW16 < 16) s = l < NROW16 ? red[o][l] : 0.0f;
+        s = row_sum(s);
+        const uint32_t row = row0 + o / TT, t = o % TT;
+        if (l == 0 && row < p.R && t < T) store_out(p.out, p.out_f16, (uint64_t)t * p.out_token_stride + row, act_apply(p.act, s));
+    }
+}
+
 // int8, one token: one workgroup per task, everything it needs requested at once.  At the
 // 7B shapes the whole matrix is a fraction of what the CUs can keep in flight, so a task
 // (ROWS rows, NT lanes along K) issues all its loads -- activations first, they are needed
@@ -325,10 +352,14 @@ __device__ __forceinline__ float row_sum(float v) {
 // Lanes reduce inside DPP rows; rows and waves meet once in LDS.
 // SINGLE: the launch holds one product; its descriptor sits at a fixed place in the kernel
 // arguments and is read in the first round of scalar loads.
-template <typename XT, int ROWS, int NT, bool SINGLE>
+// TT > 1 (f16 activations only): the same pass serves up to TT tokens of a short run -- the
+// converted codes of a row meet the activations of every token, (TT + 1) / 2 VALU ops per weight.
+template <typename XT, int ROWS, int NT, bool SINGLE, int TT>
 __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g) {
+    static_assert(TT == 1 || sizeof(XT) == 2, "several tokens per pass: f16 activations only");
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
-    __shared__ float red[ROWS][NROW16];
+    constexpr int XW = sizeof(XT) == 2 ? 2 : 4; // 16-byte loads per token and chunk
+    __shared__ float red[ROWS * TT][NROW16];
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
@@ -347,15 +378,21 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     const uint32_t *mm = reinterpret_cast<const uint32_t *>(p.scale);
     const XT *x = reinterpret_cast<const XT *>(p.x);
 
-    float acc[ROWS];
+    float acc[ROWS][TT];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
 
     for (uint32_t c = tid; c < nchunk; c += NT) {
-        uint4 xv[sizeof(XT) == 2 ? 2 : 4];
+        uint4 xv[TT][XW];
 #pragma unroll
-        for (int i = 0; i < (sizeof(XT) == 2 ? 2 : 4); i++)
-            xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)c << 4)) + 16 * i);
+        for (int t = 0; t < TT; t++) {
+            const uint32_t tok = TT == 1 ? 0u : min((uint32_t)t, g.T - 1); // tokens past the run repeat the last one
+#pragma unroll
+            for (int i = 0; i < XW; i++)
+                xv[t][i] = load128(reinterpret_cast<const uint8_t *>(x + (uint64_t)tok * p.x_token_stride + ((uint64_t)c << 4)) + 16 * i);
+        }
         uint4 wv[ROWS];
         uint32_t sc[ROWS];
 #pragma unroll
@@ -366,32 +403,44 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
             sc[r] = mm[(e0 + off) >> 7];
         }
         if constexpr (sizeof(XT) == 2) {
-            const uint32_t xd[8] = {xv[0].x, xv[0].y, xv[0].z, xv[0].w, xv[1].x, xv[1].y, xv[1].z, xv[1].w};
-            float sx = 0.0f;
+            float sx[TT];
 #pragma unroll
-            for (int j = 0; j < 8; j++) sx = dot2(xd[j], 0x3c003c00u, sx); // (1.0, 1.0)
+            for (int t = 0; t < TT; t++) {
+                const uint32_t xd[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
+                sx[t] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; j++) sx[t] = dot2(xd[j], 0x3c003c00u, sx[t]); // (1.0, 1.0)
+            }
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float pr = 0.0f;
+                uint32_t code[8]; // f16 pairs (1024 + u0, 1024 + u1)
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
-                    pr = dot2(__builtin_amdgcn_perm(0x64646464u, w[d], 0x04010400u), xd[2 * d], pr);
-                    pr = dot2(__builtin_amdgcn_perm(0x64646464u, w[d], 0x04030402u), xd[2 * d + 1], pr);
+                    code[2 * d] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04010400u);
+                    code[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04030402u);
                 }
                 const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
                 const float mx = h2f((uint16_t)(sc[r] >> 16));
                 const float s = (mx - mn) * (1.0f / 255.0f);
-                acc[r] = fmaf(s, pr, fmaf(fmaf(-1024.0f, s, mn), sx, acc[r]));
+                const float c0 = fmaf(-1024.0f, s, mn);
+#pragma unroll
+                for (int t = 0; t < TT; t++) {
+                    const uint32_t xd[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
+                    float pr = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) pr = dot2(code[j], xd[j], pr);
+                    acc[r][t] = fmaf(s, pr, fmaf(c0, sx[t], acc[r][t]));
+                }
             }
         } else {
             float xf[16];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                xf[4 * i] = __uint_as_float(xv[i].x);
-                xf[4 * i + 1] = __uint_as_float(xv[i].y);
-                xf[4 * i + 2] = __uint_as_float(xv[i].z);
-                xf[4 * i + 3] = __uint_as_float(xv[i].w);
+                xf[4 * i] = __uint_as_float(xv[0][i].x);
+                xf[4 * i + 1] = __uint_as_float(xv[0][i].y);
+                xf[4 * i + 2] = __uint_as_float(xv[0][i].z);
+                xf[4 * i + 3] = __uint_as_float(xv[0][i].w);
             }
             float sx = 0.0f;
 #pragma unroll
@@ -405,27 +454,11 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
                 const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
                 const float mx = h2f((uint16_t)(sc[r] >> 16));
                 const float s = (mx - mn) * (1.0f / 255.0f);
-                acc[r] = fmaf(s, pr, fmaf(mn, sx, acc[r]));
+                acc[r][0] = fmaf(s, pr, fmaf(mn, sx, acc[r][0]));
             }
         }
     }
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        const float s = row_sum(acc[r]);
-        if ((tid & 15) == 0) red[r][tid >> 4] = s;
-    }
-    __syncthreads();
-    // NROW16 partials per output row: 16 lanes per row sum them, again with DPP
-    if (tid < ROWS * 16) {
-        const uint32_t r = tid >> 4, l = tid & 15;
-        float s = 0.0f;
-#pragma unroll
-        for (int i = 0; i < NROW16 / 16; i++) s += red[r][l + 16 * i];
-        if (NROW16 < 16) s = l < NROW16 ? red[r][l] : 0.0f;
-        s = row_sum(s);
-        const uint32_t row = row0 + r;
-        if (l == 0 && row < p.R) store_out(p.out, p.out_f16, row, act_apply(p.act, s));
-    }
+    oneshot_reduce_store<ROWS, NT, TT>(acc, red, p, row0, g.T);
 }
 
 // nf4, one token: the same one-shot shape (one workgroup per task of ROWS rows, NT lanes along
@@ -436,11 +469,13 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
 //                    byte costs one ds_read_b64 and two v_dot2_f32_f16 against the activation pair;
 //   f32 activations: as an f32 pair and two fmas.
 // The lookups, not HBM, bound this kernel: a CU sustains about 8 of them per clock.
-template <typename XT, int ROWS, int NT, bool SINGLE>
+// TT > 1 (f16 activations only): up to TT tokens of a short run share the pass and its lookups.
+template <typename XT, int ROWS, int NT, bool SINGLE, int TT>
 __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g) {
+    static_assert(TT == 1 || sizeof(XT) == 2, "several tokens per pass: f16 activations only");
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     constexpr bool F16 = sizeof(XT) == 2;
-    __shared__ float red[ROWS][NROW16];
+    __shared__ float red[ROWS * TT][NROW16];
     __shared__ uint2 tab[256];
     const uint32_t tid = threadIdx.x;
     const uint32_t task = blockIdx.x;
@@ -459,18 +494,25 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
     const uint8_t *wbase = p.w + (((uint64_t)row0 * K) >> 1);
     const XT *x = reinterpret_cast<const XT *>(p.x);
 
-    float acc[ROWS];
+    float acc[ROWS][TT];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
 
     bool table_ready = false;
     for (uint32_t c = tid; c < nchunk || !table_ready; c += NT) {
         const bool live = c < nchunk;
         const uint32_t cc = live ? c : 0; // idle lanes of the first pass repeat chunk 0 and drop it
         constexpr int NX = F16 ? 4 : 8;
-        uint4 xv[NX];
+        uint4 xv[TT][NX];
 #pragma unroll
-        for (int i = 0; i < NX; i++) xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)cc << 5)) + 16 * i);
+        for (int t = 0; t < TT; t++) {
+            const uint32_t tok = TT == 1 ? 0u : min((uint32_t)t, g.T - 1); // tokens past the run repeat the last one
+#pragma unroll
+            for (int i = 0; i < NX; i++)
+                xv[t][i] = load128(reinterpret_cast<const uint8_t *>(x + (uint64_t)tok * p.x_token_stride + ((uint64_t)cc << 5)) + 16 * i);
+        }
         uint4 wv[ROWS];
         uint16_t sc[ROWS];
 #pragma unroll
@@ -497,28 +539,35 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
         }
         if (!live) continue;
         if constexpr (F16) {
-            const uint32_t xd[16] = {xv[0].x, xv[0].y, xv[0].z, xv[0].w, xv[1].x, xv[1].y, xv[1].z, xv[1].w,
-                                     xv[2].x, xv[2].y, xv[2].z, xv[2].w, xv[3].x, xv[3].y, xv[3].z, xv[3].w};
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float ph = 0.0f, pl = 0.0f;
+                float ph[TT], pl[TT];
+#pragma unroll
+                for (int t = 0; t < TT; t++) ph[t] = pl[t] = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 16; j++) {
                     const uint2 e = tab[(w[j >> 2] >> (8 * (j & 3))) & 0xffu];
-                    ph = dot2(e.x, xd[j], ph);
-                    pl = dot2(e.y, xd[j], pl);
+#pragma unroll
+                    for (int t = 0; t < TT; t++) {
+                        const uint4 &xq = xv[t][j >> 2];
+                        const uint32_t xd = (j & 3) == 0 ? xq.x : (j & 3) == 1 ? xq.y : (j & 3) == 2 ? xq.z : xq.w;
+                        ph[t] = dot2(e.x, xd, ph[t]);
+                        pl[t] = dot2(e.y, xd, pl[t]);
+                    }
                 }
-                acc[r] = fmaf(h2f(sc[r]), fmaf(pl, 1.0f / 2048.0f, ph), acc[r]);
+                const float am = h2f(sc[r]);
+#pragma unroll
+                for (int t = 0; t < TT; t++) acc[r][t] = fmaf(am, fmaf(pl[t], 1.0f / 2048.0f, ph[t]), acc[r][t]);
             }
         } else {
             float xf[32];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                xf[4 * i] = __uint_as_float(xv[i].x);
-                xf[4 * i + 1] = __uint_as_float(xv[i].y);
-                xf[4 * i + 2] = __uint_as_float(xv[i].z);
-                xf[4 * i + 3] = __uint_as_float(xv[i].w);
+                xf[4 * i] = __uint_as_float(xv[0][i].x);
+                xf[4 * i + 1] = __uint_as_float(xv[0][i].y);
+                xf[4 * i + 2] = __uint_as_float(xv[0][i].z);
+                xf[4 * i + 3] = __uint_as_float(xv[0][i].w);
             }
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
@@ -530,27 +579,11 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
                     pr = fmaf(__uint_as_float(e.x), xf[2 * j], pr);
                     pr = fmaf(__uint_as_float(e.y), xf[2 * j + 1], pr);
                 }
-                acc[r] = fmaf(h2f(sc[r]), pr, acc[r]);
+                acc[r][0] = fmaf(h2f(sc[r]), pr, acc[r][0]);
             }
         }
     }
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        const float s = row_sum(acc[r]);
-        if ((tid & 15) == 0) red[r][tid >> 4] = s;
-    }
-    __syncthreads();
-    // NROW16 partials per output row: 16 lanes per row sum them, again with DPP
-    if (tid < ROWS * 16) {
-        const uint32_t r = tid >> 4, l = tid & 15;
-        float s = 0.0f;
-#pragma unroll
-        for (int i = 0; i < NROW16 / 16; i++) s += red[r][l + 16 * i];
-        if (NROW16 < 16) s = l < NROW16 ? red[r][l] : 0.0f;
-        s = row_sum(s);
-        const uint32_t row = row0 + r;
-        if (l == 0 && row < p.R) store_out(p.out, p.out_f16, row, act_apply(p.act, s));
-    }
+    oneshot_reduce_store<ROWS, NT, TT>(acc, red, p, row0, g.T);
 }
 
 // f16 weights, one token (matmul_vec_fp16, src/shaders/matmul_vec_fp16.wgsl:57-120): the same
@@ -728,44 +761,55 @@ int launch_group_xt(hipStream_t stream, const GemvGroup &g, int rows, int sl, in
     return launch_group_rt<QUANT, XT, 4, 1, 1>(stream, g, grid_x, grid_y, lds);
 }
 
-template <typename XT, int ROWS, bool SINGLE>
+template <typename XT, int ROWS, bool SINGLE, int TT>
 int launch_oneshot_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
-    if (nt >= 1024)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024, SINGLE>), grid, dim3(1024), 0, stream, g);
+    if (nt >= 1024 && TT == 1)
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024, SINGLE, 1>), grid, dim3(1024), 0, stream, g);
     else if (nt >= 512)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512, SINGLE>), grid, dim3(512), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512, SINGLE, TT>), grid, dim3(512), 0, stream, g);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256, SINGLE>), grid, dim3(256), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256, SINGLE, TT>), grid, dim3(256), 0, stream, g);
     else if (nt >= 128)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128, SINGLE>), grid, dim3(128), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128, SINGLE, TT>), grid, dim3(128), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64, SINGLE>), grid, dim3(64), 0, stream, g);
+        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64, SINGLE, TT>), grid, dim3(64), 0, stream, g);
     return check_launch("matmul_vec_int8");
 }
 
+// tt tokens per pass: 1, or 2 / 4 for short runs of f16 activations.  (8 tokens per pass were
+// measured slower than the matrix-core kernel: every task re-reads the activations of all tokens
+// from L2, four times the weight bytes at 4 rows per task.)
 template <typename XT, int ROWS>
-int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt) {
-    return g.n == 1 ? launch_oneshot_nt_n<XT, ROWS, true>(stream, g, nt) : launch_oneshot_nt_n<XT, ROWS, false>(stream, g, nt);
+int launch_oneshot_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt) {
+    if constexpr (sizeof(XT) == 2) {
+        if (tt == 4) return launch_oneshot_nt_n<XT, ROWS, false, 4>(stream, g, nt);
+        if (tt == 2) return launch_oneshot_nt_n<XT, ROWS, false, 2>(stream, g, nt);
+    }
+    return g.n == 1 ? launch_oneshot_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
 
-template <typename XT, int ROWS, bool SINGLE>
+template <typename XT, int ROWS, bool SINGLE, int TT>
 int launch_oneshot_nf4_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
     if (nt >= 512)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 512, SINGLE>), grid, dim3(512), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 512, SINGLE, TT>), grid, dim3(512), 0, stream, g);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 256, SINGLE>), grid, dim3(256), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 256, SINGLE, TT>), grid, dim3(256), 0, stream, g);
     else if (nt >= 128)
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 128, SINGLE>), grid, dim3(128), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 128, SINGLE, TT>), grid, dim3(128), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 64, SINGLE>), grid, dim3(64), 0, stream, g);
+        hipLaunchKernelGGL((gemv_nf4_oneshot_kernel<XT, ROWS, 64, SINGLE, TT>), grid, dim3(64), 0, stream, g);
     return check_launch("matmul_vec_nf4");
 }
 
 template <typename XT, int ROWS>
-int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt) {
-    return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false>(stream, g, nt);
+int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt) {
+    if constexpr (sizeof(XT) == 2) {
+        if (tt == 4) return launch_oneshot_nf4_nt_n<XT, 4, false, 4>(stream, g, nt);
+        if (tt == 2) return launch_oneshot_nf4_nt_n<XT, ROWS, false, 2>(stream, g, nt);
+    }
+    return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
 
 bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
@@ -813,13 +857,14 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         g.T = T;
         size_t lds = lds_base;
         uint32_t tasks = 0;
-        uint64_t bytes = 0;
         // rows per task: 4, or 2 when the group is too small to give every wave of 256 CUs a task
         uint64_t rows_total = 0;
         for (int j = i; j < n; j++) rows_total += (uint64_t)args[j].R * args[j].B;
         // int8 at one token: the one-shot kernel (4 rows per workgroup; 8 once that still gives
         // every CU eight workgroups)
-        const bool oneshot = T == 1 && env_int("WRQ_GEMV_ONESHOT", 1);
+        // up to 8 tokens of f16 activations: the same kernel, several tokens per pass
+        const bool oneshot = (T == 1 || (in_f16 && T <= 4)) && env_int("WRQ_GEMV_ONESHOT", 1);
+        const int ott = T == 1 ? 1 : T == 2 ? 2 : 4; // tokens per pass of the one-shot kernel
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
@@ -830,8 +875,10 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (rows == 4 && sl == 4) sl = 2;
         rows = env_int("WRQ_GEMV_ROWS", rows);
         sl = env_int("WRQ_GEMV_SL", sl);
-        if (tt > 1) rows = 4, sl = 1;
+        if (!oneshot && tt > 1) rows = 4, sl = 1;
         if (oneshot && rows != 8) rows = 4;
+        // the activations of all tokens sit in registers next to the rows: fewer rows for many tokens
+        if (oneshot && quant == kNf4 && ott == 4) rows = 4;
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
         while (i < n && g.n < (uint32_t)kMaxGroup) {
@@ -840,7 +887,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 i++;
                 continue;
             }
-            const size_t need = (size_t)a.K * tt * xsz;
+            const size_t need = oneshot ? 0 : (size_t)a.K * tt * xsz; // LDS for the staged activations
             if (!fast_ok(quant, in_f16, a) || lds_base + need > kGemvLdsBudget) {
                 if (g.n) break; // flush what is collected, then come back to this one
                 const int s = launch_generic(stream, quant, in_f16, a);
@@ -871,7 +918,6 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 p.act = a.act;
                 lds += need;
                 tasks += (a.R + rows - 1) / rows;
-                bytes += (uint64_t)a.R * a.K;
             }
             if (b < a.B) {
                 // a batch too deep for one group: finish it with single-product launches
@@ -901,9 +947,9 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;
             if (rows == 8 && nt >= 128)
-                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 8>(stream, g, nt) : launch_oneshot_nf4_nt<float, 8>(stream, g, nt);
+                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 8>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 8>(stream, g, nt, ott);
             else
-                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 4>(stream, g, nt) : launch_oneshot_nf4_nt<float, 4>(stream, g, nt);
+                s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 4>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 4>(stream, g, nt, ott);
             if (s1 != WRQ_OK) return s1;
             continue;
         }
@@ -915,9 +961,9 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;
             if (rows == 8 && nt >= 128) // the final reduction uses 16 lanes per output row
-                s1 = in_f16 ? launch_oneshot_nt<__half, 8>(stream, g, nt) : launch_oneshot_nt<float, 8>(stream, g, nt);
+                s1 = in_f16 ? launch_oneshot_nt<__half, 8>(stream, g, nt, ott) : launch_oneshot_nt<float, 8>(stream, g, nt, ott);
             else
-                s1 = in_f16 ? launch_oneshot_nt<__half, 4>(stream, g, nt) : launch_oneshot_nt<float, 4>(stream, g, nt);
+                s1 = in_f16 ? launch_oneshot_nt<__half, 4>(stream, g, nt, ott) : launch_oneshot_nt<float, 4>(stream, g, nt, ott);
             if (s1 != WRQ_OK) return s1;
             continue;
         }
