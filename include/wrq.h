@@ -11,11 +11,11 @@
  * buffer.  All pointers inside tensors are device pointers owned by the caller
  * and must stay valid until the stream has passed the call.  No entry point
  * allocates, frees or copies to the host.  All may be called from several threads at
- * once.  One limit on overlap in time: products of more than 4 tokens (wrq_matmul_mat_*,
- * and wrq_matmul_vec_* from 5 tokens on) may split K over workgroups and then keep partial
- * sums in one scratch array per device, so two such calls on different streams of one
- * device must not run at the same time; on one stream, and for runs of up to 4 tokens on
- * any streams, there is no such limit.
+ * once.  One limit on overlap in time: products on the matrix-core kernel (wrq_matmul_mat_*,
+ * and wrq_matmul_vec_* from 5 tokens on, nf4 and fp16: 3) may split K over workgroups and
+ * then keep partial sums in one scratch array per device, so two such calls on different
+ * streams of one device must not run at the same time; on one stream, and for shorter runs
+ * on any streams, there is no such limit.
  *
  * Shapes use the reference's order, x fastest (src/tensor/shape.rs:97): a matrix
  * `[K, R, B, 1]` holds B * R rows of K contiguous elements.
@@ -123,8 +123,8 @@ int wrq_quantize_mat_nf4(wrq_stream stream, const wrq_tensor *input, const wrq_t
  * TensorOp::matmul_vec_int8(matrix, minmax, input, output, act, sparse)
  *                                                          src/tensor/ops.rs:791-886
  *   matrix u8 [K, R, B, 1]; input view [K, T, B, 1]; output view [R, T, B, 1].
- *   Any T: tokens share one pass over the weights (up to 4 on the decode kernels, more on
- *   the matrix-core kernel).  `sparse` (SPARSE_INPUT) never changes results for finite
+ *   Any T: tokens share one pass over the weights (up to 4, nf4: 2, on the decode kernels,
+ *   more on the matrix-core kernel).  `sparse` (SPARSE_INPUT) never changes results for finite
  *   weights and is accepted as a hint.
  */
 int wrq_matmul_vec_int8(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor *minmax,

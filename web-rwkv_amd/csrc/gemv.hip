@@ -42,6 +42,7 @@ constexpr size_t kGemvLdsBudget = 128 * 1024;
 struct GemvProblem {
     const uint8_t *w;      // packed rows of this product
     const uint16_t *scale; // its scale blocks, indexed by flat element index as below
+    const float *quant;    // nf4: the 16-entry table of this product
     const void *x;         // first activation row (view offset applied)
     void *out;             // first output row (view offset applied)
     uint64_t e_base;       // flat element index of w's first element inside the matrix (batch offset)
@@ -525,7 +526,7 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
         if (!table_ready) {
             // built once, behind the loads of the first pass
             for (uint32_t v = tid; v < 256; v += NT) {
-                const float q0 = g.quant[v & 15], q1 = g.quant[v >> 4];
+                const float q0 = p.quant[v & 15], q1 = p.quant[v >> 4];
                 if constexpr (F16) {
                     const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
                     tab[v] = make_uint2((uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16),
@@ -806,7 +807,6 @@ int launch_oneshot_nf4_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
 template <typename XT, int ROWS>
 int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt) {
     if constexpr (sizeof(XT) == 2) {
-        if (tt == 4) return launch_oneshot_nf4_nt_n<XT, 4, false, 4>(stream, g, nt);
         if (tt == 2) return launch_oneshot_nf4_nt_n<XT, ROWS, false, 2>(stream, g, nt);
     }
     return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
@@ -863,7 +863,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // int8 at one token: the one-shot kernel (4 rows per workgroup; 8 once that still gives
         // every CU eight workgroups)
         // up to 8 tokens of f16 activations: the same kernel, several tokens per pass
-        const bool oneshot = (T == 1 || (in_f16 && T <= 4)) && env_int("WRQ_GEMV_ONESHOT", 1);
+        // (nf4: 2; at 3 - 4 tokens the activations crowd the registers and the matrix-core kernel is as fast)
+        const bool oneshot = (T == 1 || (in_f16 && T <= (quant == kNf4 ? 2u : 4u))) && env_int("WRQ_GEMV_ONESHOT", 1);
         const int ott = T == 1 ? 1 : T == 2 ? 2 : 4; // tokens per pass of the one-shot kernel
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
@@ -877,8 +878,6 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         sl = env_int("WRQ_GEMV_SL", sl);
         if (!oneshot && tt > 1) rows = 4, sl = 1;
         if (oneshot && rows != 8) rows = 4;
-        // the activations of all tokens sit in registers next to the rows: fewer rows for many tokens
-        if (oneshot && quant == kNf4 && ott == 4) rows = 4;
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
         while (i < n && g.n < (uint32_t)kMaxGroup) {
@@ -895,6 +894,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 i++;
                 continue;
             }
+            // the resident kernel builds one table per workgroup: its groups share the table tensor
+            if (!oneshot && a.quant != g.quant && g.n) break;
             if (a.B > 1 && g.n + a.B > (uint32_t)kMaxGroup && g.n) break;
             if (lds + need * a.B > kGemvLdsBudget && g.n) break;
             // the batch axis unrolls into products of its own
@@ -904,6 +905,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 const uint64_t e_base = (uint64_t)b * a.R * a.K;
                 p.w = a.w + (quant == kInt8 ? e_base : e_base >> 1);
                 p.scale = a.scale;
+                p.quant = a.quant;
                 p.e_base = e_base;
                 p.x = static_cast<const uint8_t *>(a.x) + (uint64_t)b * a.x_batch_stride * xsz;
                 p.out = static_cast<uint8_t *>(a.out) + (uint64_t)b * a.out_batch_stride * (a.out_f16 ? 2 : 4);
