@@ -196,11 +196,12 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         sp = QUANT == kFp16 ? nullptr : reinterpret_cast<const uint32_t *>(a.scale) + ((((uint64_t)b * a.R + row) * K + k_begin) >> 7);
     }
 
+    // nf4: the two table values behind this thread's entry of the byte table, requested before the
+    // first weights so that they are back first; the entry is written once those are on their way
+    float tq0 = 0.0f, tq1 = 0.0f;
     if (QUANT == kNf4) {
-        // entry for byte v: (hi(q[v & 15]), hi(q[v >> 4])), (lo(..), lo(..)); lo scaled by 2^11
-        const float q0 = a.quant[tid & 15], q1 = a.quant[(tid >> 4) & 15];
-        const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
-        if (tid < 256) pair[tid] = make_uint2(pack_h2(q0, q1), pack_h2((q0 - h0) * 2048.0f, (q1 - h1) * 2048.0f));
+        tq0 = a.quant[tid & 15];
+        tq1 = a.quant[(tid >> 4) & 15];
     }
 
     // activation staging: piece p of a stage is 8 consecutive k of one token; the 16 pieces of a
@@ -416,6 +417,11 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     load_stage(0, stage);
 #pragma unroll
     for (int j = 0; j < NBUF; j++) load_w(j, ring[j]);
+    if (QUANT == kNf4) {
+        // entry for byte v: (hi(q[v & 15]), hi(q[v >> 4])), (lo(..), lo(..)); lo scaled by 2^11
+        const float h0 = h2f(f2h(tq0)), h1 = h2f(f2h(tq1));
+        if (tid < 256) pair[tid] = make_uint2(pack_h2(tq0, tq1), pack_h2((tq0 - h0) * 2048.0f, (tq1 - h1) * 2048.0f));
+    }
     constexpr int STAGES = kUnrollStages > NBUF / LSUB ? kUnrollStages : NBUF / LSUB; // stages per loop iteration
     for (uint32_t S0 = 0; S0 < nstages; S0 += STAGES) {
 #pragma unroll

@@ -501,6 +501,17 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
 #pragma unroll
         for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
 
+    // the table values this thread turns into entries: requested before anything else, so that
+    // they are back first (loads return in order) and the table is built while the weights arrive
+    constexpr int NE = NT >= 256 ? 1 : 256 / NT; // entries per thread
+    float tq0[NE], tq1[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+        const uint32_t v = (tid + e * NT) & 255u;
+        tq0[e] = p.quant[v & 15];
+        tq1[e] = p.quant[v >> 4];
+    }
+
     bool table_ready = false;
     for (uint32_t c = tid; c < nchunk || !table_ready; c += NT) {
         const bool live = c < nchunk;
@@ -524,18 +535,22 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
             sc[r] = p.scale[(e0 + off) >> 6];
         }
         if (!table_ready) {
-            // built once, behind the loads of the first pass
-            for (uint32_t v = tid; v < 256; v += NT) {
-                const float q0 = p.quant[v & 15], q1 = p.quant[v >> 4];
-                if constexpr (F16) {
-                    const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
-                    tab[v] = make_uint2((uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16),
-                                        (uint32_t)f2h((q0 - h0) * 2048.0f) | ((uint32_t)f2h((q1 - h1) * 2048.0f) << 16));
-                } else {
-                    tab[v] = make_uint2(__float_as_uint(q0), __float_as_uint(q1));
+            // built once, behind the loads of the first pass, which stay in flight across the barrier
+#pragma unroll
+            for (int e = 0; e < NE; e++) {
+                const uint32_t v = tid + e * NT;
+                const float q0 = tq0[e], q1 = tq1[e];
+                if (v < 256) {
+                    if constexpr (F16) {
+                        const float h0 = h2f(f2h(q0)), h1 = h2f(f2h(q1));
+                        tab[v] = make_uint2((uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16),
+                                            (uint32_t)f2h((q0 - h0) * 2048.0f) | ((uint32_t)f2h((q1 - h1) * 2048.0f) << 16));
+                    } else {
+                        tab[v] = make_uint2(__float_as_uint(q0), __float_as_uint(q1));
+                    }
                 }
             }
-            __syncthreads();
+            lds_barrier();
             table_ready = true;
         }
         if (!live) continue;
