@@ -646,12 +646,9 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
     const MatmulArgs &a = args[0];
     const uint32_t T = a.T;
     const uint32_t steps = a.K / kStep;
-    uint64_t rows = 0, rows_max = 0;
-    for (int i = 0; i < n; i++) {
-        rows += args[i].R;
-        rows_max = args[i].R > rows_max ? args[i].R : rows_max;
-    }
-    const uint64_t rt = rows_max * a.B * T;
+    uint64_t rows = 0;
+    for (int i = 0; i < n; i++) rows += args[i].R;
+    const uint64_t rt = rows * a.B * T; // the group as one product
     const bool small = rt <= (1u << 20);
     int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? (small ? 2 : 4) : (small && a.K <= 8192 ? 2 : 8);
     ntile = env_int("WRQ_GEMM_NTILE", ntile);
