@@ -8,24 +8,32 @@
 // 4096 x 4096 product is 17 MB, a few microseconds of HBM time, and a dispatch of its
 // own costs about as much again.
 //
-// Structure (HBM-bound; every packed byte is read once, 16 bytes per lane, 1 KiB per
-// wave instruction, contiguous along a weight row):
-//   * resident workgroups of 8 waves (two per CU) stage the activation rows of the group
-//     in LDS once, then every wave pulls tasks -- ROWS consecutive weight rows over the
-//     full K -- from a strided sequence, so consecutive tasks land on different CUs;
-//   * a wave walks its rows in slices of 64 lanes x 16 bytes, loads of slice s+1 in
-//     flight while slice s is consumed, and finishes a task with a DPP/readlane
-//     reduction: no barrier and no LDS exchange after the prologue;
-//   * int8: the 16 weights of a lane load lie inside one 128-block, so the affine
-//     dequantisation factors out of the dot product,
-//         sum_j (u_j s + m) x_j = s sum_j u_j x_j + m sum_j x_j ,  s = (max - min) / 255:
-//     one v_cvt_f32_ubyteN and one FMA per weight;
-//   * nf4: a 256-entry LDS table maps a packed byte to its two f32 table values with one
-//     ds_read_b64 (2 address ops + 2 FMA per two weights instead of 4 + 2); each of 16
-//     lane groups reads its own copy of the table, which puts the 16 lanes served in
-//     one LDS cycle in 16 different bank pairs whatever bytes they hold; absmax scales
-//     the 32-term partial sum of a lane load, which lies inside one 64-block.
-// Accumulation is f32 throughout.
+// Every packed byte is read once, 16 bytes per lane, 1 KiB per wave instruction, contiguous
+// along a weight row; accumulation is f32 throughout.  Three kernel families:
+//
+//   * one-shot kernels (gemv_int8_oneshot_kernel, gemv_nf4_oneshot_kernel,
+//     gemv_fp16_oneshot_kernel) -- the decode path: one token, or a run of up to 4 (int8) /
+//     2 (nf4) tokens of f16 activations.  One short-lived workgroup per task (4 or 8 rows over
+//     the whole K, one lane per 16-byte chunk of a row) requests everything it needs at once and
+//     consumes it in arrival order; thousands of workgroups keep the memory system full.
+//     Details stand above each kernel.
+//   * the resident kernel (gemv_kernel) -- longer runs that the matrix-core kernel cannot take
+//     (K no multiple of 128, f32 activations below 16 tokens): workgroups of 8 waves (two per
+//     CU) stage the activation rows of the group in LDS once, then every wave pulls tasks --
+//     ROWS consecutive weight rows over the full K -- from a strided sequence, so consecutive
+//     tasks land on different CUs; a wave walks its rows in slices of 64 lanes x 16 bytes,
+//     loads of slice s+1 in flight while slice s is consumed, and finishes a task with a
+//     DPP/readlane reduction: no barrier and no LDS exchange after the prologue.
+//       int8: the 16 weights of a lane load lie inside one 128-block, so the affine
+//         dequantisation factors out of the dot product,
+//             sum_j (u_j s + m) x_j = s sum_j u_j x_j + m sum_j x_j ,  s = (max - min) / 255:
+//         one v_cvt_f32_ubyteN and one FMA per weight;
+//       nf4: a 256-entry LDS table maps a packed byte to its two f32 table values with one
+//         ds_read_b64 (2 address ops + 2 FMA per two weights instead of 4 + 2); each of 32
+//         lane groups reads its own copy of the table; absmax scales the 32-term partial sum
+//         of a lane load, which lies inside one 64-block.
+//   * generic kernels (gemv_generic_kernel, gemv_fp16_generic_kernel) -- any shape the
+//     reference accepts (K % 4, blocks straddling rows, unaligned views); correctness path.
 #include "wrq_device.h"
 #include "wrq_host.h"
 
@@ -875,7 +883,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // rows per task: 4, or 2 when the group is too small to give every wave of 256 CUs a task
         uint64_t rows_total = 0;
         for (int j = i; j < n; j++) rows_total += (uint64_t)args[j].R * args[j].B;
-        // int8 at one token: the one-shot kernel (4 rows per workgroup; 8 once that still gives
+        // one token or a short run: the one-shot kernels (4 rows per workgroup; 8 once that still gives
         // every CU eight workgroups)
         // up to 8 tokens of f16 activations: the same kernel, several tokens per pass
         // (nf4: 2; at 3 - 4 tokens the activations crowd the registers and the matrix-core kernel is as fast)
