@@ -460,6 +460,33 @@ def test_short_runs_on_decode_kernels(gpu, oracle, kind, K, R, T):
     assert_close(got, one, 1e-3, "vs one call per token")  # same arithmetic up to the last f16 ulp
 
 
+@pytest.mark.parametrize("T,x_dtype", [(1, np.float16), (2, np.float16), (3, np.float32), (32, np.float16), (40, np.float16)])
+def test_grouped_nf4_products_keep_their_own_tables(gpu, oracle, T, x_dtype):
+    # every Matrix::Fp4 owns its table tensor (src/tensor/matrix.rs:180-222): ops of one group may
+    # carry different tables -- here even different contents -- on every kernel family
+    # (one-shot, resident with f32 activations, matrix cores)
+    import torch
+
+    announce("grouped nf4, own tables", T, x_dtype.__name__)
+    K, R = 1024, 768
+    rng = np.random.default_rng(SEED + 31 + T)
+    tables = [NF4_QUANT, (np.arange(-8, 8) / 8.0).astype(np.float32), NF4_QUANT.copy()]
+    x = gen_f16(rng, (T, K), 1.0).astype(x_dtype)
+    xd = dev(x)
+    ops, outs, truths = [], [], []
+    for tab in tables:
+        w = gen_f16(rng, (R, K), 0.02)
+        p, am = oracle.quant_nf4(w, tab)
+        m = gpu.Matrix("Fp4", dev(p), dev(am), torch.tensor(tab, dtype=torch.float32, device="cuda"))
+        out = torch.full((T, R), float("nan"), dtype=torch.float32, device="cuda")
+        ops.append((m, xd, out, gpu.ACT_NONE, False, {}))
+        outs.append(out)
+        truths.append(truth_matmul(nf4_dequant64(p, am, tab), x))
+    gpu.matmul_vec_group(ops)
+    for j, (out, truth) in enumerate(zip(outs, truths)):
+        assert_close(host(out), truth, EPS, f"op {j} vs float64 with its own table")
+
+
 @pytest.mark.parametrize("T", [1, 2, 4, 5, 32])
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
 def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind, T):
