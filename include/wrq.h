@@ -12,7 +12,7 @@
  * and must stay valid until the stream has passed the call.  No entry point
  * allocates, frees or copies to the host.  All may be called from several threads at
  * once.  One limit on overlap in time: products on the matrix-core kernel (wrq_matmul_mat_*,
- * and wrq_matmul_vec_* from 5 tokens on, nf4 and fp16: 3) may split K over workgroups and
+ * and wrq_matmul_vec_* from 5 tokens on, nf4: 3) may split K over workgroups and
  * then keep partial sums in one scratch array per device, so two such calls on different
  * streams of one device must not run at the same time; on one stream, and for shorter runs
  * on any streams, there is no such limit.
@@ -196,6 +196,7 @@ int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const w
  *
  * TensorOp::matmul_vec_fp16(matrix, input, output, act, sparse)   src/tensor/ops.rs:697-784
  *   matrix f16 [K, R, B, 1]; input view [K, T, B, 1]; output view [R, T, B, 1]; K % 4 == 0.
+ *   Up to 4 tokens share a pass over the weights on the decode kernel, more on the matrix-core kernel.
  * TensorOp::matmul_mat_fp16(matrix, input, output, act)           src/tensor/ops.rs:999-1061
  *   matrix: view of an f16 tensor covering its whole parent; K, R and T multiples of 4.
  */

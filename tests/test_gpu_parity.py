@@ -604,7 +604,7 @@ def test_v5_shape_layer_sequence(gpu, oracle, kind):
 # ---------------------------------------------------------------- plain f16 weights
 
 
-FP16_CASES = [(2048, 512, 1), (2048, 512, 2), (4096, 1024, 1), (324, 64, 5), (1056, 64, 3), (2048, 512, 17),
+FP16_CASES = [(2048, 512, 1), (2048, 512, 2), (2048, 516, 3), (4096, 16388, 4), (1056, 64, 7), (4096, 1024, 1), (324, 64, 5), (1056, 64, 3), (2048, 512, 17),
               (2048, 2048, 32), (2560, 2048, 64), (4096, 4096, 128), (2048, 65536, 1), (2048, 65536, 32)]
 
 

@@ -614,28 +614,37 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
 // one-shot shape without any dequantisation.  A lane holds 8 weights (16 bytes) of each of its
 // ROWS rows and the 8 activations they meet; f16 activations go through v_dot2_f32_f16, f32
 // activations through converts and fmas.  HBM-bound: 2 bytes per weight.
-template <typename XT, int ROWS, int NT>
+// TT > 1 (f16 activations only): tokens token .. token + TT - 1 of a short run share the pass.
+template <typename XT, int ROWS, int NT, int TT>
 __global__ __launch_bounds__(NT) void gemv_fp16_oneshot_kernel(const MatmulArgs a, uint32_t token) {
+    static_assert(TT == 1 || sizeof(XT) == 2, "several tokens per pass: f16 activations only");
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     constexpr bool F16 = sizeof(XT) == 2;
-    __shared__ float red[ROWS][NROW16];
+    __shared__ float red[ROWS * TT][NROW16];
     const uint32_t tid = threadIdx.x;
     const uint32_t b = blockIdx.y;
     const uint32_t K = a.K, nchunk = K >> 3;
     const uint32_t row0 = blockIdx.x * ROWS;
     const uint32_t rows_valid = min((uint32_t)ROWS, a.R - row0);
     const uint16_t *wbase = reinterpret_cast<const uint16_t *>(a.w) + ((uint64_t)b * a.R + row0) * K;
-    const XT *x = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride + (uint64_t)token * a.x_token_stride;
+    const XT *x = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
 
-    float acc[ROWS];
+    float acc[ROWS][TT];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
 
     for (uint32_t c = tid; c < nchunk; c += NT) {
         constexpr int NX = F16 ? 1 : 2;
-        uint4 xv[NX];
+        uint4 xv[TT][NX];
 #pragma unroll
-        for (int i = 0; i < NX; i++) xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)c << 3)) + 16 * i);
+        for (int t = 0; t < TT; t++) {
+            const uint32_t tok = min(token + t, a.T - 1); // tokens past the run repeat the last one
+#pragma unroll
+            for (int i = 0; i < NX; i++)
+                xv[t][i] = load128(reinterpret_cast<const uint8_t *>(x + (uint64_t)tok * a.x_token_stride + ((uint64_t)c << 3)) + 16 * i);
+        }
         uint4 wv[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
@@ -643,41 +652,46 @@ __global__ __launch_bounds__(NT) void gemv_fp16_oneshot_kernel(const MatmulArgs 
             wv[r] = load128_stream(wbase + (uint64_t)rr * K + ((uint64_t)c << 3));
         }
         if constexpr (F16) {
-            const uint32_t xd[4] = {xv[0].x, xv[0].y, xv[0].z, xv[0].w};
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
 #pragma unroll
-                for (int d = 0; d < 4; d++) acc[r] = dot2(w[d], xd[d], acc[r]);
+                for (int t = 0; t < TT; t++) {
+                    const uint32_t xd[4] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w};
+#pragma unroll
+                    for (int d = 0; d < 4; d++) acc[r][t] = dot2(w[d], xd[d], acc[r][t]);
+                }
             }
         } else {
-            const float xf[8] = {__uint_as_float(xv[0].x), __uint_as_float(xv[0].y), __uint_as_float(xv[0].z), __uint_as_float(xv[0].w),
-                                 __uint_as_float(xv[1].x), __uint_as_float(xv[1].y), __uint_as_float(xv[1].z), __uint_as_float(xv[1].w)};
+            const float xf[8] = {__uint_as_float(xv[0][0].x), __uint_as_float(xv[0][0].y), __uint_as_float(xv[0][0].z), __uint_as_float(xv[0][0].w),
+                                 __uint_as_float(xv[0][1].x), __uint_as_float(xv[0][1].y), __uint_as_float(xv[0][1].z), __uint_as_float(xv[0][1].w)};
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 float wf[8];
                 unpack8h(wv[r], wf);
 #pragma unroll
-                for (int j = 0; j < 8; j++) acc[r] = fmaf(wf[j], xf[j], acc[r]);
+                for (int j = 0; j < 8; j++) acc[r][0] = fmaf(wf[j], xf[j], acc[r][0]);
             }
         }
     }
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        const float s = row_sum(acc[r]);
-        if ((tid & 15) == 0) red[r][tid >> 4] = s;
-    }
+    for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float s = row_sum(acc[r][t]);
+            if ((tid & 15) == 0) red[r * TT + t][tid >> 4] = s;
+        }
     __syncthreads();
-    if (tid < ROWS * 16) {
-        const uint32_t r = tid >> 4, l = tid & 15;
+    const uint32_t l = tid & 15;
+    for (uint32_t o = tid >> 4; o < (uint32_t)(ROWS * TT); o += NROW16) {
         float s = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NROW16 / 16; i++) s += red[r][l + 16 * i];
-        if (NROW16 < 16) s = l < NROW16 ? red[r][l] : 0.0f;
+        for (int i = 0; i < NROW16 / 16; i++) s += red[o][l + 16 * i];
+        if (NROW16 < 16) s = l < NROW16 ? red[o][l] : 0.0f;
         s = row_sum(s);
-        const uint32_t row = row0 + r;
-        if (l == 0 && row < a.R)
-            store_out(a.out, a.out_f16, (uint64_t)b * a.out_batch_stride + (uint64_t)token * a.out_token_stride + row, act_apply(a.act, s));
+        const uint32_t row = row0 + o / TT, t = token + o % TT;
+        if (l == 0 && row < a.R && t < a.T)
+            store_out(a.out, a.out_f16, (uint64_t)b * a.out_batch_stride + (uint64_t)t * a.out_token_stride + row, act_apply(a.act, s));
     }
 }
 
@@ -1011,19 +1025,19 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
     return WRQ_OK;
 }
 
-template <typename XT, int ROWS>
+template <typename XT, int ROWS, int TT>
 void launch_fp16_nt(hipStream_t stream, const MatmulArgs &a, uint32_t token, int nt) {
     const dim3 grid((a.R + ROWS - 1) / ROWS, a.B);
     if (nt >= 512)
-        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 512>), grid, dim3(512), 0, stream, a, token);
+        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 512, TT>), grid, dim3(512), 0, stream, a, token);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 256>), grid, dim3(256), 0, stream, a, token);
+        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 256, TT>), grid, dim3(256), 0, stream, a, token);
     else
-        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 128>), grid, dim3(128), 0, stream, a, token);
+        hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 128, TT>), grid, dim3(128), 0, stream, a, token);
 }
 
-// f16 weights, decode-shaped: one pass over the weights per token (the chunk kernel takes the
-// runs with several tokens); odd shapes and unaligned views go to the generic kernel.
+// f16 weights, decode-shaped: one pass over the weights per 1 - 4 tokens (the chunk kernel takes
+// the longer runs); odd shapes and unaligned views go to the generic kernel.
 int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &a) {
     if (a.R == 0 || a.T == 0 || a.B == 0) return WRQ_OK;
     if (a.T > 65535u || a.B > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a.T > a.B ? a.T : a.B, 65535u);
@@ -1041,11 +1055,22 @@ int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &a) {
     const uint32_t nchunk = a.K / 8;
     const int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : 128;
     const bool rows8 = (uint64_t)a.R * a.B / 8 >= 2048u;
-    for (uint32_t t = 0; t < a.T; t++) {
-        if (rows8) {
-            if (in_f16) launch_fp16_nt<__half, 8>(stream, a, t, nt); else launch_fp16_nt<float, 8>(stream, a, t, nt);
+    // f16 activations: up to 4 tokens per pass over the weights; f32: one
+    for (uint32_t t = 0; t < a.T;) {
+        const uint32_t left = a.T - t;
+        if (in_f16 && left >= 3) {
+            if (rows8) launch_fp16_nt<__half, 8, 4>(stream, a, t, nt); else launch_fp16_nt<__half, 4, 4>(stream, a, t, nt);
+            t += 4;
+        } else if (in_f16 && left == 2) {
+            if (rows8) launch_fp16_nt<__half, 8, 2>(stream, a, t, nt); else launch_fp16_nt<__half, 4, 2>(stream, a, t, nt);
+            t += 2;
         } else {
-            if (in_f16) launch_fp16_nt<__half, 4>(stream, a, t, nt); else launch_fp16_nt<float, 4>(stream, a, t, nt);
+            if (rows8) {
+                if (in_f16) launch_fp16_nt<__half, 8, 1>(stream, a, t, nt); else launch_fp16_nt<float, 8, 1>(stream, a, t, nt);
+            } else {
+                if (in_f16) launch_fp16_nt<__half, 4, 1>(stream, a, t, nt); else launch_fp16_nt<float, 4, 1>(stream, a, t, nt);
+            }
+            t += 1;
         }
     }
     return check_launch("matmul_vec_fp16");

@@ -179,15 +179,16 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
                          ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0) &&
                          ((uintptr_t)a.out % (4 * osz) == 0) && ((a.out_token_stride * osz) % (4 * osz) == 0) &&
                          ((a.out_batch_stride * osz) % (4 * osz) == 0);
-    // decode entry point with several tokens: up to 4 (int8) or 2 (nf4) tokens of f16 activations
-    // share one pass of the one-shot VALU kernels (7B int8 step: 1.8 - 2.1 ms at 2 - 4 tokens against
-    // 2.8 ms); longer runs, and plain f16 weights from 3 tokens on, go to the matrix-core kernel.
+    // decode entry point with several tokens: up to 4 (int8, fp16) or 2 (nf4) tokens of f16
+    // activations share one pass of the one-shot VALU kernels (7B int8 step: 1.8 - 2.1 ms at 2 - 4
+    // tokens against 2.8 ms; f16 head: 97 us at 4 tokens against 120); longer runs go to the
+    // matrix-core kernel.
     // WRQ_VEC_CHUNK_MIN_T overrides the first token count that does
     static const int64_t chunk_min_env = [] {
         const char *e = getenv("WRQ_VEC_CHUNK_MIN_T");
         return (int64_t)((e && *e) ? atoi(e) : -1);
     }();
-    const uint64_t chunk_min_t = chunk_min_env >= 0 ? (uint64_t)chunk_min_env : quant == kInt8 ? 5u : 3u;
+    const uint64_t chunk_min_t = chunk_min_env >= 0 ? (uint64_t)chunk_min_env : quant == kNf4 ? 3u : 5u;
     // f32 activations are rounded to f16 by the matrix-core kernel: keep them on the exact VALU
     // kernels below 16 tokens
     const bool chunk = entry == kMat ? true : n >= (in_f16 ? chunk_min_t : (uint64_t)16);
