@@ -633,6 +633,46 @@ def test_fp16_matrix_products(gpu, oracle, K, R, T):
         assert_close(got32, want, EPS, "f32 activations, squared relu")
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_all_routes(gpu, oracle, seed):
+    """Seeded random walk over formats, shapes, token counts, operand types, activations and entry
+    points: whatever kernel a call is routed to, the result is the float64 product of the
+    dequantised weights."""
+    import torch
+
+    rng = np.random.default_rng(SEED + 1000 + seed)
+    acts = list(ACTS)
+    for case in range(28):
+        kind = ["int8", "nf4", "fp16"][int(rng.integers(0, 3))]
+        K = int(rng.choice([128, 256, 384, 1024, 2048, 4096, 64, 192, 320, 1056, 96, 2080]))
+        if kind == "nf4" and K % 64:
+            K += 64 - K % 64
+        R = int(rng.choice([4, 8, 36, 64, 132, 512, 1028, 2048]))
+        if kind != "fp16":
+            while (R * K) % 128:  # whole scale blocks
+                R += 4
+        T = int(rng.choice([1, 1, 2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 32, 40]))
+        x_dtype = np.float16 if rng.random() < 0.7 else np.float32
+        out_dtype = np.float16 if rng.random() < 0.5 else np.float32
+        act = int(rng.integers(0, len(acts)))
+        mat_ok = T % 4 == 0 and K % (64 if kind == "nf4" else 32) == 0 and x_dtype == np.float16
+        entry = "mat" if mat_ok and rng.random() < 0.4 else "vec"
+        announce("fuzz", seed, case, kind, K, R, T, x_dtype.__name__, out_dtype.__name__, acts[act], entry)
+        w = gen_f16(rng, (R, K), 0.05)
+        x = gen_f16(rng, (T, K), 1.0).astype(x_dtype)
+        if kind == "fp16":
+            m, wdeq = gpu.Matrix.fp16(dev(w)), w.astype(np.float64)
+        else:
+            wp, scale, wdeq = pack(oracle, kind, w)
+            m = gpu_matrix(gpu, kind, wp, scale)
+        truth = truth_matmul(wdeq, x, acts[act])
+        if acts[act] in ("stable_exp", "opposite_exp", "softplus") and not np.isfinite(truth).all():
+            continue
+        got = run(gpu, m, x, R, entry, out_dtype, act=act)
+        eps = EPS if x_dtype == np.float16 or entry == "vec" else 4e-3
+        assert_close(got, truth, eps, f"{kind} K={K} R={R} T={T} {entry} act={acts[act]}")
+
+
 def test_entry_points_from_several_threads(gpu, oracle):
     # ops are built on worker threads in the reference (src/runtime/mod.rs:138-166): the entry
     # points keep no shared mutable state (errors are per thread); every thread drives its own
