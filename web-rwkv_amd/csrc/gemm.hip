@@ -108,10 +108,20 @@ struct Geometry {
     static constexpr int NBUFH = LSUB >= 2 ? LSUB : 2;
     static constexpr int nbuf(int quant) { return quant == kFp16 ? NBUFH : NBUFQ; }
     static constexpr int TILE_FLOATS = 1024 * MRT * NTILE;                 // outputs of one workgroup
+    // Token tiles up to 64 wide are bound by the vector memory path, not by arithmetic: a wave
+    // instruction that gathers the A-operand layout straight from memory (16 rows x 64 B, or x 32 B
+    // for nf4) costs the texture path about 54 clocks, three times a line-wise one.  There the weights
+    // are fetched line-wise (a row's bytes of a step in adjacent lanes: 8 rows x 128 B per instruction
+    // for int8, 16 x 64 B for nf4, 4 x 256 B for f16) and turned into the A-operand layout through a
+    // wave-private LDS slot.  The widest tile keeps the direct gather: its LDS is the busiest unit.
+    static constexpr bool transposed_loads(int) { return NTILE <= 4 && KG == 1; }
+    static constexpr int wstep(int quant) { return quant == kFp16 ? 2 * kStep : quant == kInt8 ? kStep : kStep / 2; } // weight bytes per row and step
+    static constexpr int tpitch(int quant) { return wstep(quant) + 16; }    // bytes per row of a slot: +16 B rotates the banks
+    static constexpr size_t tslot_bytes(int quant) { return transposed_loads(quant) ? (size_t)4 * MRT * 16 * tpitch(quant) : 0; }
     // LDS: 2 x activation tile [BN][PITCH] f16 | 2 x row scales [KSUB][BM] float2 | 2 x token sums [KSUB][BN] f32 | nf4 pair table
     static constexpr size_t lds_bytes(int quant) {
         return (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) + (size_t)2 * KSUB * BN * sizeof(float) +
-               (quant == kNf4 ? 256 * sizeof(uint2) : 0);
+               (quant == kNf4 ? 256 * sizeof(uint2) : 0) + tslot_bytes(quant);
     }
     static_assert((size_t)4 * MRT * NTILE * 1024 <= (size_t)2 * BN * PITCH * sizeof(uint16_t), "partial tiles of a k group fit the activation buffers");
 };
@@ -161,6 +171,10 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         reinterpret_cast<float(*)[KSUB][BN]>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2));
     uint2 *pair = reinterpret_cast<uint2 *>(smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) +
                                             (size_t)2 * KSUB * BN * sizeof(float));
+    constexpr bool TRW = G::transposed_loads(QUANT);
+    constexpr int TPITCH = G::tpitch(QUANT);
+    uint8_t *tslots = smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) +
+                      (size_t)2 * KSUB * BN * sizeof(float) + (QUANT == kNf4 ? 256 * sizeof(uint2) : 0);
 
     uint32_t row_tile, tblock;
     tile_of_block(tile_id, ga.tblocks, row_tile, tblock);
@@ -188,6 +202,22 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         const uint64_t e = ((uint64_t)b * a.R + row) * K + k_begin; // flat element index of (row, k_begin)
         wp[i] = QUANT == kFp16 ? a.w + 2 * e + 16 * g : QUANT == kInt8 ? a.w + e + 16 * g : a.w + (e >> 1) + 8 * g;
     }
+    // line-wise fetch: the WSTEP bytes of a row and step sit in LPR adjacent lanes, load j of a row tile
+    // takes rows RPL j .. RPL j + RPL - 1
+    constexpr int LPR = WSTEP / 16, RPL = 64 / LPR; // lanes per row, rows per load (NW * RPL = 16)
+    static_assert(NW * RPL == 16, "a row tile is NW line-wise loads");
+    const uint8_t *wq[MRT][NW];
+    if constexpr (TRW) {
+#pragma unroll
+        for (int i = 0; i < MRT; i++)
+#pragma unroll
+            for (int j = 0; j < NW; j++) {
+                const uint32_t row = min(row_base + 16 * i + RPL * j + lane / LPR, a.R - 1);
+                const uint64_t e = ((uint64_t)b * a.R + row) * K + k_begin; // flat element index of (row, k_begin)
+                wq[i][j] = (QUANT == kFp16 ? a.w + 2 * e : QUANT == kInt8 ? a.w + e : a.w + (e >> 1)) + 16 * (lane % LPR);
+            }
+    }
+    uint8_t *tslot = tslots + (size_t)wave * (MRT * 16 * TPITCH); // this wave's transposition slot
     // scale words (one 32-bit word per row and step for both formats: a (min, max) pair, or the
     // absmax of two 64-blocks): thread t < BM fetches those of workgroup row t
     const uint32_t *sp;
@@ -277,7 +307,10 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
             const uint8_t *p = wp[i] + step * WSTEP;
-            if (QUANT == kFp16) {
+            if constexpr (TRW) {
+#pragma unroll
+                for (int j = 0; j < NW; j++) dst.w[i][j] = load128_stream(wq[i][j] + step * WSTEP);
+            } else if (QUANT == kFp16) {
 #pragma unroll
                 for (int j = 0; j < NW; j++) dst.w[i][j] = load128_stream(p + 64 * j); // operand j: k = 32 j + 8 g .. + 8
             } else if (QUANT == kInt8) {
@@ -300,6 +333,32 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     // one K step on the matrix cores: weights `cur` against step `sub` of the stage in LDS buffer `buf`.
     // Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
     auto compute = [&](const StepRegs &cur, int buf, uint32_t sub) {
+        // the step's packed weights of this lane in A-operand layout: as loaded, or line-wise loads
+        // passed through the wave's LDS slot (one wave writes and reads a slot, in program order: no barrier)
+        uint4 wa[MRT][NW];
+        if constexpr (TRW) {
+#pragma unroll
+            for (int i = 0; i < MRT; i++)
+#pragma unroll
+                for (int j = 0; j < NW; j++)
+                    *reinterpret_cast<uint4 *>(tslot + (i * 16 + RPL * j + lane / LPR) * TPITCH + 16 * (lane % LPR)) = cur.w[i][j];
+#pragma unroll
+            for (int i = 0; i < MRT; i++) {
+                const uint8_t *row = tslot + (i * 16 + r16) * TPITCH;
+                if constexpr (QUANT == kNf4) {
+                    const uint2 v0 = *reinterpret_cast<const uint2 *>(row + 8 * g), v1 = *reinterpret_cast<const uint2 *>(row + 32 + 8 * g);
+                    wa[i][0] = make_uint4(v0.x, v0.y, v1.x, v1.y);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NW; j++) wa[i][j] = *reinterpret_cast<const uint4 *>(row + 64 * j + 16 * g);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MRT; i++)
+#pragma unroll
+                for (int j = 0; j < NW; j++) wa[i][j] = cur.w[i][j];
+        }
         if constexpr (QUANT == kFp16) {
             // plain f16 weights are the A operands as loaded; the accumulators stay in the matrix cores
             const uint16_t *xh = xs[buf] + r16 * PITCH + sub * kStep + 8 * g;
@@ -313,7 +372,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                     for (int i = 0; i < MRT; i++) {
                         HalfPack A;
-                        const uint4 &wv = cur.w[i][j < NW ? j : 0];
+                        const uint4 &wv = wa[i][j < NW ? j : 0];
                         A.u[0] = wv.x; A.u[1] = wv.y; A.u[2] = wv.z; A.u[3] = wv.w;
                         out[i][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.h, B.h, out[i][n], 0, 0, 0);
                     }
@@ -334,8 +393,8 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
             HalfPack A[MRT][4];
 #pragma unroll
             for (int i = 0; i < MRT; i++) {
-                const uint32_t w[8] = {cur.w[i][0].x,      cur.w[i][0].y,      cur.w[i][0].z,      cur.w[i][0].w,
-                                       cur.w[i][NW - 1].x, cur.w[i][NW - 1].y, cur.w[i][NW - 1].z, cur.w[i][NW - 1].w};
+                const uint32_t w[8] = {wa[i][0].x,      wa[i][0].y,      wa[i][0].z,      wa[i][0].w,
+                                       wa[i][NW - 1].x, wa[i][NW - 1].y, wa[i][NW - 1].z, wa[i][NW - 1].w};
 #pragma unroll
                 for (int d = 0; d < 8; d++) {
                     // 4 codes of one dword -> f16 pairs 1024 + u
@@ -367,7 +426,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
             HalfPack Ah[MRT][4], Al[MRT][4];
 #pragma unroll
             for (int i = 0; i < MRT; i++) {
-                const uint32_t w[4] = {cur.w[i][0].x, cur.w[i][0].y, cur.w[i][0].z, cur.w[i][0].w};
+                const uint32_t w[4] = {wa[i][0].x, wa[i][0].y, wa[i][0].z, wa[i][0].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
 #pragma unroll
