@@ -696,39 +696,34 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
 // `n` products with one K, token count and batch count (the caller groups them so).
 template <int QUANT, typename XT>
 int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
-    // Tile choice, from sweeps over the shapes of this path (rows 4096 .. 65536, K 2048 .. 14336,
-    // 16 .. 256 tokens).  Small products (rows x tokens up to 2^20) want many small tiles: 32
-    // tokens per workgroup (4 steps per barrier), as many rows per workgroup as still give
-    // about one workgroup per CU, and K split only up to that point.  Large ones want the
-    // widest token tile, 128 rows per workgroup and K split until 2-4 workgroups per CU.
-    // A group counts as one product with the rows of all its members.
+    // Tile choice, from sweeps over the launch shapes of this path (rows 4096 .. 65536, K 2048 ..
+    // 14336, 5 .. 256 tokens, single products and groups).  A group counts as one product with the
+    // rows of all its members.  Token tile: as narrow as the run up to 32 tokens; beyond that 64
+    // tokens (32 for small products with short rows), which still fetch their weights line-wise;
+    // only very large products (the 65536-row head from 128 tokens on) take the 128-token tile.
     const MatmulArgs &a = args[0];
     const uint32_t T = a.T;
     const uint32_t steps = a.K / kStep;
     uint64_t rows = 0;
     for (int i = 0; i < n; i++) rows += args[i].R;
-    const uint64_t rt = rows * a.B * T; // the group as one product
+    const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
-    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : T <= 64 ? (small ? 2 : 4) : (small && a.K <= 8192 ? 2 : 8);
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192) ? 2 : (T > 64 && rt >= (1u << 23)) ? 8 : 4;
     ntile = env_int("WRQ_GEMM_NTILE", ntile);
     const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
+    // 64-row tiles where they give about one workgroup per CU without a split of K (a 16-token tile:
+    // also below that); otherwise 128-row tiles, fewer activation copies per weight byte, and more splits
     int mrt = 2;
-    if (ntile <= 2 && (uint64_t)((rows + 63) / 64) * tblocks * a.B <= 256) mrt = 1;
+    const uint64_t wgs64 = (uint64_t)((rows + 63) / 64) * tblocks * a.B;
+    if ((ntile == 1 && wgs64 <= 256) || (ntile == 2 && wgs64 >= 200 && wgs64 <= 256)) mrt = 1;
     mrt = env_int("WRQ_GEMM_MRT", mrt);
+    // K is split until there are one (narrow tiles) to four workgroups per CU, at most 8 ways; a group
+    // that fills most CUs unsplit stays unsplit (every split product costs a finish launch)
     const uint64_t wgs = (uint64_t)((rows + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
     const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
     uint32_t ksplit = 1;
-    while (wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
-    // A group of wide products that would be split although 64-row tiles, unsplit, fill the
-    // resident slots (two workgroups per CU) just once: take those (the four attention
-    // projections at 128 / 256 tokens: 512 workgroups, 7 - 12 % faster than 128-row tiles split 4 - 8 ways).
-    if (n >= 2 && ksplit > 1 && ntile >= 4) {
-        const int nt2 = T > 128 ? 8 : 4;
-        const uint64_t wgs2 = (uint64_t)((rows + 63) / 64) * ((T + 16 * nt2 - 1) / (16 * nt2)) * a.B;
-        if (wgs2 > 384 && wgs2 <= 512) mrt = 1, ntile = nt2, ksplit = 1;
-    }
-    mrt = env_int("WRQ_GEMM_MRT", mrt);
-    ntile = env_int("WRQ_GEMM_NTILE", ntile);
+    while (ksplit < 8 && wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
+    if (n >= 2 && wgs >= 200) ksplit = 1;
     ksplit = (uint32_t)env_int("WRQ_GEMM_KSPLIT", (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
