@@ -264,8 +264,24 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
                                      pack_h2(__uint_as_float(v1.z), __uint_as_float(v1.w)));
             }
         }
+        if constexpr (QUANT == kFp16) {
 #pragma unroll
-        for (int u = 0; u < KSUB; u++) st.sc[u] = QUANT == kFp16 ? 0u : sp[min(stage * KSUB + u, last)];
+            for (int u = 0; u < KSUB; u++) st.sc[u] = 0u;
+        } else {
+            // the scale words of a row's steps are adjacent: one 8- or 16-byte load per row and stage
+            // where the stage is whole and aligned (a load per word touches one line per row each time)
+            const uint32_t *q = sp + stage * KSUB;
+            if (KSUB == 4 && stage * KSUB + 3 <= last && (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+                const uint4 v = load128(q);
+                st.sc[0] = v.x; st.sc[KSUB > 1 ? 1 : 0] = v.y; st.sc[KSUB > 2 ? 2 : 0] = v.z; st.sc[KSUB > 3 ? 3 : 0] = v.w;
+            } else if (KSUB == 2 && stage * KSUB + 1 <= last && (reinterpret_cast<uintptr_t>(q) & 7) == 0) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(q);
+                st.sc[0] = v.x; st.sc[KSUB > 1 ? 1 : 0] = v.y;
+            } else {
+#pragma unroll
+                for (int u = 0; u < KSUB; u++) st.sc[u] = sp[min(stage * KSUB + u, last)];
+            }
+        }
     };
     auto store_stage = [&](const Stage &st, int buf) {
 #pragma unroll
