@@ -16,6 +16,10 @@
 //     operand serving MRT MFMAs;
 //   * weights are prefetched NBUF K steps ahead through a ring of register buffers, the
 //     next activation stage sits in registers while the current one is consumed from LDS;
+//   * token tiles up to 64 wide are bound by the vector memory path: their weight loads are
+//     line-wise (a row's bytes of a step in adjacent lanes, whole 128-byte lines per wave
+//     instruction) and pass through a wave-private LDS slot into the operand layout; only the
+//     128-token tile gathers the operand layout straight from memory (see Geometry);
 //   * the grid numbers workgroups so that the token blocks of one row tile run on one XCD
 //     (one L2) at about the same time: their weights cross HBM once;
 //   * K is split over workgroups (grid.y) only until there is about one workgroup per CU
