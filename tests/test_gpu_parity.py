@@ -294,15 +294,23 @@ def test_gemm_against_truth(gpu, oracle, kind, K, R, T):
         assert_close(got, ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
 
 
+# (MRT, NTILE, KG) instantiations of the chunk kernel: 64 * MRT / KG rows x 16 * NTILE tokens per
+# workgroup, KG k groups of waves that take alternate K steps
+TILE_VARIANTS = [(1, 1, 1), (1, 2, 1), (1, 4, 1), (1, 8, 1), (2, 1, 1), (2, 2, 1), (2, 4, 1), (2, 8, 1),
+                 (1, 1, 2), (1, 2, 2), (1, 4, 2), (2, 1, 2), (2, 2, 2), (2, 4, 2), (1, 1, 4), (1, 2, 4)]
+
+
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
-@pytest.mark.parametrize("mrt,ntile", [(1, 1), (1, 2), (1, 4), (1, 8), (2, 1), (2, 2), (2, 4), (2, 8)], ids=str)
-def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, monkeypatch):
+@pytest.mark.parametrize("mrt,ntile,kg", TILE_VARIANTS, ids=str)
+def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, kg, monkeypatch):
     # every tile instantiation of the chunk kernel, with and without split K, on a shape that
-    # leaves ragged edges everywhere: 5 steps of K (a partial stage), rows and tokens that do
-    # not fill the tiles.  WRQ_GEMM_* are the library's tuning overrides, read at every launch.
-    announce("chunk tile variant", kind, mrt, ntile)
+    # leaves ragged edges everywhere: 5 steps of K (a partial stage, fewer steps than some k
+    # groups get), rows and tokens that do not fill the tiles.  WRQ_GEMM_* are the library's
+    # tuning overrides, read at every launch.
+    announce("chunk tile variant", kind, mrt, ntile, kg)
     K, R, T = 640, 200, 40
-    rng = np.random.default_rng(SEED + 11 + mrt * 16 + ntile)
+    rng = np.random.default_rng(SEED + 11 + mrt * 16 + ntile + 64 * kg)
+    monkeypatch.setenv("WRQ_GEMM_KG", str(kg))
     w = gen_f16(rng, (R, K), 0.02)
     x = gen_f16(rng, (T, K), 1.0)
     wp, scale, wdeq = pack(oracle, kind, w)
@@ -314,9 +322,37 @@ def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, monkeypatch):
         monkeypatch.setenv("WRQ_GEMM_KSPLIT", str(ksplit))
         for out_dtype in (np.float16, np.float32):
             got = run(gpu, m, x, R, "mat", out_dtype, act=1)
-            assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"{kind} tile ({mrt},{ntile}) ksplit {ksplit}")
+            assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"{kind} tile ({mrt},{ntile},{kg}) ksplit {ksplit}")
         got32 = run(gpu, m, x.astype(np.float32), R, "mat", np.float32)
-        assert_close(got32, truth, EPS, f"{kind} tile ({mrt},{ntile}) ksplit {ksplit} f32 in")
+        assert_close(got32, truth, EPS, f"{kind} tile ({mrt},{ntile},{kg}) ksplit {ksplit} f32 in")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("T", [8, 24, 100, 200])
+def test_chunk_k_groups_by_default(gpu, oracle, kind, T):
+    # shapes that the tile choice sends to k groups without any override: a 4096-row product
+    # (nf4: k groups instead of a split of K) and groups of about 256 and 288 row tiles of 64
+    # at narrow token tiles (two k groups per workgroup)
+    import torch
+
+    announce("chunk k groups by default", kind, T)
+    rng = np.random.default_rng(SEED + 41 + T)
+    K = 1152
+    packed = {}
+    for R in (4096, 14336):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        packed[R] = (gpu_matrix(gpu, kind, wp, scale), wdeq)
+    x = gen_f16(rng, (T, K), 1.0)
+    m, wdeq = packed[4096]
+    assert_close(run(gpu, m, x, 4096, "mat", np.float32), truth_matmul(wdeq, x), EPS, f"{kind} 4096 rows T={T}")
+    for rows in ([4096] * 4, [14336, 4096]):
+        xs = [gen_f16(rng, (T, K), 1.0) for _ in rows]
+        xd = [dev(v) for v in xs]
+        outs = [torch.full((T, R), float("nan"), dtype=torch.float32, device="cuda") for R in rows]
+        gpu.matmul_vec_group([(packed[R][0], xv, o, gpu.ACT_NONE, False, {}) for R, xv, o in zip(rows, xd, outs)])
+        for R, xv, o in zip(rows, xs, outs):
+            assert_close(host(o), truth_matmul(packed[R][1], xv), EPS, f"{kind} group {rows} T={T}")
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])

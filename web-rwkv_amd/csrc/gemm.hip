@@ -7,8 +7,11 @@
 // The shapes of this path are skinny: 16..256 tokens against thousands of weight rows, so
 // even the chunk products are bound by streaming the packed weights once (below ~100
 // tokens) or sit close to that point.  The decomposition follows from it:
-//   * a workgroup (4 waves) owns 64*MRT weight rows x 16*NTILE tokens x one K range; wave w
-//     owns MRT row tiles of 16 as the MFMA "A" side.  Weight bytes go from HBM straight
+//   * a workgroup (4 waves) owns 64*MRT/KG weight rows x 16*NTILE tokens x one K range; a wave
+//     owns MRT row tiles of 16 as the MFMA "A" side, and with KG > 1 the waves form KG groups
+//     that share rows and activations and take alternate K steps (summed through LDS at the
+//     end): small grids get about two workgroups per CU from that instead of from a split
+//     of K over the grid.  Weight bytes go from HBM straight
 //     into registers of the one wave that uses them (each byte is read once and never
 //     shared, an LDS tile for them would only add traffic); the activation tile, shared by
 //     the four waves, is staged as f16 in double-buffered LDS, several K steps per barrier
@@ -90,35 +93,37 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// Tile geometry of one instantiation.  A workgroup has 4 * KG waves: 4 row groups times KG
-// "k groups" that share the staged activations and take alternate K steps, so that a CU holds
-// two waves per SIMD even when the grid gives it one workgroup; their partial tiles are
-// added through LDS at the end.  A stage is what one barrier covers: KSUB steps of 128 k of
-// the activation tile, so that narrow token tiles do not pay a barrier per 128 k.
-constexpr int KG = 1; // measured: a second k group (8 waves) gains nothing on these shapes
-template <int MRT, int NTILE>
+// Tile geometry of one instantiation.  The 4 waves of a workgroup are RW row groups times KG
+// "k groups": the k groups share the rows and the staged activations and take alternate K
+// steps; their partial tiles are added through LDS at the end.  Products with few rows get
+// their workgroups (about one per CU) from KG instead of from a split of K over the grid,
+// which would cost a round trip through the scratch array and a second launch.  A stage is
+// what one barrier covers: KSUB steps of 128 k of the activation tile, so that narrow token
+// tiles do not pay a barrier per 128 k.
+template <int MRT, int NTILE, int KG>
 struct Geometry {
-    static constexpr int THREADS = 256 * KG;
-    static constexpr int BN = 16 * NTILE; // tokens per workgroup
-    static constexpr int BM = 64 * MRT;   // weight rows per workgroup
+    static constexpr int THREADS = 256;
+    static constexpr int RW = 4 / KG;          // row groups: waves side by side along the rows
+    static constexpr int BN = 16 * NTILE;      // tokens per workgroup
+    static constexpr int BM = 16 * MRT * RW;   // weight rows per workgroup
     static constexpr int KSUB0 = (NTILE >= 8 ? 1 : NTILE == 4 ? 2 : 4) / MRT;
     static constexpr int KSUB = KSUB0 > KG ? KSUB0 : KG;                   // steps per stage
     static constexpr int LSUB = KSUB / KG;                                 // steps per stage and k group
     static constexpr int PITCH = kStep * KSUB + 8;                         // f16 per LDS row: +16 B rotates the banks
-    static constexpr int NPIECE = NTILE * KSUB / KG;                       // 16-byte activation pieces per thread and stage
+    static constexpr int NPIECE = NTILE * KSUB;                            // 16-byte activation pieces per thread and stage
     // weight steps in flight per wave: two stages (an even number of them), one for plain f16
     // weights, whose steps take twice the registers
     static constexpr int NBUFQ = (LSUB >= 2 || MRT >= 2) ? 2 * LSUB : 4;
     static constexpr int NBUFH = LSUB >= 2 ? LSUB : 2;
     static constexpr int nbuf(int quant) { return quant == kFp16 ? NBUFH : NBUFQ; }
-    static constexpr int TILE_FLOATS = 1024 * MRT * NTILE;                 // outputs of one workgroup
+    static constexpr int TILE_FLOATS = 256 * RW * MRT * NTILE;             // outputs of one workgroup
     // Token tiles up to 64 wide are bound by the vector memory path, not by arithmetic: a wave
     // instruction that gathers the A-operand layout straight from memory (16 rows x 64 B, or x 32 B
     // for nf4) costs the texture path about 54 clocks, three times a line-wise one.  There the weights
     // are fetched line-wise (a row's bytes of a step in adjacent lanes: 8 rows x 128 B per instruction
     // for int8, 16 x 64 B for nf4, 4 x 256 B for f16) and turned into the A-operand layout through a
     // wave-private LDS slot.  The widest tile keeps the direct gather: its LDS is the busiest unit.
-    static constexpr bool transposed_loads(int) { return NTILE <= 4 && KG == 1; }
+    static constexpr bool transposed_loads(int) { return NTILE <= 4; }
     static constexpr int wstep(int quant) { return quant == kFp16 ? 2 * kStep : quant == kInt8 ? kStep : kStep / 2; } // weight bytes per row and step
     static constexpr int tpitch(int quant) { return wstep(quant) + 16; }    // bytes per row of a slot: +16 B rotates the banks
     static constexpr size_t tslot_bytes(int quant) { return transposed_loads(quant) ? (size_t)4 * MRT * 16 * tpitch(quant) : 0; }
@@ -127,7 +132,7 @@ struct Geometry {
         return (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) + (size_t)2 * KSUB * BN * sizeof(float) +
                (quant == kNf4 ? 256 * sizeof(uint2) : 0) + tslot_bytes(quant);
     }
-    static_assert((size_t)4 * MRT * NTILE * 1024 <= (size_t)2 * BN * PITCH * sizeof(uint16_t), "partial tiles of a k group fit the activation buffers");
+    static_assert((size_t)(KG - 1) * RW * MRT * NTILE * 1024 <= (size_t)2 * BN * PITCH * sizeof(uint16_t), "partial tiles of the k groups fit the activation buffers");
 };
 
 // One launch serves up to kMaxGroup independent products with the same K, token count and
@@ -152,9 +157,9 @@ __device__ __forceinline__ void tile_of_block(uint32_t id, uint32_t tblocks, uin
     row_tile = (slot / tblocks) * 8u + xcd;
 }
 
-template <int QUANT, typename XT, int MRT, int NTILE>
-__global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
-    using G = Geometry<MRT, NTILE>;
+template <int QUANT, typename XT, int MRT, int NTILE, int KG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
+    using G = Geometry<MRT, NTILE, KG>;
     // the product of this workgroup: one scalar load of the tile starts, then its descriptor
     uint32_t pi = 0;
 #pragma unroll
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     const uint32_t tile_id = blockIdx.x - ga.tile_begin[pi];
     const uint32_t my_row_tiles = ga.row_tiles[pi];
     float *const my_scratch = ga.scratch[pi];
-    constexpr int BN = G::BN, BM = G::BM, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::nbuf(QUANT), THREADS = G::THREADS;
+    constexpr int BN = G::BN, BM = G::BM, RW = G::RW, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::nbuf(QUANT), THREADS = G::THREADS;
     constexpr int NW = QUANT == kFp16 ? 4 : QUANT == kInt8 ? 2 : 1;                        // 16-byte weight registers per row tile and step
     constexpr int WSTEP = QUANT == kFp16 ? 2 * kStep : QUANT == kInt8 ? kStep : kStep / 2; // weight bytes per row and step
     extern __shared__ __align__(16) uint8_t smem[];
@@ -184,8 +189,10 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
     tile_of_block(tile_id, ga.tblocks, row_tile, tblock);
     if (row_tile >= my_row_tiles) return; // padding of the XCD-aware grid
     const uint32_t tid = threadIdx.x, lane = tid & 63;
-    const uint32_t wave = (tid >> 6) & 3;                                        // row group of this wave
-    const uint32_t kg = KG == 1 ? 0u : __builtin_amdgcn_readfirstlane(tid >> 8); // its k group
+    // without k groups the k group is a compile-time zero: step offsets into LDS stay immediates
+    const uint32_t wv = KG == 1 ? ((tid >> 6) & 3) : __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wave = KG == 1 ? wv : wv % RW; // row group of this wave
+    const uint32_t kg = KG == 1 ? 0u : wv / RW;   // its k group
     const uint32_t r16 = lane & 15, g = lane >> 4;
     const uint32_t b = blockIdx.z;
     const uint32_t t0 = tblock * BN;
@@ -221,7 +228,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
                 wq[i][j] = (QUANT == kFp16 ? a.w + 2 * e : QUANT == kInt8 ? a.w + e : a.w + (e >> 1)) + 16 * (lane % LPR);
             }
     }
-    uint8_t *tslot = tslots + (size_t)wave * (MRT * 16 * TPITCH); // this wave's transposition slot
+    uint8_t *tslot = tslots + (size_t)wv * (MRT * 16 * TPITCH); // this wave's transposition slot
     // scale words (one 32-bit word per row and step for both formats: a (min, max) pair, or the
     // absmax of two 64-blocks): thread t < BM fetches those of workgroup row t
     const uint32_t *sp;
@@ -350,9 +357,13 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         for (int n = 0; n < NTILE; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
 
-    // one K step on the matrix cores: weights `cur` against step `sub` of the stage in LDS buffer `buf`.
-    // Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
-    auto compute = [&](const StepRegs &cur, int buf, uint32_t sub) {
+    // lane offsets into the staged tile, the row scales and the token sums; the k group of the wave is
+    // part of them, so that the step of a stage stays an immediate offset
+    const uint32_t xlane8 = r16 * PITCH + kg * kStep + 8 * g, xlane16 = r16 * PITCH + kg * kStep + 16 * g;
+    const uint32_t scl_lane = kg * BM + row_local + 4 * g, sxs_lane = kg * BN + r16;
+    // one K step on the matrix cores: weights `cur` against step `sub` (+ the k group) of the stage in
+    // LDS buffer `buf`.  Operand j of a step covers k = 64 (j / 2) + 16 g + 8 (j % 2) .. + 8
+    auto compute = [&](const StepRegs &cur, int buf, int sub) {
         // the step's packed weights of this lane in A-operand layout: as loaded, or line-wise loads
         // passed through the wave's LDS slot (one wave writes and reads a slot, in program order: no barrier)
         uint4 wa[MRT][NW];
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         }
         if constexpr (QUANT == kFp16) {
             // plain f16 weights are the A operands as loaded; the accumulators stay in the matrix cores
-            const uint16_t *xh = xs[buf] + r16 * PITCH + sub * kStep + 8 * g;
+            const uint16_t *xh = xs[buf] + sub * kStep + xlane8;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
 #pragma unroll
@@ -400,12 +411,12 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
             }
             return;
         }
-        const uint16_t *xt = xs[buf] + r16 * PITCH + sub * kStep + 16 * g;
+        const uint16_t *xt = xs[buf] + sub * kStep + xlane16;
         // scales of the 4 D-side rows of this lane, per row tile: (s, c) x 4 or (absmax0, absmax1) x 4
         float4 sc0[MRT], sc1[MRT];
 #pragma unroll
         for (int i = 0; i < MRT; i++) {
-            const float4 *q = reinterpret_cast<const float4 *>(&scl[buf][sub][row_local + 16 * i + 4 * g]);
+            const float4 *q = reinterpret_cast<const float4 *>(&scl[buf][sub][0] + scl_lane + 16 * i);
             sc0[i] = q[0];
             sc1[i] = q[1];
         }
@@ -433,7 +444,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                     for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, j == 0 ? zero4 : D[i], 0, 0, 0);
                 }
-                const float sx = sxs[buf][sub][n * 16 + r16];
+                const float sx = (&sxs[buf][sub][0])[sxs_lane + n * 16];
 #pragma unroll
                 for (int i = 0; i < MRT; i++) {
                     out[i][n][0] = fmaf(sc0[i].x, D[i][0], fmaf(sc0[i].y, sx, out[i][n][0]));
@@ -517,7 +528,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
                 const int sub = u * KG; // + kg: step of the stage taken by this k group
                 const int slot = (q * LSUB + u) % NBUF;
                 __builtin_amdgcn_sched_barrier(0); // steps do not interleave: one set of operand registers
-                if (S * KSUB + sub + kg < nsteps) compute(ring[slot], buf, sub + kg);
+                if (S * KSUB + sub + kg < nsteps) compute(ring[slot], buf, sub);
                 // refill the slot just consumed; the scheduling barrier keeps the loads below the
                 // last use of the old values, so they can target the same registers
                 __builtin_amdgcn_sched_barrier(0);
@@ -535,17 +546,20 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
             for (int i = 0; i < MRT; i++)
 #pragma unroll
                 for (int n = 0; n < NTILE; n++)
-                    red[((wave * MRT + i) * NTILE + n) * 64 + lane] = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
+                    red[((((kg - 1) * RW + wave) * MRT + i) * NTILE + n) * 64 + lane] =
+                        make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
         }
         lds_barrier();
         if (kg != 0) return;
 #pragma unroll
-        for (int i = 0; i < MRT; i++)
+        for (int q = 1; q < KG; q++)
 #pragma unroll
-            for (int n = 0; n < NTILE; n++) {
-                const float4 v = red[((wave * MRT + i) * NTILE + n) * 64 + lane];
-                out[i][n][0] += v.x; out[i][n][1] += v.y; out[i][n][2] += v.z; out[i][n][3] += v.w;
-            }
+            for (int i = 0; i < MRT; i++)
+#pragma unroll
+                for (int n = 0; n < NTILE; n++) {
+                    const float4 v = red[((((q - 1) * RW + wave) * MRT + i) * NTILE + n) * 64 + lane];
+                    out[i][n][0] += v.x; out[i][n][1] += v.y; out[i][n][2] += v.z; out[i][n][3] += v.w;
+                }
     }
 
     // D layout of a 16x16 tile: lane holds token column (lane & 15), rows 4 g .. 4 g + 3
@@ -553,7 +567,7 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
         // partial tile of this split, stored tile-major so that every store instruction writes
         // 1 KiB in one piece: [split][batch][workgroup][wave][i][n][lane][4]
         const uint32_t wg = tile_id, nwg = (my_row_tiles + 7) / 8 * 8 * ga.tblocks;
-        float *dst = my_scratch + ((((uint64_t)blockIdx.y * a.B + b) * nwg + wg) * (4 * MRT * NTILE) + wave * (MRT * NTILE)) * 256 + lane * 4;
+        float *dst = my_scratch + ((((uint64_t)blockIdx.y * a.B + b) * nwg + wg) * (RW * MRT * NTILE) + wave * (MRT * NTILE)) * 256 + lane * 4;
 #pragma unroll
         for (int i = 0; i < MRT; i++)
 #pragma unroll
@@ -589,20 +603,20 @@ __global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(2))) v
 // Second half of a split-K product: sum of the partial tiles over the splits, activation,
 // output type.  One thread per lane slot of the first kernel's tiles (same decoding).
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits, uint32_t nwg,
-                                                          uint32_t tblocks, uint32_t row_tiles, uint32_t mrt, uint32_t ntile) {
-    const uint32_t per_wg = 4 * mrt * ntile * 64; // lane slots per workgroup tile
+                                                          uint32_t tblocks, uint32_t row_tiles, uint32_t rw, uint32_t mrt, uint32_t ntile) {
+    const uint32_t per_wg = rw * mrt * ntile * 64; // lane slots per workgroup tile
     const uint64_t slots = (uint64_t)a.B * nwg * per_wg;
     const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (q >= slots) return;
     const uint32_t lane = (uint32_t)(q & 63), r16 = lane & 15, g = lane >> 4;
-    const uint32_t tp = (uint32_t)((q >> 6) % (4 * mrt * ntile));
+    const uint32_t tp = (uint32_t)((q >> 6) % (rw * mrt * ntile));
     const uint64_t bw = q / per_wg;
     const uint32_t wg = (uint32_t)(bw % nwg), b = (uint32_t)(bw / nwg);
     const uint32_t n = tp % ntile, wi = tp / ntile; // wi = wave * mrt + i
     uint32_t row_tile, tblock;
     tile_of_block(wg, tblocks, row_tile, tblock);
     if (row_tile >= row_tiles) return;
-    const uint32_t row = row_tile * 64 * mrt + wi * 16 + 4 * g;
+    const uint32_t row = row_tile * 16 * rw * mrt + wi * 16 + 4 * g;
     const uint32_t t = tblock * 16 * ntile + n * 16 + r16;
     if (t >= a.T || row >= a.R) return;
     const float *src = scratch + q * 4;
@@ -649,11 +663,11 @@ float *scratch_ptr() {
     return ptr[dev];
 }
 
-template <int QUANT, typename XT, int MRT, int NTILE>
+template <int QUANT, typename XT, int MRT, int NTILE, int KG>
 int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t ksplit) {
-    using G = Geometry<MRT, NTILE>;
+    using G = Geometry<MRT, NTILE, KG>;
     constexpr size_t lds = G::lds_bytes(QUANT);
-    auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE>;
+    auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE, KG>;
     if (lds > 48 * 1024) {
         // one-time opt-in to more than the default dynamic LDS limit
         static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -706,7 +720,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
         for (int i = 0; i < n; i++) {
             const uint64_t slots = slice[i] / 4;
             hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, args[i], ga.scratch[i], splits,
-                               nwg[i], ga.tblocks, ga.row_tiles[i], (uint32_t)MRT, (uint32_t)NTILE);
+                               nwg[i], ga.tblocks, ga.row_tiles[i], (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
         }
         s = check_launch("matmul_mat (finish)");
     }
@@ -729,30 +743,64 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
     const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
     int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192) ? 2 : (T > 64 && rt >= (1u << 23)) ? 8 : 4;
-    ntile = env_int("WRQ_GEMM_NTILE", ntile);
-    const uint32_t tblocks = (T + 16 * ntile - 1) / (16 * ntile);
+    int mrt = 2, kg = 1;
+    uint32_t ksplit = 1;
+    uint64_t wgs = 0; // workgroups of one split
+    auto tblocks_of = [&](int nt) { return (uint64_t)(T + 16 * nt - 1) / (16 * nt); };
+    // K is split over the grid until there are one (narrow tiles) to four workgroups per CU, at most
+    // 8 ways; a group that fills most CUs unsplit stays unsplit (every split product costs a finish launch)
+    auto split_for = [&]() {
+        wgs = (uint64_t)((rows * kg + 64 * mrt - 1) / (64 * mrt)) * tblocks_of(ntile) * a.B;
+        const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
+        ksplit = 1;
+        while (kg == 1 && ksplit < 8 && wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
+        if (n >= 2 && wgs >= 200) ksplit = 1;
+    };
     // 64-row tiles where they give about one workgroup per CU without a split of K (a 16-token tile:
     // also below that); otherwise 128-row tiles, fewer activation copies per weight byte, and more splits
-    int mrt = 2;
-    const uint64_t wgs64 = (uint64_t)((rows + 63) / 64) * tblocks * a.B;
+    const uint64_t wgs64 = (uint64_t)((rows + 63) / 64) * tblocks_of(ntile) * a.B;
     if ((ntile == 1 && wgs64 <= 256) || (ntile == 2 && wgs64 >= 200 && wgs64 <= 256)) mrt = 1;
+    if (QUANT != kFp16 && wgs64 >= 200 && wgs64 <= 320 && (ntile == 1 || (QUANT == kNf4 && ntile == 2))) {
+        // about one 64-row workgroup per CU at a narrow token tile: two workgroups of 32 rows with two
+        // k groups each keep twice the weight bytes in flight per CU
+        mrt = 1;
+        kg = 2;
+    }
+    if (QUANT == kNf4 && n == 1 && a.B == 1 && a.K <= 8192 && rows > 2048 && rows <= 4096) {
+        // a small single product gets its workgroups from k groups instead of a split over the grid
+        // (measured on 4096 x 4096: no scratch round trip, no finish launch)
+        ntile = T <= 16 ? 1 : 2;
+        mrt = T > 128 ? 2 : 1;
+        kg = T <= 32 ? 4 : 2;
+    }
+    split_for();
+    if (QUANT == kInt8 && kg == 1 && T > 64) {
+        // two workgroups fit a CU (512 slots).  A grid of 64-token tiles that fills half of them runs at
+        // one wave per SIMD: 32-token tiles double it.
+        if (ntile == 4 && wgs * ksplit <= 256) {
+            ntile = 2;
+            split_for();
+        }
+    }
+    ntile = env_int("WRQ_GEMM_NTILE", ntile);
     mrt = env_int("WRQ_GEMM_MRT", mrt);
-    // K is split until there are one (narrow tiles) to four workgroups per CU, at most 8 ways; a group
-    // that fills most CUs unsplit stays unsplit (every split product costs a finish launch)
-    const uint64_t wgs = (uint64_t)((rows + 64 * mrt - 1) / (64 * mrt)) * tblocks * a.B;
-    const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
-    uint32_t ksplit = 1;
-    while (ksplit < 8 && wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
-    if (n >= 2 && wgs >= 200) ksplit = 1;
+    kg = env_int("WRQ_GEMM_KG", kg);
+    if (kg != 1 && kg != 2 && kg != 4) kg = 1;
+    if (kg == 4 && (mrt != 1 || ntile > 2)) kg = 2;
+    if (kg == 2 && ntile > 4) kg = 1;
+    if (getenv("WRQ_GEMM_NTILE") || getenv("WRQ_GEMM_MRT") || getenv("WRQ_GEMM_KG")) split_for();
     ksplit = (uint32_t)env_int("WRQ_GEMM_KSPLIT", (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
-#define WRQ_CASE(M, N) \
-    if (mrt == M && ntile == N) return launch_one<QUANT, XT, M, N>(stream, args, n, ksplit);
-    WRQ_CASE(1, 1) WRQ_CASE(1, 2) WRQ_CASE(1, 4) WRQ_CASE(1, 8)
-    WRQ_CASE(2, 1) WRQ_CASE(2, 2) WRQ_CASE(2, 4) WRQ_CASE(2, 8)
+#define WRQ_CASE(M, N, G) \
+    if (mrt == M && ntile == N && kg == G) return launch_one<QUANT, XT, M, N, G>(stream, args, n, ksplit);
+    WRQ_CASE(1, 1, 1) WRQ_CASE(1, 2, 1) WRQ_CASE(1, 4, 1) WRQ_CASE(1, 8, 1)
+    WRQ_CASE(2, 1, 1) WRQ_CASE(2, 2, 1) WRQ_CASE(2, 4, 1) WRQ_CASE(2, 8, 1)
+    WRQ_CASE(1, 1, 2) WRQ_CASE(1, 2, 2) WRQ_CASE(1, 4, 2)
+    WRQ_CASE(2, 1, 2) WRQ_CASE(2, 2, 2) WRQ_CASE(2, 4, 2)
+    WRQ_CASE(1, 1, 4) WRQ_CASE(1, 2, 4)
 #undef WRQ_CASE
-    return launch_one<QUANT, XT, 1, 2>(stream, args, n, ksplit);
+    return launch_one<QUANT, XT, 1, 2, 1>(stream, args, n, ksplit);
 }
 
 } // namespace
