@@ -62,7 +62,7 @@ def test_oracle_against_exact_fixtures(oracle, c):
     check_packing(c, p, s)
     if not c["sensitive"]:  # products of the exact codes: comparable when no code is ambiguous
         assert_close(out, np.array(c["product_f64"]), EPS, "vec vs exact product")
-        if c["T"] % 4 == 0:  # the mat entry points take multiples of 4 tokens (ops.rs:1088, 1166)
+        if c["T"] % 4 == 0:  # the mat entry points take multiples of 4 tokens (ops.rs:1068-1070, 1146-1149)
             assert_close(mat, np.array(c["product_f64"]), EPS, "mat vs exact product")
     else:
         assert_close(out, np.array(c["product_f64"]), 5e-3, "vec vs exact product (codes within 1 at boundaries)")
