@@ -205,6 +205,35 @@ int wrq_matmul_vec_fp16(wrq_stream stream, const wrq_tensor *matrix, const wrq_t
 int wrq_matmul_mat_fp16(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor_view *input,
                         const wrq_tensor_view *output, int act);
 
+/*
+ * The ops between the matrix products of a layer.  Tensors are in place, rows of 4-element units
+ * as in the shaders (row length % 4 == 0); `dtype` is the element type of `x`.
+ *
+ * TensorOp::softmax(x)                      src/tensor/ops.rs:300-347, src/shaders/softmax.wgsl
+ *   x [C, T, B, 1]: every row of C elements becomes exp(x - max) / sum.
+ * TensorOp::layer_norm(w, b, x, eps)        src/tensor/ops.rs:407-458, src/shaders/layer_norm.wgsl
+ *   x [C, T, B, 1]; w, b f16 [C, 1, 1, 1]: (x - mean) / sqrt(var + eps) * w + b, biased variance.
+ * TensorOp::group_norm(w, b, x, eps)        src/tensor/ops.rs:460-509 (the same shader, GROUP_NORM)
+ *   x [S, H, A, 1]; w, b f16 [S, H, 1, 1]: the same per row of S elements, head h uses w[.., h].
+ */
+int wrq_softmax(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype);
+int wrq_layer_norm(wrq_stream stream, const wrq_tensor *w, const wrq_tensor *b, const wrq_tensor *x,
+                   wrq_dtype dtype, float eps);
+int wrq_group_norm(wrq_stream stream, const wrq_tensor *w, const wrq_tensor *b, const wrq_tensor *x,
+                   wrq_dtype dtype, float eps);
+
+/*
+ * TensorOp::add_activate / mul_activate(input, output, act_x, act_y, act_out)
+ *                                           src/tensor/ops.rs:1227-1391, src/shaders/binary.wgsl
+ *   output [C, T, B, 1] = act_out(act_x(input) + act_y(output))   (mul: the product);
+ *   input [C, T, B, 1], [C, T, 1, B], [C, 1, B, 1] or [C, 1, 1, 1]: an extent of 1 is broadcast.
+ *   TensorOp::add / mul are these with WRQ_ACT_NONE three times.
+ */
+int wrq_add_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output,
+                     int act_x, int act_y, int act_out);
+int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output,
+                     int act_x, int act_y, int act_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,142 @@
+"""CPU restatement (numpy, f32) of the shaders of the ops between the matrix products.
+
+TEST INFRASTRUCTURE ONLY: tests/ and nothing else import this; the library never does.
+
+Each function follows its shader lane by lane: a workgroup of BLOCK_SIZE threads, each thread a
+`vec4<f32>` lane group, strided over the row, then the shader's tree over the threads.
+  softmax                 src/shaders/softmax.wgsl:52-110           (BLOCK_SIZE 128, ops.rs:301)
+  layer_norm, group_norm  src/shaders/layer_norm.wgsl:27-120        (128 / 32, ops.rs:415, :468)
+  add / mul + activations src/shaders/binary.wgsl:36-77, activations src/tensor/ops.rs:205-233
+What pins them: the closed forms of the reference's own tests (softmax ops.rs:2655-2662, layer
+norm ops.rs:2726-2746: sequential Welford) and float64 textbook forms, in tests/test_layer_ops.py.
+Parity unpinned: group_norm's tree starts at a stride (64) beyond its 32 threads; the reads past
+the workgroup arrays are taken to find zero counts (nothing merged), which only a run of the
+reference could confirm.  f16 rounding of results: round to nearest even (numpy), as for the
+matrix products.
+"""
+import numpy as np
+
+F = np.float32
+
+
+def _rows(x):
+    """(..., C) array -> (rows, C) f32 copy."""
+    a = np.asarray(x)
+    return a.reshape(-1, a.shape[-1]).astype(F), a.shape, a.dtype
+
+
+def _lanes(row, block):
+    """Row of C elements -> [iterations, block, 4] vectors as thread `index` meets them
+    (`for i = index; i < stride; i += BLOCK_SIZE`), and the validity of every slot."""
+    nv = row.size // 4
+    iters = (nv + block - 1) // block
+    v = np.zeros((iters * block, 4), dtype=F)
+    ok = np.zeros(iters * block, dtype=bool)
+    v[:nv] = row.reshape(nv, 4)
+    ok[:nv] = True
+    return v.reshape(iters, block, 4), ok.reshape(iters, block)
+
+
+def softmax(x, block=128):
+    rows, shape, dt = _rows(x)
+    out = np.empty_like(rows)
+    for r, row in enumerate(rows):
+        v, ok = _lanes(row, block)
+        mx = np.full((block, 4), F(-1.0e30))
+        for it in range(v.shape[0]):
+            mx = np.where(ok[it][:, None], np.maximum(mx, v[it]), mx)
+        s = 64
+        while s >= 1:  # reduce_max(index, 64 .. 1)
+            if s < block:
+                mx[:s] = np.maximum(mx[:s], mx[s:2 * s])
+            s //= 2
+        m = F(max(mx[0]))
+        sm = np.zeros((block, 4), dtype=F)
+        for it in range(v.shape[0]):
+            sm = np.where(ok[it][:, None], sm + np.exp(v[it] - m, dtype=F), sm)
+        s = 64
+        while s >= 1:
+            if s < block:
+                sm[:s] = sm[:s] + sm[s:2 * s]
+            s //= 2
+        total = F(((sm[0][0] + sm[0][1]) + sm[0][2]) + sm[0][3])  # dot(sketch[0], 1)
+        out[r] = np.exp(row - m, dtype=F) / total
+    return out.reshape(shape).astype(dt)
+
+
+def layer_norm(w, b, x, eps, block=128, group=False):
+    """x (..., C); w, b (C,) f16 -- or, group norm, x (A, H, S), w, b (H, S)."""
+    rows, shape, dt = _rows(x)
+    out = np.empty_like(rows)
+    wf = np.asarray(w).astype(F).reshape(-1, rows.shape[1])
+    bf = np.asarray(b).astype(F).reshape(-1, rows.shape[1])
+    n = F(rows.shape[1])
+    for r, row in enumerate(rows):
+        v, ok = _lanes(row, block)
+        mu = np.zeros((block, 4), dtype=F)
+        m2 = np.zeros((block, 4), dtype=F)
+        cnt = np.zeros((block, 4), dtype=np.uint32)
+        for it in range(v.shape[0]):  # per-lane Welford
+            k = ok[it][:, None]
+            delta = v[it] - mu
+            c1 = cnt + np.uint32(1)
+            with np.errstate(divide="ignore", invalid="ignore"):
+                mu1 = mu + delta / c1.astype(F)
+            m21 = m2 + delta * (v[it] - mu1)
+            cnt, mu, m2 = np.where(k, c1, cnt), np.where(k, mu1, mu), np.where(k, m21, m2)
+        s = 64
+        while s >= 1:  # reduce_step(index, 64 .. 1); strides beyond the workgroup merge nothing
+            if s < block:
+                mu1, mu2, c1, c2 = mu[:s], mu[s:2 * s], cnt[:s], cnt[s:2 * s]
+                delta = mu2 - mu1
+                tot = c1 + c2
+                with np.errstate(divide="ignore", invalid="ignore"):
+                    nm = (mu1 * c1.astype(F) + mu2 * c2.astype(F)) / tot.astype(F)
+                    n2 = m2[:s] + m2[s:2 * s] + delta * delta * (c1 * c2).astype(F) / tot.astype(F)
+                mu[:s] = np.where(tot > 0, nm, F(0))
+                m2[:s] = np.where(tot > 0, n2, F(0))
+                cnt[:s] = tot
+            s //= 2
+        c0 = cnt[0].astype(F)
+        mean = F(np.dot(mu[0], c0 / n))
+        d = mu[0] - mean
+        var = F((F(m2[0].sum(dtype=F)) + F(np.dot(d * d, c0))) / n + F(eps))
+        dev = F(1.0) / np.sqrt(var, dtype=F)
+        h = r % wf.shape[0] if group else 0
+        out[r] = ((row - mean) * dev) * wf[h] + bf[h]
+    return out.reshape(shape).astype(dt)
+
+
+def group_norm(w, b, x, eps):
+    return layer_norm(w, b, x, eps, block=32, group=True)
+
+
+def activation(act, x):
+    """Activation::{None, SquaredRelu, Tanh, StableExp, OppositeExp, Softplus, Sigmoid, Silu} on f32."""
+    x = np.asarray(x, dtype=F)
+    with np.errstate(over="ignore"):
+        if act == 0:
+            return x
+        if act == 1:
+            p = np.maximum(x, F(0))
+            return p * p
+        if act == 2:
+            return np.where(x > F(42), F(1), np.tanh(x, dtype=F))
+        if act == 3:
+            return np.exp(-np.exp(x, dtype=F), dtype=F)
+        if act == 4:
+            return -np.exp(x, dtype=F)
+        if act == 5:
+            return np.log(F(1) + np.exp(x, dtype=F), dtype=F)
+        if act == 6:
+            return F(1) / (F(1) + np.exp(-x, dtype=F))
+        if act == 7:
+            return x / (F(1) + np.exp(-x, dtype=F))
+    raise ValueError(act)
+
+
+def binary(op, x, y, act_x=0, act_y=0, act_out=0):
+    """ACT_OUT(ACT_X(x) op ACT_Y(y)) with numpy broadcasting of x; result in y's type."""
+    a, c = activation(act_x, np.asarray(x).astype(F)), activation(act_y, np.asarray(y).astype(F))
+    r = activation(act_out, a * c if op == "mul" else a + c)
+    return r.astype(np.asarray(y).dtype)

@@ -1,0 +1,193 @@
+"""The ops between the matrix products: oracle against the closed forms of the reference's own
+tests and float64, and -- marked gpu -- the library against the oracle through the C ABI."""
+import importlib
+import os
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import assert_close
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SEED = 0x57525200
+
+
+@pytest.fixture(scope="module")
+def lop():
+    sys.path.insert(0, ROOT)
+    return importlib.import_module("oracle.layer_ops")
+
+
+def softmax64(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+def layer_norm64(w, b, x, eps):
+    x = x.astype(np.float64)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    return (x - mean) / np.sqrt(var + eps) * w.astype(np.float64) + b.astype(np.float64)
+
+
+def layer_norm_reference_test_form(w, b, x, eps):
+    """ops.rs:2726-2746: sequential f32 Welford over the row, then (x - mean) * deviation * w + b."""
+    out = np.empty(x.shape, dtype=np.float32)
+    for r, row in enumerate(x.reshape(-1, x.shape[-1]).astype(np.float32)):
+        mean, m2 = np.float32(0), np.float32(0)
+        for count, v in enumerate(row, start=1):
+            delta = v - mean
+            mean = np.float32(mean + delta / np.float32(count))
+            m2 = np.float32(m2 + delta * (v - mean))
+        dev = np.float32(1.0) / np.sqrt(np.float32(m2 / np.float32(row.size) + np.float32(eps)))
+        out.reshape(-1, x.shape[-1])[r] = (row - mean) * dev * w.astype(np.float32) + b.astype(np.float32)
+    return out
+
+
+def reference_test_inputs(rng, C=1000, T=3, B=2):
+    """the shapes and distributions of test_softmax / test_layer_norm (ops.rs:2636-2646, :2677-2697)"""
+    x = (10.0 * (rng.random((B, T, C), dtype=np.float32) - 0.5)).astype(np.float32)
+    w = (rng.random(C, dtype=np.float32) - 0.5).astype(np.float16)
+    b = (rng.random(C, dtype=np.float32) - 0.5).astype(np.float16)
+    return x, w, b
+
+
+def test_oracle_softmax(lop):
+    rng = np.random.default_rng(SEED + 1)
+    x, _, _ = reference_test_inputs(rng)
+    got = lop.softmax(x)
+    assert_close(got, softmax64(x), 1e-6, "softmax vs float64")
+    assert np.allclose(got.sum(axis=-1), 1.0, atol=1e-5)
+    # invariances of the definition: a shift of the row changes nothing, a constant row is uniform
+    assert_close(lop.softmax(x + np.float32(3.0)), got, 1e-5, "shift invariance")
+    assert_close(lop.softmax(np.full((2, 64), 7.0, dtype=np.float32)), np.full((2, 64), 1 / 64), 1e-6, "constant row")
+    h = lop.softmax(x.astype(np.float16))
+    assert h.dtype == np.float16
+    assert_close(h, softmax64(x.astype(np.float16)), 1e-3, "f16 rows")
+
+
+@pytest.mark.parametrize("C", [1000, 4096, 64, 4])
+def test_oracle_layer_norm(lop, C):
+    rng = np.random.default_rng(SEED + 2 + C)
+    x, w, b = reference_test_inputs(rng, C=C)
+    got = lop.layer_norm(w, b, x, 1e-5)
+    assert_close(got, layer_norm64(w, b, x, 1e-5), 1e-4, "vs float64")
+    if C <= 1000:
+        assert_close(got, layer_norm_reference_test_form(w, b, x, 1e-5), 1e-3, "vs the reference test's sequential form")  # its own bar
+    # a dropped bias, a missing eps or the unbiased variance would show here
+    one, zero = np.ones(C, dtype=np.float16), np.zeros(C, dtype=np.float16)
+    y = lop.layer_norm(one, zero, x, 0.0).astype(np.float64)
+    assert np.allclose(y.mean(axis=-1), 0.0, atol=1e-5) and np.allclose((y ** 2).mean(axis=-1), 1.0, atol=1e-4)
+    big = lop.layer_norm(one, zero, np.full((1, C), 5.0, dtype=np.float32), 1e-5)
+    assert np.all(big == 0.0)  # zero variance: eps keeps the division finite
+
+
+def test_oracle_group_norm(lop):
+    rng = np.random.default_rng(SEED + 3)
+    A, H, S = 5, 8, 64
+    x = (4.0 * rng.standard_normal((A, H, S))).astype(np.float32)
+    w = rng.standard_normal((H, S)).astype(np.float16)
+    b = rng.standard_normal((H, S)).astype(np.float16)
+    got = lop.group_norm(w, b, x, 64e-5)
+    assert_close(got, layer_norm64(w[None], b[None], x, 64e-5), 1e-4, "vs float64, per head")
+    # heads must not share weights: permuting the heads of x, w and b together permutes the result
+    p = rng.permutation(H)
+    assert_close(lop.group_norm(w[p], b[p], x[:, p], 64e-5), got[:, p], 1e-6, "head permutation")
+
+
+@pytest.mark.parametrize("op", ["add", "mul"])
+def test_oracle_binary(lop, op):
+    rng = np.random.default_rng(SEED + 4)
+    x = rng.standard_normal((2, 3, 64)).astype(np.float16)
+    y = rng.standard_normal((2, 3, 64)).astype(np.float32)
+    f = (lambda a, c: a * c) if op == "mul" else (lambda a, c: a + c)
+    assert_close(lop.binary(op, x, y), f(x.astype(np.float64), y.astype(np.float64)), 1e-6, "plain")
+    # the gate of the attention output (v6.rs:881-887): silu(g) * x
+    g = x.astype(np.float64)
+    want = g / (1 + np.exp(-g)) * y if op == "mul" else g / (1 + np.exp(-g)) + y
+    assert_close(lop.binary(op, x, y, act_x=7), want, 1e-6, "silu on the input")
+    # broadcast of a [C, 1, 1] input, the closed forms of every activation at known points
+    assert_close(lop.binary(op, x[0, 0], y), f(x[0, 0].astype(np.float64), y.astype(np.float64)), 1e-6, "broadcast")
+    pts = np.array([-2.0, 0.0, 0.5, 50.0], dtype=np.float32)
+    want = {1: [0, 0, 0.25, 2500], 2: [np.tanh(-2), 0, np.tanh(0.5), 1], 3: [np.exp(-np.exp(-2)), np.exp(-1), np.exp(-np.exp(0.5)), 0],
+            4: [-np.exp(-2), -1, -np.exp(0.5), -np.exp(50)], 5: [np.log1p(np.exp(-2)), np.log(2), np.log1p(np.exp(0.5)), 50],
+            6: [1 / (1 + np.exp(2)), 0.5, 1 / (1 + np.exp(-0.5)), 1], 7: [-2 / (1 + np.exp(2)), 0, 0.5 / (1 + np.exp(-0.5)), 50]}
+    for act, w in want.items():
+        assert_close(lop.activation(act, pts), np.array(w, dtype=np.float64), 1e-6, f"activation {act}")
+
+
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("C,T,B", [(1000, 3, 2), (4096, 1, 1), (4096, 128, 1), (65536, 2, 1), (64, 5, 1), (4, 1, 3)])
+def test_gpu_softmax_layer_norm(gpu, lop, dtype, C, T, B):
+    import torch
+
+    print("softmax / layer norm on the GPU", dtype.__name__, C, T, B, flush=True)
+    rng = np.random.default_rng(SEED + 10 + C + T)
+    x, w, b = reference_test_inputs(rng, C=C, T=T, B=B)
+    x = x.astype(dtype)
+    eps_out = 1e-3 if dtype == np.float16 else 2e-5
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.softmax(xd)
+    if T * C <= 20000:
+        assert_close(xd.cpu().numpy(), lop.softmax(x), eps_out if dtype == np.float16 else 1e-6, "softmax vs oracle")
+    assert_close(xd.cpu().numpy(), softmax64(x), eps_out if dtype == np.float16 else 1e-6, "softmax vs float64")
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.layer_norm(torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda(), xd, 1e-5)
+    if T * C <= 20000:
+        assert_close(xd.cpu().numpy(), lop.layer_norm(w, b, x, 1e-5), eps_out * 2, "layer norm vs oracle")
+    assert_close(xd.cpu().numpy(), layer_norm64(w, b, x, 1e-5), 1e-3, "layer norm vs float64")  # the reference's bar (ops.rs:2750)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("A,H,S", [(1, 64, 64), (33, 64, 64), (4, 32, 128), (2, 3, 2048)])
+def test_gpu_group_norm(gpu, lop, dtype, A, H, S):
+    import torch
+
+    print("group norm on the GPU", dtype.__name__, A, H, S, flush=True)
+    rng = np.random.default_rng(SEED + 20 + A + S)
+    x = (4.0 * rng.standard_normal((A, H, S))).astype(dtype)
+    w = rng.standard_normal((H, S)).astype(np.float16)
+    b = rng.standard_normal((H, S)).astype(np.float16)
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.group_norm(torch.from_numpy(w).cuda(), torch.from_numpy(b).cuda(), xd, 64e-5)
+    eps = 2e-3 if dtype == np.float16 else 1e-4
+    if A * H * S <= 20000:
+        assert_close(xd.cpu().numpy(), lop.group_norm(w, b, x, 64e-5), eps, "vs oracle")
+    assert_close(xd.cpu().numpy(), layer_norm64(w[None], b[None], x, 64e-5), max(eps, 1e-3), "vs float64")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op", ["add", "mul"])
+def test_gpu_binary(gpu, lop, op):
+    import torch
+
+    print("binary ops on the GPU", op, flush=True)
+    rng = np.random.default_rng(SEED + 30)
+    C, T, B = 256, 5, 2
+    fn = gpu.LayerOp.mul_activate if op == "mul" else gpu.LayerOp.add_activate
+    for it, ot in ((np.float16, np.float32), (np.float32, np.float16), (np.float16, np.float16), (np.float32, np.float32)):
+        y = rng.standard_normal((B, T, C)).astype(ot)
+        for xs in ((B, T, C), (B, 1, C), (1, 1, C)):
+            x = rng.standard_normal(xs).astype(it)
+            for acts in ((0, 0, 0), (7, 0, 0), (2, 6, 1), (0, 3, 5)):
+                yd = torch.from_numpy(y.copy()).cuda()
+                fn(torch.from_numpy(x).cuda(), yd, *acts)
+                want = lop.binary(op, lop.activation(acts[0], x.astype(np.float32)), lop.activation(acts[1], y.astype(np.float32)))
+                want = lop.activation(acts[2], want.astype(np.float32)).astype(ot)
+                assert_close(yd.cpu().numpy(), want, 2e-3 if ot == np.float16 else 1e-5, f"{op} {it.__name__}->{ot.__name__} {xs} {acts}")
+    # views: the input is slice 2 of a [C, T, 5] stack, the output rows 1..3 of a taller tensor
+    stack = rng.standard_normal((5, T, C)).astype(np.float16)
+    tall = rng.standard_normal((1, T + 2, C)).astype(np.float32)
+    td = torch.from_numpy(tall.copy()).cuda()
+    fn(torch.from_numpy(stack).cuda(), td, 0, 0, 0, input_view=((C, T, 1), (C, T, 5), (0, 0, 2)), output_view=((C, T, 1), (C, T + 2, 1), (0, 1, 0)))
+    want = tall.copy()
+    want[0, 1:T + 1] = lop.binary(op, stack[2], tall[0, 1:T + 1])
+    assert_close(td.cpu().numpy(), want, 1e-5, "views")
+    # the constructor's shape rule
+    with pytest.raises(gpu.TensorError):
+        fn(torch.zeros((B, T, C // 2), dtype=torch.float16, device="cuda"), torch.zeros((B, T, C), dtype=torch.float16, device="cuda"))

@@ -41,6 +41,7 @@ EXPORTS = [
     "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
+    "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
 ]
 MAX_GROUP = 8
 
@@ -181,6 +182,11 @@ def lib():
         L.wrq_matmul_mat_fp16.argtypes = [vp, V, V, V, i]
         L.wrq_matmul_vec_int8_group.argtypes = [vp, C.POINTER(CVecInt8Op), i]
         L.wrq_matmul_vec_nf4_group.argtypes = [vp, C.POINTER(CVecNf4Op), i]
+        L.wrq_softmax.argtypes = [vp, T, i]
+        L.wrq_layer_norm.argtypes = [vp, T, T, T, i, C.c_float]
+        L.wrq_group_norm.argtypes = [vp, T, T, T, i, C.c_float]
+        L.wrq_add_activate.argtypes = [vp, V, V, i, i, i]
+        L.wrq_mul_activate.argtypes = [vp, V, V, i, i, i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -275,6 +281,34 @@ class TensorOp:
     def matmul_mat_fp16(matrix, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
         _check(lib().wrq_matmul_mat_fp16(_stream(), C.byref(as_view(matrix, matrix_view)), C.byref(as_view(input, input_view)),
                                          C.byref(as_view(output, output_view)), act))
+
+
+class LayerOp:
+    """The row-wise and element-wise ops between the matrix products (src/tensor/ops.rs:300-509,
+    :1227-1391); each enqueues on torch's current stream and works in place like the reference."""
+
+    @staticmethod
+    def softmax(x):
+        _check(lib().wrq_softmax(_stream(), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def layer_norm(w, b, x, eps):
+        _check(lib().wrq_layer_norm(_stream(), C.byref(as_tensor(w)), C.byref(as_tensor(b)), C.byref(as_tensor(x)), _dtype(x), eps))
+
+    @staticmethod
+    def group_norm(w, b, x, eps):
+        _check(lib().wrq_group_norm(_stream(), C.byref(as_tensor(w)), C.byref(as_tensor(b)), C.byref(as_tensor(x)), _dtype(x), eps))
+
+    @staticmethod
+    def add_activate(input, output, act_x=ACT_NONE, act_y=ACT_NONE, act_out=ACT_NONE, input_view=None, output_view=None):
+        _check(lib().wrq_add_activate(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act_x, act_y, act_out))
+
+    @staticmethod
+    def mul_activate(input, output, act_x=ACT_NONE, act_y=ACT_NONE, act_out=ACT_NONE, input_view=None, output_view=None):
+        _check(lib().wrq_mul_activate(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act_x, act_y, act_out))
+
+    add = add_activate
+    mul = mul_activate
 
 
 def matmul_vec_group(ops):

@@ -1,0 +1,275 @@
+// Row-wise and element-wise ops that sit between the matrix products of a layer:
+//   softmax                 src/tensor/ops.rs:300-347,   src/shaders/softmax.wgsl
+//   layer_norm, group_norm  src/tensor/ops.rs:407-509,   src/shaders/layer_norm.wgsl
+//   add / mul (+activations) src/tensor/ops.rs:1227-1391, src/shaders/binary.wgsl
+//
+// All are bound by memory latency, not bandwidth, at the sizes of this path (a row is 2 - 16 KiB, a
+// run has 1 - 256 rows): one workgroup per row keeps the row in registers between the statistics
+// and the write-back where it fits (one read, one write per element), reductions go through DPP and
+// one LDS exchange, every access is a whole 8- or 16-byte vector of 4 elements as in the shaders.
+// The statistics are two-pass (mean, then the sum of squared deviations) in f32: the shaders merge
+// per-lane Welford states; both agree with the exact value far inside the reference's 1e-3 test bar.
+#include "wrq_device.h"
+#include "wrq_host.h"
+
+namespace wrq {
+
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kRowCache = 8; // vectors of 4 elements a thread keeps: rows up to 8192 elements stay in registers
+
+template <typename XT>
+__device__ __forceinline__ float4 load_vec4(const XT *p) {
+    if constexpr (sizeof(XT) == 2) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
+    } else {
+        return *reinterpret_cast<const float4 *>(p);
+    }
+}
+
+template <typename XT>
+__device__ __forceinline__ void store_vec4(XT *p, float4 v) {
+    if constexpr (sizeof(XT) == 2) {
+        *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f2h(v.x) | ((uint32_t)f2h(v.y) << 16), (uint32_t)f2h(v.z) | ((uint32_t)f2h(v.w) << 16));
+    } else {
+        *reinterpret_cast<float4 *>(p) = v;
+    }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// sum or maximum over the workgroup, the same value in every thread
+template <bool MAX, int THREADS>
+__device__ __forceinline__ float block_reduce(float v, float *red) {
+    v = MAX ? wave_max(v) : wave_sum(v);
+    if constexpr (THREADS == 64) return v;
+    const uint32_t wave = threadIdx.x >> 6;
+    __syncthreads(); // `red` may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; w++) r = MAX ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+}
+
+// One workgroup per row of `n` elements (n % 4 == 0).  MODE 0: softmax; 1: layer norm (w, b of the
+// row's length); 2: group norm (w, b indexed by head * n, the row index modulo `heads`).
+template <typename XT, int MODE, int THREADS>
+__global__ __launch_bounds__(THREADS) void row_kernel(XT *x, const uint16_t *w, const uint16_t *b, uint32_t n, uint32_t heads, float eps) {
+    __shared__ float red[THREADS / 64];
+    XT *row = x + (uint64_t)blockIdx.x * n;
+    const uint32_t nv = n / 4;
+    float4 cache[kRowCache];
+    const bool cached = nv <= (uint32_t)(THREADS * kRowCache);
+    // pass 1: the row into registers (or a first reading), maximum / sum
+    float part = MODE == 0 ? -1.0e30f : 0.0f;
+    if (cached) {
+#pragma unroll
+        for (int c = 0; c < kRowCache; c++) {
+            const uint32_t i = threadIdx.x + c * THREADS;
+            if (i < nv) {
+                cache[c] = load_vec4(row + 4 * i);
+                if (MODE == 0) part = fmaxf(part, fmaxf(fmaxf(cache[c].x, cache[c].y), fmaxf(cache[c].z, cache[c].w)));
+                else part += (cache[c].x + cache[c].y) + (cache[c].z + cache[c].w);
+            }
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < nv; i += THREADS) {
+            const float4 v = load_vec4(row + 4 * i);
+            if (MODE == 0) part = fmaxf(part, fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
+            else part += (v.x + v.y) + (v.z + v.w);
+        }
+    }
+    const float first = block_reduce<MODE == 0, THREADS>(part, red); // maximum, or the sum
+    const float centre = MODE == 0 ? first : first / (float)n;
+    // pass 2: sum of exp(x - max), or of squared deviations
+    float acc = 0.0f;
+    auto term = [&](float v) { return MODE == 0 ? expf(v - centre) : (v - centre) * (v - centre); };
+    if (cached) {
+#pragma unroll
+        for (int c = 0; c < kRowCache; c++)
+            if (threadIdx.x + c * THREADS < nv) acc += (term(cache[c].x) + term(cache[c].y)) + (term(cache[c].z) + term(cache[c].w));
+    } else {
+        for (uint32_t i = threadIdx.x; i < nv; i += THREADS) {
+            const float4 v = load_vec4(row + 4 * i);
+            acc += (term(v.x) + term(v.y)) + (term(v.z) + term(v.w));
+        }
+    }
+    const float total = block_reduce<false, THREADS>(acc, red);
+    const float scale = MODE == 0 ? 1.0f / total : rsqrtf(total / (float)n + eps);
+    const uint16_t *wr = MODE == 2 ? w + (uint64_t)(blockIdx.x % heads) * n : w;
+    const uint16_t *br = MODE == 2 ? b + (uint64_t)(blockIdx.x % heads) * n : b;
+    auto finish = [&](uint32_t i, float4 v) {
+        float4 o;
+        if (MODE == 0) {
+            o = make_float4(expf(v.x - centre) * scale, expf(v.y - centre) * scale, expf(v.z - centre) * scale, expf(v.w - centre) * scale);
+        } else {
+            const float4 wv = load_vec4(wr + 4 * i), bv = load_vec4(br + 4 * i);
+            o = make_float4(fmaf((v.x - centre) * scale, wv.x, bv.x), fmaf((v.y - centre) * scale, wv.y, bv.y),
+                            fmaf((v.z - centre) * scale, wv.z, bv.z), fmaf((v.w - centre) * scale, wv.w, bv.w));
+        }
+        store_vec4(row + 4 * i, o);
+    };
+    if (cached) {
+#pragma unroll
+        for (int c = 0; c < kRowCache; c++) {
+            const uint32_t i = threadIdx.x + c * THREADS;
+            if (i < nv) finish(i, cache[c]);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < nv; i += THREADS) finish(i, load_vec4(row + 4 * i));
+    }
+}
+
+struct ViewArgs {
+    uint32_t shape[4], stride[4], offset[4];
+};
+
+// element index of vector `index` of (batch, token) in a view, in units of 4 elements
+// (compute_index of the shaders: src/shaders/binary.wgsl:30-34)
+__device__ __forceinline__ uint64_t view_index(const ViewArgs &v, uint32_t batch, uint32_t token, uint32_t index) {
+    const uint64_t stride = v.stride[0] >> 2;
+    return ((uint64_t)(batch + v.offset[2]) * v.stride[1] + (token + v.offset[1])) * stride + index + (v.offset[0] >> 2);
+}
+
+// output = ACT_OUT(ACT_X(input) op ACT_Y(output)); input broadcast over tokens / batches of extent 1
+template <typename IT, typename OT, bool MUL>
+__global__ __launch_bounds__(256) void binary_kernel(const IT *input, OT *output, ViewArgs src, ViewArgs dst, int act_x, int act_y, int act_out) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, token = blockIdx.y, batch = blockIdx.z;
+    if (index >= dst.shape[0] / 4) return;
+    const float4 x = load_vec4(input + 4 * view_index(src, src.shape[2] == 1 ? 0u : batch, src.shape[1] == 1 ? 0u : token, index));
+    OT *out = output + 4 * view_index(dst, batch, token, index);
+    const float4 y = load_vec4(out);
+    auto f = [&](float a, float c) {
+        const float p = act_apply(act_x, a), q = act_apply(act_y, c);
+        return act_apply(act_out, MUL ? p * q : p + q);
+    };
+    store_vec4(out, make_float4(f(x.x, y.x), f(x.y, y.y), f(x.z, y.z), f(x.w, y.w)));
+}
+
+int check_row_tensor(const wrq_tensor *x, int dtype, const char *what) {
+    if (!x || !x->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
+    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, dtype);
+    if (x->shape[3] != 1) return fail(WRQ_ERR_SHAPE, "%s: data shape [%u, %u, %u, %u] not match", what, x->shape[0], x->shape[1], x->shape[2], x->shape[3]);
+    if (x->shape[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "%s: row length %u not a multiple of 4", what, x->shape[0]);
+    if ((uintptr_t)x->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
+    return WRQ_OK;
+}
+
+template <int MODE>
+int launch_rows(hipStream_t stream, void *x, int dtype, const void *w, const void *b, uint32_t n, uint64_t rows, uint32_t heads, float eps, const char *what) {
+    if (rows == 0 || n == 0) return WRQ_OK;
+    if (rows > 0x7fffffffull) return fail(WRQ_ERR_SIZE, "%s: data size not match", what);
+    const uint16_t *wp = static_cast<const uint16_t *>(w), *bp = static_cast<const uint16_t *>(b);
+    // short rows (a head of a group norm) take one wave, no LDS exchange
+    if (n <= 1024) {
+        if (dtype == WRQ_F16) hipLaunchKernelGGL((row_kernel<uint16_t, MODE, 64>), dim3((uint32_t)rows), dim3(64), 0, stream, static_cast<uint16_t *>(x), wp, bp, n, heads, eps);
+        else hipLaunchKernelGGL((row_kernel<float, MODE, 64>), dim3((uint32_t)rows), dim3(64), 0, stream, static_cast<float *>(x), wp, bp, n, heads, eps);
+    } else {
+        if (dtype == WRQ_F16) hipLaunchKernelGGL((row_kernel<uint16_t, MODE, kRowThreads>), dim3((uint32_t)rows), dim3(kRowThreads), 0, stream, static_cast<uint16_t *>(x), wp, bp, n, heads, eps);
+        else hipLaunchKernelGGL((row_kernel<float, MODE, kRowThreads>), dim3((uint32_t)rows), dim3(kRowThreads), 0, stream, static_cast<float *>(x), wp, bp, n, heads, eps);
+    }
+    return check_launch(what);
+}
+
+ViewArgs view_args(const wrq_view &v) {
+    ViewArgs a;
+    for (int i = 0; i < 4; i++) a.shape[i] = v.shape[i], a.stride[i] = v.stride[i], a.offset[i] = v.offset[i];
+    return a;
+}
+
+int check_view(const wrq_tensor_view *t, const char *what) {
+    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
+    if (t->dtype != WRQ_F16 && t->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, (int)t->dtype);
+    for (int i = 0; i < 4; i++)
+        if ((uint64_t)t->view.offset[i] + t->view.shape[i] > t->view.stride[i])
+            return fail(WRQ_ERR_SHAPE, "%s: slice out of range", what);
+    if (t->view.shape[0] % 4 || t->view.stride[0] % 4 || t->view.offset[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "%s: rows not in units of 4 elements", what);
+    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
+    return WRQ_OK;
+}
+
+template <bool MUL>
+int binary(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_view *output, int act_x, int act_y, int act_out) {
+    const char *what = MUL ? "mul" : "add";
+    int s = check_view(input, what);
+    if (s != WRQ_OK) return s;
+    s = check_view(output, what);
+    if (s != WRQ_OK) return s;
+    for (int a : {act_x, act_y, act_out})
+        if (a < 0 || a > WRQ_ACT_SILU) return fail(WRQ_ERR_UNSUPPORTED, "%s: unknown activation %d", what, a);
+    const uint32_t *o = output->view.shape, *i = input->view.shape;
+    // the shapes check_shape_any accepts (src/tensor/ops.rs:1243-1249)
+    const bool ok = o[3] == 1 && i[0] == o[0] &&
+                    ((i[1] == o[1] && i[2] == o[2] && i[3] == 1) || (i[1] == o[1] && i[2] == 1 && i[3] == o[2]) || (i[1] == 1 && i[2] == o[2] && i[3] == 1) ||
+                     (i[1] == 1 && i[2] == 1 && i[3] == 1));
+    if (!ok) return fail(WRQ_ERR_SHAPE, "%s: data shape [%u, %u, %u, %u] not match [%u, %u, %u, %u]", what, i[0], i[1], i[2], i[3], o[0], o[1], o[2], o[3]);
+    if (o[0] == 0 || o[1] == 0 || o[2] == 0) return WRQ_OK;
+    if (o[1] > 65535u || o[2] > 65535u) return fail(WRQ_ERR_SIZE, "%s: data size not match", what);
+    const dim3 grid((o[0] / 4 + 255) / 256, o[1], o[2]);
+    const ViewArgs src = view_args(input->view), dst = view_args(output->view);
+    const bool i16 = input->dtype == WRQ_F16, o16 = output->dtype == WRQ_F16;
+    if (i16 && o16) hipLaunchKernelGGL((binary_kernel<uint16_t, uint16_t, MUL>), grid, dim3(256), 0, stream, static_cast<const uint16_t *>(input->data), static_cast<uint16_t *>(output->data), src, dst, act_x, act_y, act_out);
+    else if (i16) hipLaunchKernelGGL((binary_kernel<uint16_t, float, MUL>), grid, dim3(256), 0, stream, static_cast<const uint16_t *>(input->data), static_cast<float *>(output->data), src, dst, act_x, act_y, act_out);
+    else if (o16) hipLaunchKernelGGL((binary_kernel<float, uint16_t, MUL>), grid, dim3(256), 0, stream, static_cast<const float *>(input->data), static_cast<uint16_t *>(output->data), src, dst, act_x, act_y, act_out);
+    else hipLaunchKernelGGL((binary_kernel<float, float, MUL>), grid, dim3(256), 0, stream, static_cast<const float *>(input->data), static_cast<float *>(output->data), src, dst, act_x, act_y, act_out);
+    return check_launch(what);
+}
+
+} // namespace
+
+} // namespace wrq
+
+using namespace wrq;
+
+extern "C" {
+
+int wrq_softmax(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype) {
+    const int s = check_row_tensor(x, dtype, "softmax");
+    if (s != WRQ_OK) return s;
+    return launch_rows<0>(static_cast<hipStream_t>(stream), x->data, dtype, nullptr, nullptr, x->shape[0], (uint64_t)x->shape[1] * x->shape[2], 1, 0.0f, "softmax");
+}
+
+int wrq_layer_norm(wrq_stream stream, const wrq_tensor *w, const wrq_tensor *b, const wrq_tensor *x, wrq_dtype dtype, float eps) {
+    const int s = check_row_tensor(x, dtype, "layer_norm");
+    if (s != WRQ_OK) return s;
+    if (!w || !b || !w->data || !b->data) return fail(WRQ_ERR_NULL, "layer_norm: null tensor");
+    for (const wrq_tensor *t : {w, b})
+        if (t->shape[0] != x->shape[0] || t->shape[1] != 1 || t->shape[2] != 1 || t->shape[3] != 1)
+            return fail(WRQ_ERR_SHAPE, "layer_norm: data shape [%u, %u, %u, %u] not match [%u, 1, 1, 1]", t->shape[0], t->shape[1], t->shape[2], t->shape[3], x->shape[0]);
+    if ((uintptr_t)w->data % 8 || (uintptr_t)b->data % 8) return fail(WRQ_ERR_ALIGNMENT, "layer_norm: device pointers must be 8-byte aligned");
+    return launch_rows<1>(static_cast<hipStream_t>(stream), x->data, dtype, w->data, b->data, x->shape[0], (uint64_t)x->shape[1] * x->shape[2], 1, eps, "layer_norm");
+}
+
+int wrq_group_norm(wrq_stream stream, const wrq_tensor *w, const wrq_tensor *b, const wrq_tensor *x, wrq_dtype dtype, float eps) {
+    const int s = check_row_tensor(x, dtype, "group_norm");
+    if (s != WRQ_OK) return s;
+    if (!w || !b || !w->data || !b->data) return fail(WRQ_ERR_NULL, "group_norm: null tensor");
+    for (const wrq_tensor *t : {w, b})
+        if (t->shape[0] != x->shape[0] || t->shape[1] != x->shape[1] || t->shape[2] != 1 || t->shape[3] != 1)
+            return fail(WRQ_ERR_SHAPE, "group_norm: data shape [%u, %u, %u, %u] not match [%u, %u, 1, 1]", t->shape[0], t->shape[1], t->shape[2], t->shape[3], x->shape[0], x->shape[1]);
+    if ((uintptr_t)w->data % 8 || (uintptr_t)b->data % 8) return fail(WRQ_ERR_ALIGNMENT, "group_norm: device pointers must be 8-byte aligned");
+    return launch_rows<2>(static_cast<hipStream_t>(stream), x->data, dtype, w->data, b->data, x->shape[0], (uint64_t)x->shape[1] * x->shape[2], x->shape[1], eps, "group_norm");
+}
+
+int wrq_add_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output, int act_x, int act_y, int act_out) {
+    return binary<false>(static_cast<hipStream_t>(stream), input, output, act_x, act_y, act_out);
+}
+
+int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output, int act_x, int act_y, int act_out) {
+    return binary<true>(static_cast<hipStream_t>(stream), input, output, act_x, act_y, act_out);
+}
+
+} // extern "C"
