@@ -234,6 +234,24 @@ int wrq_add_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_
 int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output,
                      int act_x, int act_y, int act_out);
 
+/*
+ * TensorOp::blit(input, output)             src/tensor/ops.rs:2015-2068, src/shaders/blit.wgsl
+ *   copies a view into a view of the same shape, converting the element type.
+ * TensorOp::transpose(input, output)        src/tensor/ops.rs:2121-2169, src/shaders/reshape.wgsl:58-77
+ *   input [C, T, B, 1] -> output [C, B, T, 1].
+ * TensorOp::activate(x, act)                src/tensor/ops.rs:1973-2013, src/shaders/activation.wgsl
+ * TensorOp::affine(x, scale, bias)          src/tensor/ops.rs:2352-2391, src/shaders/affine.wgsl
+ *   x <- scale * x + bias on a whole tensor [C, T, B, 1].
+ * TensorOp::lerp(input, output, factor, reversed)   src/tensor/ops.rs:2284-2350, src/shaders/lerp.wgsl
+ *   output <- input (1 - f) + output f (reversed: the two swapped); factor [C, T|1, B|1, 1].
+ */
+int wrq_blit(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output);
+int wrq_transpose(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output);
+int wrq_activate(wrq_stream stream, const wrq_tensor_view *x, int act);
+int wrq_affine(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype, float scale, float bias);
+int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output,
+             const wrq_tensor_view *factor, int reversed);
+
 #ifdef __cplusplus
 }
 #endif

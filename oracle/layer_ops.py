@@ -140,3 +140,32 @@ def binary(op, x, y, act_x=0, act_y=0, act_out=0):
     a, c = activation(act_x, np.asarray(x).astype(F)), activation(act_y, np.asarray(y).astype(F))
     r = activation(act_out, a * c if op == "mul" else a + c)
     return r.astype(np.asarray(y).dtype)
+
+
+def view(a, shape, offset):
+    """The slice a `View` names: numpy array (B, T, C) (last axis = x), reference-order shape / offset."""
+    a = np.asarray(a)
+    a = a.reshape((1,) * (3 - a.ndim) + a.shape) if a.ndim < 3 else a
+    (c, t, b), (oc, ot, ob) = shape[:3], offset[:3]
+    return a[ob:ob + b, ot:ot + t, oc:oc + c]
+
+
+def blit(src, dst):
+    """dst[...] = src converted to dst's type (src/shaders/blit.wgsl:35-53); both already sliced."""
+    dst[...] = np.asarray(src).astype(F).astype(dst.dtype)
+
+
+def transpose(src, dst):
+    """input [C, T, B] -> output [C, B, T] (src/shaders/reshape.wgsl:58-77): numpy (B, T, C) -> (T, B, C)."""
+    dst[...] = np.swapaxes(np.asarray(src), 0, 1).astype(F).astype(dst.dtype)
+
+
+def affine(x, scale, bias):
+    return (F(scale) * np.asarray(x).astype(F) + F(bias)).astype(np.asarray(x).dtype)
+
+
+def lerp(x, y, f, reversed=False):
+    """mix(x, y, f) = x (1 - f) + y f in f32, result in y's type (src/shaders/lerp.wgsl:82-93)."""
+    a, c, t = np.asarray(x).astype(F), np.asarray(y).astype(F), np.asarray(f).astype(F)
+    r = c * (F(1) - t) + a * t if reversed else a * (F(1) - t) + c * t
+    return r.astype(np.asarray(y).dtype)

@@ -107,3 +107,5 @@ if __name__ == "__main__":
     with open(os.path.join(HERE, "rnn_iter_kats.json"), "w") as f:
         json.dump(RNN_KATS, f, indent=1)
     print("wrote", len(cases), "cases")
+    # data_movement_kats.json beside these holds the literal buffers of test_blit / test_transpose
+    # (src/tensor/ops.rs:3302-3365); it is data copied by hand, nothing computes it

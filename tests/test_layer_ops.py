@@ -118,7 +118,99 @@ def test_oracle_binary(lop, op):
         assert_close(lop.activation(act, pts), np.array(w, dtype=np.float64), 1e-6, f"activation {act}")
 
 
+def movement_kats():
+    import json
+
+    with open(os.path.join(ROOT, "tests", "golden", "data_movement_kats.json")) as f:
+        return json.load(f)
+
+
+def test_oracle_data_movement_kats(lop):
+    k = movement_kats()
+    out = np.zeros(k["blit"]["output_shape"][::-1][1:], dtype=np.float32)  # (B, T, C)
+    for op in k["blit"]["ops"]:
+        src = np.array(op["input"], dtype=np.float32).reshape(op["input_shape"][::-1][1:])
+        lop.blit(src, lop.view(out, op["view_shape"], op["view_offset"]))
+    assert out.reshape(-1).tolist() == k["blit"]["expected"]
+    t = k["transpose"]
+    out = np.zeros(t["output_shape"][::-1][1:], dtype=np.float32)
+    src = np.array(t["input"], dtype=np.float32).reshape(t["input_shape"][::-1][1:])
+    lop.transpose(src, lop.view(out, t["view_shape"], t["view_offset"]))
+    assert out.reshape(-1).tolist() == t["expected"]
+
+
+def test_oracle_lerp_affine(lop):
+    rng = np.random.default_rng(SEED + 5)
+    x = (rng.random((2, 3, 1000), dtype=np.float32) - 0.5).astype(np.float32)
+    y = (rng.random((2, 3, 1000), dtype=np.float32) - 0.5).astype(np.float32)
+    f = rng.random((2, 3, 1000), dtype=np.float32)
+    want = x.astype(np.float64) * (1 - f.astype(np.float64)) + y.astype(np.float64) * f  # ops.rs:3286-3290
+    assert_close(lop.lerp(x, y, f), want, 1e-6, "lerp")
+    assert_close(lop.lerp(x, y, f, reversed=True), y.astype(np.float64) * (1 - f.astype(np.float64)) + x.astype(np.float64) * f, 1e-6, "reversed")
+    assert np.array_equal(lop.lerp(x, y, np.zeros_like(f)), x) and np.array_equal(lop.lerp(x, y, np.ones_like(f)), y)
+    assert_close(lop.affine(x, 0.5, 0.0), x / 2, 0.0, "affine halves exactly")  # the rescale of v6.rs:953-955
+
+
 # ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_gpu_data_movement_kats(gpu):
+    import torch
+
+    print("blit / transpose KATs on the GPU", flush=True)
+    k = movement_kats()
+    for dt in (torch.float32, torch.float16):
+        out = torch.zeros(k["blit"]["output_shape"][::-1][1:], dtype=dt, device="cuda")
+        for op in k["blit"]["ops"]:
+            src = torch.tensor(op["input"], dtype=torch.float32, device="cuda").reshape(op["input_shape"][::-1][1:])
+            gpu.LayerOp.blit(src, out, output_view=(op["view_shape"], k["blit"]["output_shape"], op["view_offset"]))
+        assert out.float().reshape(-1).tolist() == k["blit"]["expected"]
+        t = k["transpose"]
+        out = torch.zeros(t["output_shape"][::-1][1:], dtype=dt, device="cuda")
+        src = torch.tensor(t["input"], dtype=torch.float32, device="cuda").reshape(t["input_shape"][::-1][1:])
+        gpu.LayerOp.transpose(src, out, output_view=(t["view_shape"], t["output_shape"], t["view_offset"]))
+        assert out.float().reshape(-1).tolist() == t["expected"]
+    with pytest.raises(gpu.TensorError):
+        gpu.LayerOp.transpose(src, torch.zeros((3, 2, 8), dtype=torch.float32, device="cuda"))
+
+
+@pytest.mark.gpu
+def test_gpu_lerp_activate_affine(gpu, lop):
+    import torch
+
+    print("lerp / activate / affine on the GPU", flush=True)
+    rng = np.random.default_rng(SEED + 40)
+    B, T, C = 2, 3, 1000
+    x = (rng.random((B, T, C), dtype=np.float32) - 0.5).astype(np.float32)
+    y = (rng.random((B, T, C), dtype=np.float32) - 0.5).astype(np.float32)
+    for fshape in ((B, T, C), (1, T, C), (B, 1, C), (1, 1, C)):
+        f = rng.random(fshape, dtype=np.float32)
+        for rev in (False, True):
+            for ft, it, ot in ((np.float32, np.float32, np.float32), (np.float16, np.float16, np.float32), (np.float32, np.float16, np.float16)):
+                yd = torch.from_numpy(y.astype(ot)).cuda()
+                gpu.LayerOp.lerp(torch.from_numpy(x.astype(it)).cuda(), yd, torch.from_numpy(f.astype(ft)).cuda(), rev)
+                want = lop.lerp(x.astype(it), y.astype(ot), f.astype(ft), rev)
+                assert_close(yd.cpu().numpy(), want, 1e-3 if ot == np.float16 else 1e-6, f"lerp {fshape} {rev} {ot.__name__}")
+    for act in range(8):
+        for dt in (np.float32, np.float16):
+            v = (1.5 * rng.standard_normal((B, T, C))).astype(dt)  # exp stays inside f16
+            vd = torch.from_numpy(v.copy()).cuda()
+            gpu.LayerOp.activate(vd, act)
+            assert_close(vd.cpu().numpy(), lop.activation(act, v.astype(np.float32)).astype(dt), 2e-3 if dt == np.float16 else 2e-6, f"activate {act} {dt.__name__}")
+    # a view: only slice 1 of 3 changes
+    v = rng.standard_normal((3, T, C)).astype(np.float32)
+    vd = torch.from_numpy(v.copy()).cuda()
+    gpu.LayerOp.activate(vd, gpu.ACT_STABLE_EXP, view=((C, T, 1), (C, T, 3), (0, 0, 1)))
+    want = v.copy()
+    want[1] = lop.activation(3, v[1])
+    assert_close(vd.cpu().numpy(), want, 2e-6, "activate on a view")
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.affine(xd, 0.5, 0.0)
+    assert np.array_equal(xd.cpu().numpy(), x * np.float32(0.5))
+    hd = torch.from_numpy(x.astype(np.float16)).cuda()
+    gpu.LayerOp.affine(hd, 2.0, 1.0)
+    assert_close(hd.cpu().numpy(), lop.affine(x.astype(np.float16), 2.0, 1.0), 1e-3, "affine f16")
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("C,T,B", [(1000, 3, 2), (4096, 1, 1), (4096, 128, 1), (65536, 2, 1), (64, 5, 1), (4, 1, 3)])

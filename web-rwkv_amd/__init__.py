@@ -42,6 +42,7 @@ EXPORTS = [
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
+    "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
 ]
 MAX_GROUP = 8
 
@@ -187,6 +188,11 @@ def lib():
         L.wrq_group_norm.argtypes = [vp, T, T, T, i, C.c_float]
         L.wrq_add_activate.argtypes = [vp, V, V, i, i, i]
         L.wrq_mul_activate.argtypes = [vp, V, V, i, i, i]
+        L.wrq_blit.argtypes = [vp, V, V]
+        L.wrq_transpose.argtypes = [vp, V, V]
+        L.wrq_activate.argtypes = [vp, V, i]
+        L.wrq_affine.argtypes = [vp, T, i, C.c_float, C.c_float]
+        L.wrq_lerp.argtypes = [vp, V, V, V, i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -309,6 +315,27 @@ class LayerOp:
 
     add = add_activate
     mul = mul_activate
+
+    @staticmethod
+    def blit(input, output, input_view=None, output_view=None):
+        _check(lib().wrq_blit(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view))))
+
+    @staticmethod
+    def transpose(input, output, input_view=None, output_view=None):
+        _check(lib().wrq_transpose(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view))))
+
+    @staticmethod
+    def activate(x, act, view=None):
+        _check(lib().wrq_activate(_stream(), C.byref(as_view(x, view)), act))
+
+    @staticmethod
+    def affine(x, scale, bias):
+        _check(lib().wrq_affine(_stream(), C.byref(as_tensor(x)), _dtype(x), scale, bias))
+
+    @staticmethod
+    def lerp(input, output, factor, reversed=False, input_view=None, output_view=None, factor_view=None):
+        _check(lib().wrq_lerp(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)),
+                              C.byref(as_view(factor, factor_view)), int(reversed)))
 
 
 def matmul_vec_group(ops):

@@ -159,6 +159,41 @@ __global__ __launch_bounds__(256) void binary_kernel(const IT *input, OT *output
     store_vec4(out, make_float4(f(x.x, y.x), f(x.y, y.y), f(x.z, y.z), f(x.w, y.w)));
 }
 
+// output view <- input view, element types converted (blit); MODE 1 swaps token and batch on the
+// way out (transpose); src/shaders/blit.wgsl:35-53, reshape.wgsl:58-77
+template <typename IT, typename OT, int MODE>
+__global__ __launch_bounds__(256) void copy_kernel(const IT *input, OT *output, ViewArgs src, ViewArgs dst) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, token = blockIdx.y, batch = blockIdx.z;
+    if (index >= src.shape[0] / 4) return;
+    const float4 x = load_vec4(input + 4 * view_index(src, batch, token, index));
+    store_vec4(output + 4 * (MODE == 1 ? view_index(dst, token, batch, index) : view_index(dst, batch, token, index)), x);
+}
+
+// x <- act(x) over a view (src/shaders/activation.wgsl:30-45), or scale * x + bias (affine.wgsl:16-30)
+template <typename XT, bool AFFINE>
+__global__ __launch_bounds__(256) void unary_kernel(XT *x, ViewArgs v, int act, float scale, float bias) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, token = blockIdx.y, batch = blockIdx.z;
+    if (index >= v.shape[0] / 4) return;
+    XT *p = x + 4 * view_index(v, batch, token, index);
+    const float4 a = load_vec4(p);
+    if (AFFINE) store_vec4(p, make_float4(scale * a.x + bias, scale * a.y + bias, scale * a.z + bias, scale * a.w + bias));
+    else store_vec4(p, make_float4(act_apply(act, a.x), act_apply(act, a.y), act_apply(act, a.z), act_apply(act, a.w)));
+}
+
+// y <- mix(x, y, f) = x (1 - f) + y f, or mix(y, x, f) when reversed; f broadcast over extents of 1
+// (src/shaders/lerp.wgsl:72-93)
+template <typename FT, typename IT, typename OT>
+__global__ __launch_bounds__(256) void lerp_kernel(const FT *f, const IT *x, OT *y, ViewArgs vf, ViewArgs vx, ViewArgs vy, int reversed) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, token = blockIdx.y, batch = blockIdx.z;
+    if (index >= vy.shape[0] / 4) return;
+    const float4 ff = load_vec4(f + 4 * view_index(vf, vf.shape[2] == 1 ? 0u : batch, vf.shape[1] == 1 ? 0u : token, index));
+    const float4 a = load_vec4(x + 4 * view_index(vx, batch, token, index));
+    OT *out = y + 4 * view_index(vy, batch, token, index);
+    const float4 c = load_vec4(out);
+    auto mix = [&](float p, float q, float t) { return reversed ? q * (1.0f - t) + p * t : p * (1.0f - t) + q * t; };
+    store_vec4(out, make_float4(mix(a.x, c.x, ff.x), mix(a.y, c.y, ff.y), mix(a.z, c.z, ff.z), mix(a.w, c.w, ff.w)));
+}
+
 int check_row_tensor(const wrq_tensor *x, int dtype, const char *what) {
     if (!x || !x->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, dtype);
@@ -228,6 +263,53 @@ int binary(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_vi
     return check_launch(what);
 }
 
+template <int MODE>
+int copy(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_view *output) {
+    const char *what = MODE == 1 ? "transpose" : "blit";
+    int s = check_view(input, what);
+    if (s != WRQ_OK) return s;
+    s = check_view(output, what);
+    if (s != WRQ_OK) return s;
+    const uint32_t *i = input->view.shape, *o = output->view.shape;
+    const bool ok = MODE == 1 ? (o[0] == i[0] && o[1] == i[2] && o[2] == i[1] && o[3] == 1 && i[3] == 1) : (o[0] == i[0] && o[1] == i[1] && o[2] == i[2] && o[3] == i[3]);
+    if (!ok) return fail(WRQ_ERR_SHAPE, "%s: data shape [%u, %u, %u, %u] not match [%u, %u, %u, %u]", what, i[0], i[1], i[2], i[3], o[0], o[1], o[2], o[3]);
+    if (i[0] == 0 || i[1] == 0 || i[2] == 0) return WRQ_OK;
+    if (i[1] > 65535u || i[2] > 65535u) return fail(WRQ_ERR_SIZE, "%s: data size not match", what);
+    const dim3 grid((i[0] / 4 + 255) / 256, i[1], i[2]);
+    const ViewArgs src = view_args(input->view), dst = view_args(output->view);
+    const bool i16 = input->dtype == WRQ_F16, o16 = output->dtype == WRQ_F16;
+    if (i16 && o16) hipLaunchKernelGGL((copy_kernel<uint16_t, uint16_t, MODE>), grid, dim3(256), 0, stream, static_cast<const uint16_t *>(input->data), static_cast<uint16_t *>(output->data), src, dst);
+    else if (i16) hipLaunchKernelGGL((copy_kernel<uint16_t, float, MODE>), grid, dim3(256), 0, stream, static_cast<const uint16_t *>(input->data), static_cast<float *>(output->data), src, dst);
+    else if (o16) hipLaunchKernelGGL((copy_kernel<float, uint16_t, MODE>), grid, dim3(256), 0, stream, static_cast<const float *>(input->data), static_cast<uint16_t *>(output->data), src, dst);
+    else hipLaunchKernelGGL((copy_kernel<float, float, MODE>), grid, dim3(256), 0, stream, static_cast<const float *>(input->data), static_cast<float *>(output->data), src, dst);
+    return check_launch(what);
+}
+
+template <bool AFFINE>
+int unary(hipStream_t stream, const wrq_tensor_view *x, int act, float scale, float bias) {
+    const char *what = AFFINE ? "affine" : "activate";
+    const int s = check_view(x, what);
+    if (s != WRQ_OK) return s;
+    if (!AFFINE && (act < 0 || act > WRQ_ACT_SILU)) return fail(WRQ_ERR_UNSUPPORTED, "%s: unknown activation %d", what, act);
+    const uint32_t *v = x->view.shape;
+    if (v[3] != 1) return fail(WRQ_ERR_SHAPE, "%s: data shape [%u, %u, %u, %u] not match", what, v[0], v[1], v[2], v[3]);
+    if (v[0] == 0 || v[1] == 0 || v[2] == 0) return WRQ_OK;
+    if (v[1] > 65535u || v[2] > 65535u) return fail(WRQ_ERR_SIZE, "%s: data size not match", what);
+    const dim3 grid((v[0] / 4 + 255) / 256, v[1], v[2]);
+    const ViewArgs va = view_args(x->view);
+    if (x->dtype == WRQ_F16) hipLaunchKernelGGL((unary_kernel<uint16_t, AFFINE>), grid, dim3(256), 0, stream, static_cast<uint16_t *>(x->data), va, act, scale, bias);
+    else hipLaunchKernelGGL((unary_kernel<float, AFFINE>), grid, dim3(256), 0, stream, static_cast<float *>(x->data), va, act, scale, bias);
+    return check_launch(what);
+}
+
+template <typename FT, typename IT>
+int lerp_out(hipStream_t stream, const wrq_tensor_view *f, const wrq_tensor_view *x, const wrq_tensor_view *y, dim3 grid, int reversed) {
+    const ViewArgs vf = view_args(f->view), vx = view_args(x->view), vy = view_args(y->view);
+    if (y->dtype == WRQ_F16) hipLaunchKernelGGL((lerp_kernel<FT, IT, uint16_t>), grid, dim3(256), 0, stream, static_cast<const FT *>(f->data), static_cast<const IT *>(x->data), static_cast<uint16_t *>(y->data), vf, vx, vy, reversed);
+    else hipLaunchKernelGGL((lerp_kernel<FT, IT, float>), grid, dim3(256), 0, stream, static_cast<const FT *>(f->data), static_cast<const IT *>(x->data), static_cast<float *>(y->data), vf, vx, vy, reversed);
+    return check_launch("lerp");
+}
+
 } // namespace
 
 } // namespace wrq
@@ -270,6 +352,48 @@ int wrq_add_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_
 
 int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output, int act_x, int act_y, int act_out) {
     return binary<true>(static_cast<hipStream_t>(stream), input, output, act_x, act_y, act_out);
+}
+
+int wrq_blit(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output) {
+    return copy<0>(static_cast<hipStream_t>(stream), input, output);
+}
+
+int wrq_transpose(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output) {
+    return copy<1>(static_cast<hipStream_t>(stream), input, output);
+}
+
+int wrq_activate(wrq_stream stream, const wrq_tensor_view *x, int act) {
+    return unary<false>(static_cast<hipStream_t>(stream), x, act, 1.0f, 0.0f);
+}
+
+int wrq_affine(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype, float scale, float bias) {
+    if (!x) return fail(WRQ_ERR_NULL, "affine: null tensor");
+    wrq_tensor_view v;
+    v.data = x->data;
+    v.dtype = dtype;
+    for (int i = 0; i < 4; i++) v.view.shape[i] = v.view.stride[i] = x->shape[i], v.view.offset[i] = 0;
+    return unary<true>(static_cast<hipStream_t>(stream), &v, 0, scale, bias);
+}
+
+int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output, const wrq_tensor_view *factor, int reversed) {
+    int s = check_view(input, "lerp");
+    if (s == WRQ_OK) s = check_view(output, "lerp");
+    if (s == WRQ_OK) s = check_view(factor, "lerp");
+    if (s != WRQ_OK) return s;
+    const uint32_t *o = output->view.shape, *i = input->view.shape, *f = factor->view.shape;
+    // src/tensor/ops.rs:2298-2307
+    const bool fok = f[0] == o[0] && f[3] == 1 && (f[1] == o[1] || f[1] == 1) && (f[2] == o[2] || f[2] == 1);
+    if (o[3] != 1 || !fok || i[0] != o[0] || i[1] != o[1] || i[2] != o[2] || i[3] != 1)
+        return fail(WRQ_ERR_SHAPE, "lerp: data shape [%u, %u, %u, %u] / [%u, %u, %u, %u] not match [%u, %u, %u, %u]", i[0], i[1], i[2], i[3], f[0], f[1], f[2], f[3], o[0], o[1], o[2], o[3]);
+    if (o[0] == 0 || o[1] == 0 || o[2] == 0) return WRQ_OK;
+    if (o[1] > 65535u || o[2] > 65535u) return fail(WRQ_ERR_SIZE, "lerp: data size not match");
+    const dim3 grid((o[0] / 4 + 255) / 256, o[1], o[2]);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool f16 = factor->dtype == WRQ_F16, i16 = input->dtype == WRQ_F16;
+    if (f16 && i16) return lerp_out<uint16_t, uint16_t>(st, factor, input, output, grid, reversed);
+    if (f16) return lerp_out<uint16_t, float>(st, factor, input, output, grid, reversed);
+    if (i16) return lerp_out<float, uint16_t>(st, factor, input, output, grid, reversed);
+    return lerp_out<float, float>(st, factor, input, output, grid, reversed);
 }
 
 } // extern "C"
