@@ -252,6 +252,35 @@ int wrq_affine(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype, float sc
 int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output,
              const wrq_tensor_view *factor, int reversed);
 
+/*
+ * The ops that carry state from token to token.  A run is a stack of A tokens of several requests;
+ * cursors u32 [A, 1, 1, 1]: for the request of token a, its state slot | first token in the stack << 8
+ * | number of its tokens in the stack << 24 (compute_cursor of the shaders).  States are f32 views.
+ *
+ * TensorOp::token_shift(cursors, time_mix, state, input, output, reversed)
+ *                                           src/tensor/ops.rs:1393-1462, src/shaders/token_shift.wgsl
+ *   output [C, A, I, 1] <- mix(previous token, this token, time_mix) (reversed: the two swapped);
+ *   input [C, A, 1|I, 1] (slice 0 is read), time_mix [C, A, I, 1] or [C, 1, 1, 1], state [C, _, B, 1]
+ *   (row 0 of the view is the token before a request's first token of the stack).
+ * TensorOp::channel_mix(cursors, state, r, v, x)
+ *                                           src/tensor/ops.rs:1860-1915, src/shaders/channel_mix.wgsl
+ *   state [C, 1, B, 1] <- x at every request's last token; x [C, A, 1, 1] <- sigmoid(r) * v.
+ * TensorOp::time_mix_v6(cursors, time_decay, time_first, state, k, v, r, x)
+ *                                           src/tensor/ops.rs:1601-1677, src/shaders/time_mix_v6.wgsl
+ *   x, k, v, r, time_decay(f32) [S, H, A, 1]; time_first f32 [S, H, 1, 1]; state [S H, S + 1, B, 1]:
+ *   row 0 <- x at every request's last token, rows 1 + j hold S[j][.];
+ *   x[i] <- sum_j r[j] (time_first[j] k[j] v[i] + S[j][i]),  S[j][i] <- time_decay[j] S[j][i] + k[j] v[i].
+ *   Head sizes 16, 32, 64, 128 and 256 are built.
+ */
+int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix,
+                    const wrq_tensor_view *state, const wrq_tensor *input, wrq_dtype input_dtype,
+                    const wrq_tensor *output, wrq_dtype output_dtype, int reversed);
+int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state,
+                    const wrq_tensor *r, const wrq_tensor *v, const wrq_tensor *x, wrq_dtype dtype);
+int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay,
+                    const wrq_tensor *time_first, const wrq_tensor_view *state, const wrq_tensor *k,
+                    const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -169,3 +169,76 @@ def lerp(x, y, f, reversed=False):
     a, c, t = np.asarray(x).astype(F), np.asarray(y).astype(F), np.asarray(f).astype(F)
     r = c * (F(1) - t) + a * t if reversed else a * (F(1) - t) + c * t
     return r.astype(np.asarray(y).dtype)
+
+
+# ---- ops that carry state -----------------------------------------------------------------------
+def pack_cursors(runs):
+    """runs: list of (state slot, tokens of that request in the stack), in stack order ->
+    u32 per token: slot | first token << 8 | count << 24 (compute_cursor, token_shift.wgsl:44-51)."""
+    out, first = [], 0
+    for slot, n in runs:
+        out += [np.uint32(slot | (first << 8) | (n << 24))] * n
+        first += n
+    return np.array(out, dtype=np.uint32)
+
+
+def _cursor(c):
+    c = int(c)
+    return c & 0xff, (c >> 8) & 0xffff, (c >> 24) & 0xff
+
+
+def _mix(a, b, t):
+    return a * (F(1) - t) + b * t
+
+
+def token_shift(cursors, time_mix, state_row, x, out_dtype, counts=1, reversed=False):
+    """src/shaders/token_shift.wgsl:91-116.  x (A, C); time_mix (counts, A, C), (counts, 1, C) or (C,);
+    state_row (B, C) f32 = row 0 of the state view; result (counts, A, C)."""
+    x32 = np.asarray(x).astype(F)
+    A, C = x32.shape
+    tm = np.asarray(time_mix).astype(F)
+    tm = np.broadcast_to(tm.reshape((1, 1, C)) if tm.ndim == 1 else tm, (counts, A, C))
+    out = np.empty((counts, A, C), dtype=F)
+    for a in range(A):
+        slot, first, _ = _cursor(cursors[a])
+        prev = np.asarray(state_row)[slot].astype(F) if a == first else x32[a - 1]
+        for c in range(counts):
+            out[c, a] = _mix(x32[a], prev, tm[c, a]) if reversed else _mix(prev, x32[a], tm[c, a])
+    return out.astype(out_dtype)
+
+
+def channel_mix(cursors, state_row, r, v, x):
+    """src/shaders/channel_mix.wgsl:83-106: state_row (B, C) f32 updated in place; returns the new x."""
+    x = np.asarray(x)
+    for a in range(x.shape[0]):
+        slot, first, n = _cursor(cursors[a])
+        if a - first + 1 == n:
+            state_row[slot] = x[a].astype(F)
+    rr = F(1) / (F(1) + np.exp(-np.asarray(r).astype(F), dtype=F))
+    return (rr * np.asarray(v).astype(F)).astype(x.dtype)
+
+
+def _fma(a, b, c):
+    return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(F)
+
+
+def time_mix_v6(cursors, time_decay, time_first, state, k, v, r, x):
+    """src/shaders/time_mix_v6.wgsl:83-155.  k, v, r, x, time_decay (A, H, S); time_first (H, S);
+    state (B, S + 1, H * S) f32 updated in place (row 0: x at a request's last token; row 1 + j:
+    S[j][.]); the sum over j runs in the shader's order, one chain.  Returns the new x."""
+    x = np.asarray(x)
+    A, H, S = x.shape
+    k32, v32, r32, w32, u32 = (np.asarray(t).astype(F) for t in (k, v, r, time_decay, time_first))
+    out = np.empty((A, H, S), dtype=F)
+    for t in range(A):
+        slot, first, n = _cursor(cursors[t])
+        if t - first + 1 == n:
+            state[slot, 0] = x[first + n - 1].astype(F).reshape(-1)
+        y = np.zeros((H, S), dtype=F)
+        for j in range(S):
+            ss = state[slot, 1 + j].reshape(H, S)
+            kv = k32[t, :, j:j + 1] * v32[t]
+            y = y + r32[t, :, j:j + 1] * _fma(np.broadcast_to(u32[:, j:j + 1], (H, S)), kv, ss)
+            state[slot, 1 + j] = _fma(np.broadcast_to(w32[t, :, j:j + 1], (H, S)), ss, kv).reshape(-1)
+        out[t] = y
+    return out.astype(x.dtype)

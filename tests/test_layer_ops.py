@@ -151,6 +151,167 @@ def test_oracle_lerp_affine(lop):
     assert_close(lop.affine(x, 0.5, 0.0), x / 2, 0.0, "affine halves exactly")  # the rescale of v6.rs:953-955
 
 
+RUNS = [(2, 3), (0, 1), (5, 4)]  # (state slot, tokens in the stack): three requests, 8 tokens
+
+
+def test_oracle_token_shift_channel_mix(lop):
+    rng = np.random.default_rng(SEED + 6)
+    C, B = 64, 6
+    cur = lop.pack_cursors(RUNS)
+    A = len(cur)
+    x = rng.standard_normal((A, C)).astype(np.float16)
+    state = rng.standard_normal((B, C)).astype(np.float32)
+    tm = rng.random(C).astype(np.float16)
+    got = lop.token_shift(cur, tm, state, x, np.float32, reversed=True)
+    # by hand: the token before a request's first token is its state row, else the token before in the stack
+    prev = np.stack([state[2], x[0], x[1], state[0], state[5], x[4], x[5], x[6]]).astype(np.float64)
+    f = tm.astype(np.float64)
+    assert_close(got[0], x.astype(np.float64) * (1 - f) + prev * f, 1e-6, "reversed: mix(x, prev, f)")
+    assert_close(lop.token_shift(cur, tm, state, x, np.float32)[0], prev * (1 - f) + x.astype(np.float64) * f, 1e-6, "mix(prev, x, f)")
+    # per token and per count factors (the five data-dependent shifts of v6.rs:796-805)
+    tm5 = rng.random((5, A, C)).astype(np.float32)
+    got5 = lop.token_shift(cur, tm5, state, x, np.float16, counts=5, reversed=True)
+    assert got5.shape == (5, A, C) and got5.dtype == np.float16
+    assert_close(got5[3], x.astype(np.float64) * (1 - tm5[3]) + prev * tm5[3], 1e-3, "count 3")
+    # channel mix: the state takes x at every request's last token, x becomes sigmoid(r) v
+    r = rng.standard_normal((A, C)).astype(np.float16)
+    v = rng.standard_normal((A, C)).astype(np.float16)
+    st = state.copy()
+    out = lop.channel_mix(cur, st, r, v, x)
+    assert np.array_equal(st[2], x[2].astype(np.float32)) and np.array_equal(st[0], x[3].astype(np.float32)) and np.array_equal(st[5], x[7].astype(np.float32))
+    assert np.array_equal(st[[1, 3, 4]], state[[1, 3, 4]])
+    assert_close(out, v.astype(np.float64) / (1 + np.exp(-r.astype(np.float64))), 1e-3, "sigmoid(r) v")
+
+
+def wkv6_float64(cursors, w, u, state, k, v, r, x):
+    """textbook form of the recurrence per request and head, in float64, one token at a time:
+    y = r^T (diag(u) k v^T + S),  S <- diag(w) S + k v^T"""
+    A, H, S = x.shape
+    st = state.astype(np.float64).copy()
+    out = np.zeros((A, H, S))
+    for t in range(A):
+        c = int(cursors[t])
+        slot, first, n = c & 0xff, (c >> 8) & 0xffff, (c >> 24) & 0xff
+        if t - first + 1 == n:
+            st[slot, 0] = x[t].astype(np.float64).reshape(-1)
+        for h in range(H):
+            Sm = st[slot, 1:, h * S:(h + 1) * S]  # [j, i]
+            kv = np.outer(k[t, h].astype(np.float64), v[t, h].astype(np.float64))
+            out[t, h] = r[t, h].astype(np.float64) @ (u[h].astype(np.float64)[:, None] * kv + Sm)
+            st[slot, 1:, h * S:(h + 1) * S] = w[t, h].astype(np.float64)[:, None] * Sm + kv
+    return out, st
+
+
+def wkv6_inputs(rng, A, H, S, B, dtype):
+    k = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    v = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    r = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    x = rng.standard_normal((A, H, S)).astype(dtype)
+    w = np.exp(-np.exp(rng.standard_normal((A, H, S)).astype(np.float32))).astype(np.float32)  # the decay after StableExp
+    u = (0.3 * rng.standard_normal((H, S))).astype(np.float32)
+    state = (0.1 * rng.standard_normal((B, S + 1, H * S))).astype(np.float32)
+    return k, v, r, x, w, u, state
+
+
+def test_oracle_time_mix_v6(lop):
+    rng = np.random.default_rng(SEED + 7)
+    H, S, B = 3, 16, 6
+    cur = lop.pack_cursors(RUNS)
+    k, v, r, x, w, u, state = wkv6_inputs(rng, len(cur), H, S, B, np.float32)
+    st = state.copy()
+    got = lop.time_mix_v6(cur, w, u, st, k, v, r, x)
+    want, want_state = wkv6_float64(cur, w, u, state, k, v, r, x)
+    assert_close(got, want, 1e-5, "y vs float64")
+    assert_close(st, want_state, 1e-5, "state vs float64")
+    assert np.array_equal(st[[1, 3, 4]], state[[1, 3, 4]])  # requests that are not in the stack keep their state
+    # one token, zero state: y = (r . (u k)) v exactly as a closed form; the state becomes k v^T
+    z = np.zeros_like(state)
+    one = lop.pack_cursors([(1, 1)])
+    y1 = lop.time_mix_v6(one, w[:1], u, z, k[:1], v[:1], r[:1], x[:1])
+    assert_close(y1[0], (r[0] * u * k[0]).sum(axis=-1, keepdims=True).astype(np.float64) * v[0], 1e-5, "first token")
+    assert_close(z[1, 1:, :S], np.outer(k[0, 0], v[0, 0]), 1e-6, "state after the first token")
+    # a run of 2 tokens equals two runs of 1 token (the state carries everything)
+    s_a, s_b = state.copy(), state.copy()
+    two = lop.time_mix_v6(lop.pack_cursors([(4, 2)]), w[:2], u, s_a, k[:2], v[:2], r[:2], x[:2])
+    first = lop.time_mix_v6(lop.pack_cursors([(4, 1)]), w[:1], u, s_b, k[:1], v[:1], r[:1], x[:1])
+    second = lop.time_mix_v6(lop.pack_cursors([(4, 1)]), w[1:2], u, s_b, k[1:2], v[1:2], r[1:2], x[1:2])
+    assert np.array_equal(two, np.concatenate([first, second])) and np.array_equal(s_a, s_b)
+
+
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_gpu_token_shift_channel_mix(gpu, lop, dtype):
+    import torch
+
+    print("token shift / channel mix on the GPU", dtype.__name__, flush=True)
+    rng = np.random.default_rng(SEED + 50)
+    C, B, L = 256, 6, 3
+    cur = lop.pack_cursors(RUNS)
+    A = len(cur)
+    curd = torch.from_numpy(cur.view(np.int32)).cuda()
+    x = rng.standard_normal((A, C)).astype(dtype)
+    # the state of a model: [C, rows per layer * layers, B]; this layer's row is picked by the view
+    rows = 2 * L
+    state = rng.standard_normal((B, rows, C)).astype(np.float32)
+    row = 3
+    sview = ((C, 1, B), (C, rows, B), (0, row, 0))
+    sd = torch.from_numpy(state.copy()).cuda()
+    xd = torch.from_numpy(x).cuda()
+    tm = rng.random((1, 1, C)).astype(np.float16)
+    for rev in (True, False):
+        for ot in (np.float16, np.float32):
+            out = torch.empty((1, A, C), dtype=torch.float16 if ot == np.float16 else torch.float32, device="cuda")
+            gpu.LayerOp.token_shift(curd, torch.from_numpy(tm).cuda(), sd, xd.reshape(1, A, C), out, rev, state_view=sview)
+            want = lop.token_shift(cur, tm.reshape(C), state[:, row], x, ot, reversed=rev)
+            assert_close(out.cpu().numpy(), want, 1e-3 if ot == np.float16 else 1e-6, f"token shift {rev} {ot.__name__}")
+    tm5 = rng.random((5, A, C)).astype(np.float32)
+    out5 = torch.empty((5, A, C), dtype=torch.float16, device="cuda")
+    gpu.LayerOp.token_shift(curd, torch.from_numpy(tm5).cuda(), sd, xd.reshape(1, A, C), out5, True, state_view=sview)
+    assert_close(out5.cpu().numpy(), lop.token_shift(cur, tm5, state[:, row], x, np.float16, counts=5, reversed=True), 1e-3, "five shifts")
+    r = rng.standard_normal((A, C)).astype(dtype)
+    v = rng.standard_normal((A, C)).astype(dtype)
+    st = state[:, row].copy()
+    want = lop.channel_mix(cur, st, r, v, x)
+    xm = torch.from_numpy(x.copy()).cuda().reshape(1, A, C)
+    gpu.LayerOp.channel_mix(curd, sd, torch.from_numpy(r).cuda().reshape(1, A, C), torch.from_numpy(v).cuda().reshape(1, A, C), xm, state_view=sview)
+    assert_close(xm.cpu().numpy()[0], want, 1e-3 if dtype == np.float16 else 1e-6, "channel mix")
+    want_state = state.copy()
+    want_state[:, row] = st
+    assert np.array_equal(sd.cpu().numpy(), want_state)  # only this layer's row of the requests in the stack changed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("H,S,runs", [(3, 16, RUNS), (4, 64, RUNS), (64, 64, [(0, 1)]), (2, 128, [(1, 2), (3, 2)]), (8, 64, [(b, 1) for b in range(6)]), (2, 64, [(4, 100)])])
+def test_gpu_time_mix_v6(gpu, lop, dtype, H, S, runs):
+    import torch
+
+    print("time mix v6 on the GPU", dtype.__name__, H, S, runs[:3], flush=True)
+    rng = np.random.default_rng(SEED + 60 + H + S)
+    B = 6
+    cur = lop.pack_cursors(runs)
+    A = len(cur)
+    k, v, r, x, w, u, state = wkv6_inputs(rng, A, H, S, B, dtype)
+    # the model's state tensor holds S + 1 rows per layer; layer 1 of 2 is used here
+    full = np.concatenate([np.zeros_like(state), state], axis=1)
+    sview = ((H * S, S + 1, B), (H * S, 2 * (S + 1), B), (0, S + 1, 0))
+    sd = torch.from_numpy(full.copy()).cuda()
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.time_mix_v6(torch.from_numpy(cur.view(np.int32)).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(u).cuda(), sd,
+                            torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), torch.from_numpy(r).cuda(), xd, state_view=sview)
+    want, want_state = wkv6_float64(cur, w, u, state, k, v, r, x)
+    eps = 2e-3 if dtype == np.float16 else 2e-5
+    assert_close(xd.cpu().numpy(), want, eps, "y vs float64")
+    got_state = sd.cpu().numpy()
+    assert_close(got_state[:, S + 1:], want_state, 2e-5, "state vs float64")
+    assert np.array_equal(got_state[:, :S + 1], full[:, :S + 1])  # the other layer's rows are untouched
+    if A * H * S * S <= 2000000:
+        st = state.copy()
+        assert_close(xd.cpu().numpy(), lop.time_mix_v6(cur, w, u, st, k, v, r, x), eps, "y vs oracle")
+        assert_close(got_state[:, S + 1:], st, 2e-5, "state vs oracle")
+
+
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_data_movement_kats(gpu):

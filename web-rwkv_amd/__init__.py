@@ -43,6 +43,7 @@ EXPORTS = [
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
+    "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v6",
 ]
 MAX_GROUP = 8
 
@@ -193,6 +194,9 @@ def lib():
         L.wrq_activate.argtypes = [vp, V, i]
         L.wrq_affine.argtypes = [vp, T, i, C.c_float, C.c_float]
         L.wrq_lerp.argtypes = [vp, V, V, V, i]
+        L.wrq_token_shift.argtypes = [vp, T, V, V, T, i, T, i, i]
+        L.wrq_channel_mix.argtypes = [vp, T, V, T, T, T, i]
+        L.wrq_time_mix_v6.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -331,6 +335,22 @@ class LayerOp:
     @staticmethod
     def affine(x, scale, bias):
         _check(lib().wrq_affine(_stream(), C.byref(as_tensor(x)), _dtype(x), scale, bias))
+
+    @staticmethod
+    def token_shift(cursors, time_mix, state, input, output, reversed=False, time_mix_view=None, state_view=None):
+        _check(lib().wrq_token_shift(_stream(), C.byref(as_tensor(cursors)), C.byref(as_view(time_mix, time_mix_view)), C.byref(as_view(state, state_view)),
+                                     C.byref(as_tensor(input)), _dtype(input), C.byref(as_tensor(output)), _dtype(output), int(reversed)))
+
+    @staticmethod
+    def channel_mix(cursors, state, r, v, x, state_view=None):
+        _check(lib().wrq_channel_mix(_stream(), C.byref(as_tensor(cursors)), C.byref(as_view(state, state_view)), C.byref(as_tensor(r)),
+                                     C.byref(as_tensor(v)), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def time_mix_v6(cursors, time_decay, time_first, state, k, v, r, x, state_view=None):
+        _check(lib().wrq_time_mix_v6(_stream(), C.byref(as_tensor(cursors)), C.byref(as_tensor(time_decay)), C.byref(as_tensor(time_first)),
+                                     C.byref(as_view(state, state_view)), C.byref(as_tensor(k)), C.byref(as_tensor(v)), C.byref(as_tensor(r)),
+                                     C.byref(as_tensor(x)), _dtype(x)))
 
     @staticmethod
     def lerp(input, output, factor, reversed=False, input_view=None, output_view=None, factor_view=None):

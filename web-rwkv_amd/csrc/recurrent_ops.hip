@@ -1,0 +1,303 @@
+// The ops of a v6 layer that carry state from token to token:
+//   token_shift   src/tensor/ops.rs:1393-1462, src/shaders/token_shift.wgsl
+//   channel_mix   src/tensor/ops.rs:1860-1915, src/shaders/channel_mix.wgsl
+//   time_mix_v6   src/tensor/ops.rs:1601-1677, src/shaders/time_mix_v6.wgsl
+//
+// A run is a stack of A tokens from several requests; `cursors[a]` packs, for the request of token
+// a, its state slot (8 bits), the position of its first token in the stack (16 bits) and the number
+// of its tokens in the stack (8 bits) (`compute_cursor` of the shaders).
+//
+// time_mix_v6 is the recurrence  y[i] = sum_j r[j] (u[j] k[j] v[i] + S[j][i]),  S[j][i] <- w[j] S[j][i] + k[j] v[i]
+// per head, token after token.  The shader re-reads and re-writes the head's S (64 x 64 f32) in memory
+// for every token; here a request's S stays in registers for all its tokens of the run: four lanes
+// share an output element i and hold a quarter of j each (16 values of S), one DPP quad reduction
+// per token, no LDS and no barrier; S is read when a request's tokens begin and written when they
+// end.  The sum over j is therefore taken in four interleaved partial sums instead of one chain
+// (a difference of rounding order only).
+#include "wrq_device.h"
+#include "wrq_host.h"
+
+namespace wrq {
+
+namespace {
+
+struct ViewArgs {
+    uint32_t shape[4], stride[4], offset[4];
+};
+
+ViewArgs view_args(const wrq_view &v) {
+    ViewArgs a;
+    for (int i = 0; i < 4; i++) a.shape[i] = v.shape[i], a.stride[i] = v.stride[i], a.offset[i] = v.offset[i];
+    return a;
+}
+
+// element index (units of 1 element) of (batch, token, element) in a view: compute_index of the shaders
+__device__ __forceinline__ uint64_t view_elem(const ViewArgs &v, uint32_t batch, uint32_t token, uint32_t elem) {
+    return ((uint64_t)(batch + v.offset[2]) * v.stride[1] + (token + v.offset[1])) * v.stride[0] + elem + v.offset[0];
+}
+
+template <typename XT>
+__device__ __forceinline__ float4 load_vec4(const XT *p) {
+    if constexpr (sizeof(XT) == 2) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
+    } else {
+        return *reinterpret_cast<const float4 *>(p);
+    }
+}
+
+template <typename XT>
+__device__ __forceinline__ void store_vec4(XT *p, float4 v) {
+    if constexpr (sizeof(XT) == 2) {
+        *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f2h(v.x) | ((uint32_t)f2h(v.y) << 16), (uint32_t)f2h(v.z) | ((uint32_t)f2h(v.w) << 16));
+    } else {
+        *reinterpret_cast<float4 *>(p) = v;
+    }
+}
+
+template <typename XT>
+__device__ __forceinline__ float load_one(const XT *p) {
+    if constexpr (sizeof(XT) == 2) return h2f(*p);
+    else return *p;
+}
+
+struct Cursor {
+    uint32_t batch, token, len;
+};
+__device__ __forceinline__ Cursor unpack_cursor(uint32_t x) { return Cursor{x & 0xffu, (x >> 8) & 0xffffu, (x >> 24) & 0xffu}; }
+// Cursors live in device memory, the host cannot check them: a state slot beyond the view is clamped
+// to its last slot and a first token beyond the token itself counts as the token itself, so that a
+// malformed cursor reads and writes inside the tensors (the shaders rely on WebGPU's bounds clamping).
+__device__ __forceinline__ Cursor read_cursor(const uint32_t *cursors, uint32_t stack, const ViewArgs &vs) {
+    Cursor c = unpack_cursor(cursors[stack]);
+    c.batch = min(c.batch, vs.shape[2] - 1);
+    c.token = min(c.token, stack);
+    return c;
+}
+
+// output[count][stack] = mix(previous token, this token, time_mix) (reversed: the two swapped); the
+// previous token of a request's first token in the stack is its state row
+template <typename FT, typename IT, typename OT>
+__global__ __launch_bounds__(256) void token_shift_kernel(const uint32_t *cursors, const FT *time_mix, const float *state, const IT *input, OT *output,
+                                                          ViewArgs vt, ViewArgs vs, uint32_t C, uint32_t A, int reversed) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, stack = blockIdx.y, count = blockIdx.z;
+    if (index >= C / 4) return;
+    const Cursor cur = read_cursor(cursors, stack, vs);
+    const float4 f = load_vec4(time_mix + view_elem(vt, count, vt.shape[1] == 1 ? 0u : stack, 4 * index));
+    const float4 x = load_vec4(input + ((uint64_t)stack * C + 4 * index));
+    const float4 p = stack == cur.token ? load_vec4(state + view_elem(vs, cur.batch, 0, 4 * index)) : load_vec4(input + ((uint64_t)(stack - 1) * C + 4 * index));
+    // mix(a, b, t) = a (1 - t) + b t
+    auto mix = [&](float a, float b, float t) { return reversed ? a * (1.0f - t) + b * t : b * (1.0f - t) + a * t; };
+    store_vec4(output + (((uint64_t)count * A + stack) * C + 4 * index), make_float4(mix(x.x, p.x, f.x), mix(x.y, p.y, f.y), mix(x.z, p.z, f.z), mix(x.w, p.w, f.w)));
+}
+
+// state[request] <- x at the request's last token of the stack; x <- sigmoid(r) * v
+template <typename XT>
+__global__ __launch_bounds__(256) void channel_mix_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *v, XT *x, ViewArgs vs, uint32_t C) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, stack = blockIdx.y;
+    if (index >= C / 4) return;
+    const Cursor cur = read_cursor(cursors, stack, vs);
+    const uint64_t bti = (uint64_t)stack * C + 4 * index;
+    if (stack - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = load_vec4(x + bti);
+    const float4 rr = load_vec4(r + bti), vv = load_vec4(v + bti);
+    auto g = [](float a, float b) { return 1.0f / (1.0f + expf(-a)) * b; };
+    store_vec4(x + bti, make_float4(g(rr.x, vv.x), g(rr.y, vv.y), g(rr.z, vv.z), g(rr.w, vv.w)));
+}
+
+__device__ __forceinline__ float quad_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true)); // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true)); // quad_perm [2,3,0,1]
+    return v;
+}
+
+// One workgroup per head: thread = (output element i of the head, quarter q of the j range), four
+// waves of 16 i x 4 q.  S = head size (a multiple of 16, at most 256: JQ = S / 4 values of S per lane).
+template <typename XT, int JQ>
+__global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursors, const float *time_decay, const float *time_first, float *state, const XT *k,
+                                                          const XT *v, const XT *r, XT *x, ViewArgs vs, uint32_t S, uint32_t H, uint32_t A) {
+    const uint32_t head = blockIdx.x;
+    const uint32_t q = threadIdx.x & 3;
+    const uint32_t C = S * H;
+    for (uint32_t i = threadIdx.x >> 2; i < S; i += 64) {
+        const uint32_t chan = head * S + i; // channel of this output element
+        float u[JQ], s[JQ];
+#pragma unroll
+        for (int jj = 0; jj < JQ; jj++) u[jj] = time_first[head * S + q * JQ + jj];
+        uint32_t held = 0xffffffffu; // request whose S is in registers
+        for (uint32_t t = 0; t < A; t++) {
+            const Cursor cur = read_cursor(cursors, t, vs);
+            if (cur.batch != held) {
+                if (held != 0xffffffffu) {
+#pragma unroll
+                    for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
+                }
+                held = cur.batch;
+#pragma unroll
+                for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
+            }
+            const uint64_t ti = (uint64_t)t * C + head * S;
+            // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
+            if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti + i);
+            const float vv = load_one(v + ti + i);
+            float y = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < JQ; jj++) {
+                const uint32_t j = q * JQ + jj;
+                const float kk = load_one(k + ti + j), rr = load_one(r + ti + j), ww = time_decay[ti + j];
+                const float kv = kk * vv;
+                y += rr * fmaf(u[jj], kv, s[jj]);
+                s[jj] = fmaf(ww, s[jj], kv);
+            }
+            y = quad_sum(y);
+            if (q == 0) {
+                if constexpr (sizeof(XT) == 2) x[ti + i] = f2h(y);
+                else x[ti + i] = y;
+            }
+        }
+        if (held != 0xffffffffu) {
+#pragma unroll
+            for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
+        }
+    }
+}
+
+int check_view(const wrq_tensor_view *t, const char *what) {
+    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
+    if (t->dtype != WRQ_F16 && t->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, (int)t->dtype);
+    for (int i = 0; i < 4; i++)
+        if ((uint64_t)t->view.offset[i] + t->view.shape[i] > t->view.stride[i]) return fail(WRQ_ERR_SHAPE, "%s: slice out of range", what);
+    if (t->view.shape[0] % 4 || t->view.stride[0] % 4 || t->view.offset[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "%s: rows not in units of 4 elements", what);
+    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
+    return WRQ_OK;
+}
+
+int check_tensor(const wrq_tensor *t, const char *what) {
+    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
+    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
+    return WRQ_OK;
+}
+
+bool same_shape(const uint32_t *a, const uint32_t *b) { return a[0] == b[0] && a[1] == b[1] && a[2] == b[2] && a[3] == b[3]; }
+
+template <typename FT, typename IT>
+int token_shift_out(hipStream_t stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix, const wrq_tensor_view *state, const wrq_tensor *input,
+                    const wrq_tensor *output, int out_dtype, dim3 grid, int reversed) {
+    const ViewArgs vt = view_args(time_mix->view), vs = view_args(state->view);
+    const uint32_t C = output->shape[0], A = output->shape[1];
+    const uint32_t *cur = static_cast<const uint32_t *>(cursors->data);
+    if (out_dtype == WRQ_F16)
+        hipLaunchKernelGGL((token_shift_kernel<FT, IT, uint16_t>), grid, dim3(256), 0, stream, cur, static_cast<const FT *>(time_mix->data), static_cast<const float *>(state->data),
+                           static_cast<const IT *>(input->data), static_cast<uint16_t *>(output->data), vt, vs, C, A, reversed);
+    else
+        hipLaunchKernelGGL((token_shift_kernel<FT, IT, float>), grid, dim3(256), 0, stream, cur, static_cast<const FT *>(time_mix->data), static_cast<const float *>(state->data),
+                           static_cast<const IT *>(input->data), static_cast<float *>(output->data), vt, vs, C, A, reversed);
+    return check_launch("token_shift");
+}
+
+} // namespace
+
+} // namespace wrq
+
+using namespace wrq;
+
+extern "C" {
+
+int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix, const wrq_tensor_view *state, const wrq_tensor *input,
+                    wrq_dtype input_dtype, const wrq_tensor *output, wrq_dtype output_dtype, int reversed) {
+    int s = check_tensor(cursors, "token_shift");
+    if (s == WRQ_OK) s = check_tensor(input, "token_shift");
+    if (s == WRQ_OK) s = check_tensor(output, "token_shift");
+    if (s == WRQ_OK) s = check_view(time_mix, "token_shift");
+    if (s == WRQ_OK) s = check_view(state, "token_shift");
+    if (s != WRQ_OK) return s;
+    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "token_shift: the state is f32");
+    for (int d : {(int)input_dtype, (int)output_dtype})
+        if (d != WRQ_F16 && d != WRQ_F32) return fail(WRQ_ERR_TYPE, "token_shift: unsupported element type %d", d);
+    const uint32_t *o = output->shape, *i = input->shape, *t = time_mix->view.shape, *st = state->view.shape;
+    // src/tensor/ops.rs:1409-1414
+    const bool ok = o[3] == 1 && i[0] == o[0] && i[1] == o[1] && (i[2] == o[2] || i[2] == 1) && i[3] == 1 &&
+                    ((t[0] == o[0] && t[1] == o[1] && t[2] == o[2] && t[3] == 1) || (t[0] == o[0] && t[1] == 1 && t[2] == 1 && t[3] == 1)) && st[0] == o[0] && st[3] == 1;
+    if (!ok) return fail(WRQ_ERR_SHAPE, "token_shift: data shape not match [%u, %u, %u, %u]", o[0], o[1], o[2], o[3]);
+    if (cursors->shape[0] < o[1]) return fail(WRQ_ERR_SHAPE, "token_shift: %u cursors for %u tokens", cursors->shape[0], o[1]);
+    if (o[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "token_shift: row length %u not a multiple of 4", o[0]);
+    if (o[0] == 0 || o[1] == 0 || o[2] == 0) return WRQ_OK;
+    if (o[1] > 65535u || o[2] > 65535u) return fail(WRQ_ERR_SIZE, "token_shift: data size not match");
+    const dim3 grid((o[0] / 4 + 255) / 256, o[1], o[2]);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const bool f16 = time_mix->dtype == WRQ_F16, i16 = input_dtype == WRQ_F16;
+    if (f16 && i16) return token_shift_out<uint16_t, uint16_t>(hs, cursors, time_mix, state, input, output, output_dtype, grid, reversed);
+    if (f16) return token_shift_out<uint16_t, float>(hs, cursors, time_mix, state, input, output, output_dtype, grid, reversed);
+    if (i16) return token_shift_out<float, uint16_t>(hs, cursors, time_mix, state, input, output, output_dtype, grid, reversed);
+    return token_shift_out<float, float>(hs, cursors, time_mix, state, input, output, output_dtype, grid, reversed);
+}
+
+int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state, const wrq_tensor *r, const wrq_tensor *v, const wrq_tensor *x,
+                    wrq_dtype dtype) {
+    int s = check_tensor(cursors, "channel_mix");
+    for (const wrq_tensor *t : {r, v, x})
+        if (s == WRQ_OK) s = check_tensor(t, "channel_mix");
+    if (s == WRQ_OK) s = check_view(state, "channel_mix");
+    if (s != WRQ_OK) return s;
+    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: the state is f32");
+    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: unsupported element type %d", (int)dtype);
+    const uint32_t *sh = x->shape, *st = state->view.shape;
+    // src/tensor/ops.rs:1873-1877
+    if (!same_shape(r->shape, sh) || !same_shape(v->shape, sh) || st[0] != sh[0] || st[1] != 1 || st[3] != 1 || sh[2] != 1 || sh[3] != 1)
+        return fail(WRQ_ERR_SHAPE, "channel_mix: data shape not match [%u, %u, %u, %u]", sh[0], sh[1], sh[2], sh[3]);
+    if (cursors->shape[0] < sh[1]) return fail(WRQ_ERR_SHAPE, "channel_mix: %u cursors for %u tokens", cursors->shape[0], sh[1]);
+    if (sh[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "channel_mix: row length %u not a multiple of 4", sh[0]);
+    if (sh[0] == 0 || sh[1] == 0) return WRQ_OK;
+    if (sh[1] > 65535u) return fail(WRQ_ERR_SIZE, "channel_mix: data size not match");
+    const dim3 grid((sh[0] / 4 + 255) / 256, sh[1]);
+    const ViewArgs vs = view_args(state->view);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const uint32_t *cur = static_cast<const uint32_t *>(cursors->data);
+    if (dtype == WRQ_F16)
+        hipLaunchKernelGGL((channel_mix_kernel<uint16_t>), grid, dim3(256), 0, hs, cur, static_cast<float *>(state->data), static_cast<const uint16_t *>(r->data),
+                           static_cast<const uint16_t *>(v->data), static_cast<uint16_t *>(x->data), vs, sh[0]);
+    else
+        hipLaunchKernelGGL((channel_mix_kernel<float>), grid, dim3(256), 0, hs, cur, static_cast<float *>(state->data), static_cast<const float *>(r->data),
+                           static_cast<const float *>(v->data), static_cast<float *>(x->data), vs, sh[0]);
+    return check_launch("channel_mix");
+}
+
+int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
+                    const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
+    int s = check_tensor(cursors, "time_mix_v6");
+    for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
+        if (s == WRQ_OK) s = check_tensor(t, "time_mix_v6");
+    if (s == WRQ_OK) s = check_view(state, "time_mix_v6");
+    if (s != WRQ_OK) return s;
+    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: the state is f32");
+    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: unsupported element type %d", (int)dtype);
+    const uint32_t *sh = x->shape, *st = state->view.shape; // [S, H, A, 1]
+    const uint32_t S = sh[0], H = sh[1], A = sh[2];
+    // src/tensor/ops.rs:1620-1625
+    const uint32_t tf[4] = {S, H, 1, 1};
+    if (sh[3] != 1 || !same_shape(k->shape, sh) || !same_shape(v->shape, sh) || !same_shape(r->shape, sh) || !same_shape(time_decay->shape, sh) ||
+        !same_shape(time_first->shape, tf) || st[0] != S * H || st[1] != S + 1 || st[3] != 1)
+        return fail(WRQ_ERR_SHAPE, "time_mix_v6: data shape not match [%u, %u, %u, %u]", sh[0], sh[1], sh[2], sh[3]);
+    if (cursors->shape[0] < A) return fail(WRQ_ERR_SHAPE, "time_mix_v6: %u cursors for %u tokens", cursors->shape[0], A);
+    if (S == 0 || H == 0 || A == 0) return WRQ_OK;
+    if (S % 16 || S > 256) return fail(WRQ_ERR_UNSUPPORTED, "time_mix_v6: head size %u (a multiple of 16 up to 256 is built)", S);
+    const ViewArgs vs = view_args(state->view);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const uint32_t *cur = static_cast<const uint32_t *>(cursors->data);
+    const float *td = static_cast<const float *>(time_decay->data), *tfp = static_cast<const float *>(time_first->data);
+    float *sp = static_cast<float *>(state->data);
+#define WRQ_TM(JQ)                                                                                                                                           \
+    if (S == 4 * JQ) {                                                                                                                                       \
+        if (dtype == WRQ_F16)                                                                                                                                \
+            hipLaunchKernelGGL((time_mix_v6_kernel<uint16_t, JQ>), dim3(H), dim3(256), 0, hs, cur, td, tfp, sp, static_cast<const uint16_t *>(k->data),      \
+                               static_cast<const uint16_t *>(v->data), static_cast<const uint16_t *>(r->data), static_cast<uint16_t *>(x->data), vs, S, H, A); \
+        else                                                                                                                                                 \
+            hipLaunchKernelGGL((time_mix_v6_kernel<float, JQ>), dim3(H), dim3(256), 0, hs, cur, td, tfp, sp, static_cast<const float *>(k->data),            \
+                               static_cast<const float *>(v->data), static_cast<const float *>(r->data), static_cast<float *>(x->data), vs, S, H, A);        \
+        return check_launch("time_mix_v6");                                                                                                                  \
+    }
+    WRQ_TM(4) WRQ_TM(8) WRQ_TM(16) WRQ_TM(32) WRQ_TM(64)
+#undef WRQ_TM
+    return fail(WRQ_ERR_UNSUPPORTED, "time_mix_v6: head size %u (16, 32, 64, 128 or 256 is built)", S);
+}
+
+} // extern "C"
