@@ -388,6 +388,98 @@ def schedule(wrq, torch, args, layers, C, H):
     print(json.dumps(out), flush=True)
 
 
+def full_layers(wrq, torch, args, C, H):
+    """Every op of the v6 layers, dispatched like the reference (src/runtime/v6.rs:758-955): 35 ops
+    per layer, 8 of them the quantized products.  One run of `--tokens` tokens of one request per
+    step, replayed from a HIP graph.  Model tok/s without embedding and head."""
+    v6 = importlib.import_module("web-rwkv_amd.v6")
+    heads, S, slots = C // 64, 64, 4
+    rng = np.random.default_rng(SEED + 7)
+    layers, states = [], []
+    for i in range(args.layers):
+        layers.append(v6.Layer(torch, v6.random_layer_weights(rng, C, heads, S, H, layer=i), args.quant))
+        states.append(torch.zeros((slots, S + 2, C), dtype=torch.float32, device="cuda"))
+    A = args.tokens
+    buf = v6.Runtime(torch, C, H, A)
+    buf.x.copy_(torch.randn((1, A, C), device="cuda").half())
+    # one request in slot 0 whose A tokens fill the stack (the reference packs the count into 8 bits)
+    cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
+    x0 = buf.x.clone()
+
+    def step():
+        buf.x.copy_(x0)  # the embedding of the next token would land here
+        for i, (layer, st) in enumerate(zip(layers, states)):
+            v6.dispatch_layer(layer, buf, st, cursors, A, heads, S, rescale_now=(i + 1) % 6 == 0)
+
+    step()
+    torch.cuda.synchronize()
+    if args.no_graph:
+        fn = step
+    else:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        fn = graph.replay
+    ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
+    assert torch.isfinite(buf.x.float()).all()
+    print(json.dumps({"metric": "RWKV-v6 7B-shape layers, every op (no embedding, no head), tokens/s", "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
+                      "config": {"workload": f"{args.layers} v6 layers ({C} x {H}, {heads} heads), {args.quant}, {A} token(s) of one request per step, 35 ops per layer",
+                                 "hip_graph": not args.no_graph}, "data": "synthetic"}))
+
+
+def ops_table(wrq, torch, args, C):
+    """Time of every layer op alone at the 7B layer shape, A tokens (HIP graph of 20 calls)."""
+    LayerOp = wrq.LayerOp
+    A, S = args.tokens, 64
+    heads = C // S
+    h = lambda *s: torch.randn(s, device="cuda").half()
+    f = lambda *s: torch.randn(s, device="cuda")
+    cur = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
+    state = torch.zeros((4, S + 2, C), dtype=torch.float32, device="cuda")
+    att = ((C, S + 1, 4), (C, S + 2, 4), (0, 0, 0))
+    ffn = ((C, 1, 4), (C, S + 2, 4), (0, S + 1, 0))
+    x, y, w, b, x5, tm5 = h(1, A, C), h(1, A, C), h(C), h(C), h(5, A, C), h(5, A, C)
+    k, v, r, aux, decay, u = f(A, heads, S), f(A, heads, S), f(A, heads, S), f(A, heads, S), torch.rand((A, heads, S), device="cuda"), f(heads, S)
+    gw, gb = h(heads, S), h(heads, S)
+    cases = {
+        "layer_norm": (lambda: LayerOp.layer_norm(w, b, x, 1e-5), 2 * A * C * 2),
+        "group_norm": (lambda: LayerOp.group_norm(gw, gb, aux, 64e-5), 2 * A * C * 4),
+        "token_shift (1)": (lambda: LayerOp.token_shift(cur, w, state, x, y, True, state_view=att), 2 * A * C * 2),
+        "token_shift (5)": (lambda: LayerOp.token_shift(cur, tm5, state, x, x5, True, state_view=att), 11 * A * C * 2),
+        "add": (lambda: LayerOp.add(x, y), 3 * A * C * 2),
+        "mul_activate silu": (lambda: LayerOp.mul_activate(x, y, wrq.ACT_SILU), 3 * A * C * 2),
+        "blit f16 -> f32": (lambda: LayerOp.blit(x, aux.view(1, A, C)), A * C * 6),
+        "activate stable_exp": (lambda: LayerOp.activate(decay.view(1, A, C), wrq.ACT_STABLE_EXP), 2 * A * C * 4),
+        "channel_mix": (lambda: LayerOp.channel_mix(cur, state, x, y, x5[0:1], state_view=ffn), 4 * A * C * 2),
+        "time_mix_v6": (lambda: LayerOp.time_mix_v6(cur, decay, u, state, k, v, r, aux, state_view=att), 5 * A * C * 4 + 2 * S * C * 4),
+        "softmax (65536)": (lambda: LayerOp.softmax(f(1, 1, 65536)), 0),
+    }
+    for name, (fn, nbytes) in cases.items():
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        if name.startswith("softmax"):
+            logits = f(1, 1, 65536)
+            fn = lambda: LayerOp.softmax(logits)
+            nbytes = 2 * 65536 * 4
+            fn()
+            torch.cuda.synchronize()
+        with torch.cuda.graph(g):
+            for _ in range(20):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 200
+        print(json.dumps({"op": name, "tokens": A, "us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -407,6 +499,8 @@ def main():
     ap.add_argument("--with-head", action="store_true", help="add the fp16 head (65536 x 4096, matmul_vec_fp16 / matmul_mat_fp16) to every step")
     ap.add_argument("--schedule", action="store_true", help="config 5: multi-slot serving schedule (use with --quant nf4) instead of one step size")
     ap.add_argument("--slots", type=int, default=32)
+    ap.add_argument("--full-layers", action="store_true", help="every op of the v6 layers (35 per layer), not only the quantized products")
+    ap.add_argument("--ops", action="store_true", help="time of every layer op alone at the 7B layer shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
@@ -424,6 +518,12 @@ def main():
     probe = run_probe(torch) if args.probe else None
 
     C, H = 4096, 14336
+    if args.ops:
+        ops_table(wrq, torch, args, C)
+        return
+    if args.full_layers:
+        full_layers(wrq, torch, args, C, H)
+        return
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
     if args.schedule:
         schedule(wrq, torch, args, layers, C, H)

@@ -616,7 +616,8 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
 // activations through converts and fmas.  HBM-bound: 2 bytes per weight.
 // TT > 1 (f16 activations only): tokens token .. token + TT - 1 of a short run share the pass.
 template <typename XT, int ROWS, int NT, int TT>
-__global__ __launch_bounds__(NT) void gemv_fp16_oneshot_kernel(const MatmulArgs a, uint32_t token) {
+__global__ __launch_bounds__(NT) void gemv_fp16_oneshot_kernel(const MatmulArgs a, uint32_t first_token) {
+    const uint32_t token = first_token + blockIdx.z * TT; // grid.z: consecutive groups of TT tokens
     static_assert(TT == 1 || sizeof(XT) == 2, "several tokens per pass: f16 activations only");
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     constexpr bool F16 = sizeof(XT) == 2;
@@ -1029,8 +1030,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
 }
 
 template <typename XT, int ROWS, int TT>
-void launch_fp16_nt(hipStream_t stream, const MatmulArgs &a, uint32_t token, int nt) {
-    const dim3 grid((a.R + ROWS - 1) / ROWS, a.B);
+void launch_fp16_nt(hipStream_t stream, const MatmulArgs &a, uint32_t token, int nt, uint32_t groups = 1) {
+    const dim3 grid((a.R + ROWS - 1) / ROWS, a.B, groups);
     if (nt >= 512)
         hipLaunchKernelGGL((gemv_fp16_oneshot_kernel<XT, ROWS, 512, TT>), grid, dim3(512), 0, stream, a, token);
     else if (nt >= 256)
@@ -1061,7 +1062,12 @@ int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &a) {
     // f16 activations: up to 4 tokens per pass over the weights; f32: one
     for (uint32_t t = 0; t < a.T;) {
         const uint32_t left = a.T - t;
-        if (in_f16 && left >= 3) {
+        if (in_f16 && left >= 4) {
+            // whole groups of 4 tokens in one launch (long runs come here when K rules out the matrix cores)
+            const uint32_t groups = left / 4;
+            if (rows8) launch_fp16_nt<__half, 8, 4>(stream, a, t, nt, groups); else launch_fp16_nt<__half, 4, 4>(stream, a, t, nt, groups);
+            t += 4 * groups;
+        } else if (in_f16 && left == 3) {
             if (rows8) launch_fp16_nt<__half, 8, 4>(stream, a, t, nt); else launch_fp16_nt<__half, 4, 4>(stream, a, t, nt);
             t += 4;
         } else if (in_f16 && left == 2) {

@@ -112,49 +112,101 @@ __device__ __forceinline__ float quad_sum(float v) {
 
 // One workgroup per head: thread = (output element i of the head, quarter q of the j range), four
 // waves of 16 i x 4 q.  S = head size (a multiple of 16, at most 256: JQ = S / 4 values of S per lane).
+// One workgroup per head: thread = (output element i of the head, quarter q of the j range), four
+// waves of 16 i x 4 q; JQ = S / 4 values of S[.][i] per lane.  The operands of the head (k, r, w, v:
+// S values each per token) come in chunks of 1024 / S tokens: every thread fetches one 4-element
+// vector of each while the previous chunk is worked on, and the chunk is passed round through LDS
+// (two buffers), from where the lanes of a quarter read their j range as broadcasts.
 template <typename XT, int JQ>
 __global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursors, const float *time_decay, const float *time_first, float *state, const XT *k,
                                                           const XT *v, const XT *r, XT *x, ViewArgs vs, uint32_t S, uint32_t H, uint32_t A) {
-    const uint32_t head = blockIdx.x;
-    const uint32_t q = threadIdx.x & 3;
+    constexpr int SZ = 4 * JQ;      // head size
+    constexpr int TB = 1024 / SZ;   // tokens per chunk
+    __shared__ __align__(16) float ks[2][1024], rs[2][1024], ws[2][1024], vsh[2][1024];
+    __shared__ uint32_t csh[2][TB]; // the chunk's cursors
+    const uint32_t head = blockIdx.x, tid = threadIdx.x;
+    const uint32_t q = tid & 3;
     const uint32_t C = S * H;
-    for (uint32_t i = threadIdx.x >> 2; i < S; i += 64) {
-        const uint32_t chan = head * S + i; // channel of this output element
+    const uint32_t nchunk = (A + TB - 1) / TB;
+    // this thread's vector of a chunk: token tid / (SZ / 4) of the chunk, elements 4 (tid % (SZ / 4)) ..
+    const uint32_t lt = tid / (SZ / 4), le = 4 * (tid % (SZ / 4));
+    float4 fk, fr, fw, fv;
+    uint32_t fc = 0;
+    auto fetch = [&](uint32_t chunk) {
+        const uint32_t t = min(chunk * TB + lt, A - 1); // clamped: tokens past the run are never used
+        const uint64_t g = (uint64_t)t * C + head * SZ + le;
+        fk = load_vec4(k + g), fr = load_vec4(r + g), fw = load_vec4(time_decay + g), fv = load_vec4(v + g);
+        if (tid < (uint32_t)TB) fc = cursors[min(chunk * TB + tid, A - 1)];
+    };
+    auto stage = [&](int buf) {
+        *reinterpret_cast<float4 *>(&ks[buf][4 * tid]) = fk;
+        *reinterpret_cast<float4 *>(&rs[buf][4 * tid]) = fr;
+        *reinterpret_cast<float4 *>(&ws[buf][4 * tid]) = fw;
+        *reinterpret_cast<float4 *>(&vsh[buf][4 * tid]) = fv;
+        if (tid < (uint32_t)TB) csh[buf][tid] = fc;
+    };
+    for (uint32_t i0 = 0; i0 < SZ; i0 += 64) {
+        const uint32_t i = i0 + (tid >> 2);
+        const bool live = i < SZ; // head sizes below 64 leave waves without an output element
+        const uint32_t chan = head * SZ + min(i, (uint32_t)SZ - 1);
         float u[JQ], s[JQ];
 #pragma unroll
-        for (int jj = 0; jj < JQ; jj++) u[jj] = time_first[head * S + q * JQ + jj];
-        uint32_t held = 0xffffffffu; // request whose S is in registers
-        for (uint32_t t = 0; t < A; t++) {
-            const Cursor cur = read_cursor(cursors, t, vs);
-            if (cur.batch != held) {
-                if (held != 0xffffffffu) {
-#pragma unroll
-                    for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
-                }
-                held = cur.batch;
-#pragma unroll
-                for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
-            }
-            const uint64_t ti = (uint64_t)t * C + head * S;
-            // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
-            if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti + i);
-            const float vv = load_one(v + ti + i);
-            float y = 0.0f;
-#pragma unroll
-            for (int jj = 0; jj < JQ; jj++) {
-                const uint32_t j = q * JQ + jj;
-                const float kk = load_one(k + ti + j), rr = load_one(r + ti + j), ww = time_decay[ti + j];
-                const float kv = kk * vv;
-                y += rr * fmaf(u[jj], kv, s[jj]);
-                s[jj] = fmaf(ww, s[jj], kv);
-            }
-            y = quad_sum(y);
-            if (q == 0) {
-                if constexpr (sizeof(XT) == 2) x[ti + i] = f2h(y);
-                else x[ti + i] = y;
-            }
+        for (int c = 0; c < JQ / 4; c++) {
+            const float4 t4 = *reinterpret_cast<const float4 *>(time_first + head * SZ + q * JQ + 4 * c);
+            u[4 * c] = t4.x, u[4 * c + 1] = t4.y, u[4 * c + 2] = t4.z, u[4 * c + 3] = t4.w;
         }
-        if (held != 0xffffffffu) {
+        uint32_t held = 0xffffffffu; // request whose S is in registers
+        fetch(0);
+        __syncthreads(); // the buffers may still be read by the previous pass over i
+        stage(0);
+        for (uint32_t chunk = 0; chunk < nchunk; chunk++) {
+            const int buf = chunk & 1;
+            if (chunk + 1 < nchunk) fetch(chunk + 1);
+            __syncthreads(); // chunk `chunk` is in LDS; buffer buf ^ 1 is free
+            const uint32_t tend = min((uint32_t)TB, A - chunk * TB);
+            if (live) {
+                for (uint32_t tt = 0; tt < tend; tt++) {
+                    const uint32_t t = chunk * TB + tt;
+                    Cursor cur = unpack_cursor(csh[buf][tt]);
+                    cur.batch = min(cur.batch, vs.shape[2] - 1); // as read_cursor
+                    cur.token = min(cur.token, t);
+                    if (cur.batch != held) {
+                        if (held != 0xffffffffu) {
+#pragma unroll
+                            for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
+                        }
+                        held = cur.batch;
+#pragma unroll
+                        for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
+                    }
+                    const uint64_t ti = (uint64_t)t * C + chan;
+                    // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
+                    if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti);
+                    const float vv = vsh[buf][tt * SZ + i];
+                    const float *kp = &ks[buf][tt * SZ + q * JQ], *rp = &rs[buf][tt * SZ + q * JQ], *wp = &ws[buf][tt * SZ + q * JQ];
+                    float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // four chains instead of one of JQ dependent adds
+#pragma unroll
+                    for (int c = 0; c < JQ / 4; c++) {
+                        const float4 k4 = *reinterpret_cast<const float4 *>(kp + 4 * c), r4 = *reinterpret_cast<const float4 *>(rp + 4 * c),
+                                     w4 = *reinterpret_cast<const float4 *>(wp + 4 * c);
+                        const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, rr[4] = {r4.x, r4.y, r4.z, r4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float kv = kk[e] * vv;
+                            y4[e] += rr[e] * fmaf(u[4 * c + e], kv, s[4 * c + e]);
+                            s[4 * c + e] = fmaf(ww[e], s[4 * c + e], kv);
+                        }
+                    }
+                    const float y = quad_sum((y4[0] + y4[1]) + (y4[2] + y4[3]));
+                    if (q == 0) {
+                        if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
+                        else x[ti] = y;
+                    }
+                }
+            }
+            if (chunk + 1 < nchunk) stage(buf ^ 1); // read two chunks ago, before the barrier above
+        }
+        if (live && held != 0xffffffffu) {
 #pragma unroll
             for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
         }

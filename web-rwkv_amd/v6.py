@@ -7,7 +7,7 @@ import importlib
 import numpy as np
 
 _pkg = importlib.import_module(__name__.rsplit(".", 1)[0])
-LayerOp, Matrix, turbo = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo
+LayerOp, Matrix, turbo, matmul_vec_group = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo, _pkg.matmul_vec_group
 ACT_NONE, ACT_SQUARED_RELU, ACT_TANH, ACT_STABLE_EXP, ACT_SILU = _pkg.ACT_NONE, _pkg.ACT_SQUARED_RELU, _pkg.ACT_TANH, _pkg.ACT_STABLE_EXP, _pkg.ACT_SILU
 
 LN_EPS = 1.0e-5   # Model::LN_EPS, src/runtime/v6.rs:46
@@ -90,10 +90,9 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now=False):
     m["time_mix_w2"].matmul_op(buf.time_mix_t, buf.time_mix, ACT_NONE, fast)
     LayerOp.add(t["time_mix"], buf.time_mix)
     LayerOp.token_shift(cursors, buf.time_mix, state, buf.att_x, buf.att_sx, True, state_view=att_state)
-    m["att_w_k"].matmul_op(buf.att_sx, buf.att_k, ACT_NONE, fast, input_view=slice_of(1))
-    m["att_w_v"].matmul_op(buf.att_sx, buf.att_v, ACT_NONE, fast, input_view=slice_of(2))
-    m["att_w_r"].matmul_op(buf.att_sx, buf.att_r, ACT_NONE, fast, input_view=slice_of(3))
-    m["att_w_g"].matmul_op(buf.att_sx, buf.att_g, ACT_NONE, fast, input_view=slice_of(4))
+    # the four independent projections in one call: the library's form of a `TensorOp::List` of them
+    matmul_vec_group([(m[n], buf.att_sx, out, ACT_NONE, False, dict(input_view=slice_of(i)))
+                      for n, out, i in (("att_w_k", buf.att_k, 1), ("att_w_v", buf.att_v, 2), ("att_w_r", buf.att_r, 3), ("att_w_g", buf.att_g, 4))])
     m["time_decay_w1"].matmul_op(buf.att_sx, buf.att_w, ACT_TANH, fast, input_view=slice_of(0))
     m["time_decay_w2"].matmul_op(buf.att_w, buf.time_decay, ACT_NONE, fast)
     LayerOp.add(t["time_decay"], buf.time_decay)
@@ -111,9 +110,8 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now=False):
     LayerOp.layer_norm(t["ffn_ln_w"], t["ffn_ln_b"], buf.ffn_x, LN_EPS)
     LayerOp.token_shift(cursors, t["ffn_time_mix_k"], state, buf.ffn_x, buf.ffn_kx, True, state_view=ffn_state)
     LayerOp.token_shift(cursors, t["ffn_time_mix_r"], state, buf.ffn_x, buf.ffn_rx, True, state_view=ffn_state)
-    m["ffn_w_k"].matmul_op(buf.ffn_kx, buf.ffn_k, ACT_SQUARED_RELU, fast)
+    matmul_vec_group([(m["ffn_w_k"], buf.ffn_kx, buf.ffn_k, ACT_SQUARED_RELU, False, {}), (m["ffn_w_r"], buf.ffn_rx, buf.ffn_r, ACT_NONE, False, {})])
     m["ffn_w_v"].matmul_op_sparse(buf.ffn_k, buf.ffn_v, ACT_NONE, fast)
-    m["ffn_w_r"].matmul_op(buf.ffn_rx, buf.ffn_r, ACT_NONE, fast)
     LayerOp.channel_mix(cursors, state, buf.ffn_r, buf.ffn_v, buf.ffn_x, state_view=ffn_state)
     LayerOp.add(buf.ffn_x, buf.x)
     if rescale_now:
