@@ -641,7 +641,8 @@ def test_v5_shape_layer_sequence(gpu, oracle, kind):
 
 
 FP16_CASES = [(2048, 512, 1), (2048, 512, 2), (2048, 516, 3), (4096, 16388, 4), (1056, 64, 7), (4096, 1024, 1), (324, 64, 5), (1056, 64, 3), (2048, 512, 17),
-              (2048, 2048, 32), (2560, 2048, 64), (4096, 4096, 128), (2048, 65536, 1), (2048, 65536, 32)]
+              (2048, 2048, 32), (2560, 2048, 64), (4096, 4096, 128), (2048, 65536, 1), (2048, 65536, 32),
+              (32, 4096, 128), (64, 4100, 37), (128, 516, 4), (32, 160, 5)]  # short rows over runs: the adapters' shapes
 
 
 @pytest.mark.parametrize("K,R,T", FP16_CASES, ids=str)

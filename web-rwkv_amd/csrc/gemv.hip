@@ -1029,6 +1029,61 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
     return WRQ_OK;
 }
 
+// f16 weights with short rows (K <= 128: the low-rank adapters of a layer) over a run of tokens: a
+// thread keeps one weight row in registers and meets TCH tokens, whose activations the workgroup
+// stages in LDS once (broadcast reads); outputs of a token are consecutive over the threads.  The
+// one-shot kernel above spends a workgroup of 128 lanes on 4 - 16 sixteen-byte chunks of such a row.
+template <typename XT, int KV, int TCH>
+__global__ __launch_bounds__(256) void gemv_fp16_thin_kernel(const MatmulArgs a) {
+    __shared__ __align__(16) uint16_t xs[TCH][8 * KV]; // KV = K / 8 sixteen-byte chunks per row
+    const uint32_t tid = threadIdx.x, b = blockIdx.z;
+    const uint32_t row = blockIdx.x * 256 + tid, t0 = blockIdx.y * TCH;
+    const uint32_t nt = min((uint32_t)TCH, a.T - t0);
+    const XT *x = reinterpret_cast<const XT *>(a.x) + (uint64_t)b * a.x_batch_stride;
+    for (uint32_t e = tid; e < nt * KV; e += 256) {
+        const uint32_t t = e / KV, c = e % KV;
+        const XT *src = x + (uint64_t)(t0 + t) * a.x_token_stride + 8 * c;
+        uint4 v;
+        if constexpr (sizeof(XT) == 2) {
+            v = load128(src);
+        } else {
+            const uint4 v0 = load128(src), v1 = load128(src + 4);
+            v = make_uint4((uint32_t)f2h(__uint_as_float(v0.x)) | ((uint32_t)f2h(__uint_as_float(v0.y)) << 16),
+                           (uint32_t)f2h(__uint_as_float(v0.z)) | ((uint32_t)f2h(__uint_as_float(v0.w)) << 16),
+                           (uint32_t)f2h(__uint_as_float(v1.x)) | ((uint32_t)f2h(__uint_as_float(v1.y)) << 16),
+                           (uint32_t)f2h(__uint_as_float(v1.z)) | ((uint32_t)f2h(__uint_as_float(v1.w)) << 16));
+        }
+        *reinterpret_cast<uint4 *>(&xs[t][8 * c]) = v;
+    }
+    uint4 w[KV];
+    const uint32_t r = min(row, a.R - 1);
+    const uint16_t *wrow = reinterpret_cast<const uint16_t *>(a.w) + ((uint64_t)b * a.R + r) * (8 * KV);
+#pragma unroll
+    for (int c = 0; c < KV; c++) w[c] = load128(wrow + 8 * c);
+    __syncthreads();
+    if (row >= a.R) return;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    for (uint32_t t = 0; t < nt; t++) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < KV; c++) {
+            const uint4 xv = *reinterpret_cast<const uint4 *>(&xs[t][8 * c]);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w[c].x), __builtin_bit_cast(h2, xv.x), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w[c].y), __builtin_bit_cast(h2, xv.y), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w[c].z), __builtin_bit_cast(h2, xv.z), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w[c].w), __builtin_bit_cast(h2, xv.w), acc, false);
+        }
+        store_out(a.out, a.out_f16, (uint64_t)b * a.out_batch_stride + (uint64_t)(t0 + t) * a.out_token_stride + row, act_apply(a.act, acc));
+    }
+}
+
+template <typename XT, int KV>
+void launch_fp16_thin(hipStream_t stream, const MatmulArgs &a) {
+    constexpr int TCH = 16;
+    const dim3 grid((a.R + 255) / 256, (a.T + TCH - 1) / TCH, a.B);
+    hipLaunchKernelGGL((gemv_fp16_thin_kernel<XT, KV, TCH>), grid, dim3(256), 0, stream, a);
+}
+
 template <typename XT, int ROWS, int TT>
 void launch_fp16_nt(hipStream_t stream, const MatmulArgs &a, uint32_t token, int nt, uint32_t groups = 1) {
     const dim3 grid((a.R + ROWS - 1) / ROWS, a.B, groups);
@@ -1057,6 +1112,15 @@ int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &a) {
         return check_launch("matmul_vec_fp16 (generic)");
     }
     const uint32_t nchunk = a.K / 8;
+    if (a.T >= 4 && (a.K == 32 || a.K == 64 || a.K == 128) && a.T <= 65535u * 16u) {
+        // short rows over a run (the adapters' second halves): the thin kernel
+        switch (a.K) {
+        case 32: in_f16 ? launch_fp16_thin<__half, 4>(stream, a) : launch_fp16_thin<float, 4>(stream, a); break;
+        case 64: in_f16 ? launch_fp16_thin<__half, 8>(stream, a) : launch_fp16_thin<float, 8>(stream, a); break;
+        default: in_f16 ? launch_fp16_thin<__half, 16>(stream, a) : launch_fp16_thin<float, 16>(stream, a); break;
+        }
+        return check_launch("matmul_vec_fp16 (short rows)");
+    }
     const int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : 128;
     const bool rows8 = (uint64_t)a.R * a.B / 8 >= 2048u;
     // f16 activations: up to 4 tokens per pass over the weights; f32: one
