@@ -359,6 +359,95 @@ class TensorOp {
         });
     }
 
+    // ---- the ops between the matrix products; shapes are checked by the library as the reference's
+    // constructors check them, a failed check throws TensorError
+
+    // src/tensor/ops.rs:300-347
+    template <typename F>
+    static TensorOp softmax(const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) { const wrq_tensor t = x.c(); return wrq_softmax(s, &t, (wrq_dtype)dtype_of<F>::value); });
+    }
+    // src/tensor/ops.rs:407-458, :460-509
+    template <typename F>
+    static TensorOp layer_norm(const TensorGpu<f16> &w, const TensorGpu<f16> &b, const TensorGpu<F> &x, float eps) {
+        x.check_shape(Shape(x.shape()[0], x.shape()[1], x.shape()[2], 1));
+        w.check_shape(Shape(x.shape()[0], 1, 1, 1));
+        b.check_shape(Shape(x.shape()[0], 1, 1, 1));
+        return checked([=](wrq_stream s) { const wrq_tensor tw = w.c(), tb = b.c(), tx = x.c(); return wrq_layer_norm(s, &tw, &tb, &tx, (wrq_dtype)dtype_of<F>::value, eps); });
+    }
+    template <typename F>
+    static TensorOp group_norm(const TensorGpu<f16> &w, const TensorGpu<f16> &b, const TensorGpu<F> &x, float eps) {
+        w.check_shape(Shape(x.shape()[0], x.shape()[1], 1, 1));
+        b.check_shape(Shape(x.shape()[0], x.shape()[1], 1, 1));
+        return checked([=](wrq_stream s) { const wrq_tensor tw = w.c(), tb = b.c(), tx = x.c(); return wrq_group_norm(s, &tw, &tb, &tx, (wrq_dtype)dtype_of<F>::value, eps); });
+    }
+    // src/tensor/ops.rs:1227-1391
+    template <typename F0, typename F1>
+    static TensorOp add_activate(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output, Activation x, Activation y, Activation out) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(); return wrq_add_activate(s, &i, &o, (int)x, (int)y, (int)out); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp mul_activate(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output, Activation x, Activation y, Activation out) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(); return wrq_mul_activate(s, &i, &o, (int)x, (int)y, (int)out); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp add(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
+        return add_activate(input, output, Activation::None, Activation::None, Activation::None);
+    }
+    template <typename F0, typename F1>
+    static TensorOp mul(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
+        return mul_activate(input, output, Activation::None, Activation::None, Activation::None);
+    }
+    // src/tensor/ops.rs:2015-2068, :2121-2169, :1973-2013, :2352-2391, :2284-2350
+    template <typename F0, typename F1>
+    static TensorOp blit(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(); return wrq_blit(s, &i, &o); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp transpose(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(); return wrq_transpose(s, &i, &o); });
+    }
+    template <typename F>
+    static TensorOp activate(const TensorGpuView<F> &x, Activation act) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view v = x.c(); return wrq_activate(s, &v, (int)act); });
+    }
+    template <typename F>
+    static TensorOp affine(const TensorGpu<F> &x, float scale, float bias) {
+        return checked([=](wrq_stream s) { const wrq_tensor t = x.c(); return wrq_affine(s, &t, (wrq_dtype)dtype_of<F>::value, scale, bias); });
+    }
+    template <typename F0, typename F1, typename F2>
+    static TensorOp lerp(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output, const TensorGpuView<F2> &factor, bool reversed) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(), f = factor.c(); return wrq_lerp(s, &i, &o, &f, reversed ? 1 : 0); });
+    }
+    // src/tensor/ops.rs:1393-1462, :1860-1915, :1601-1677
+    template <typename FT, typename F0, typename F1>
+    static TensorOp token_shift(const TensorGpu<uint32_t> &cursors, const TensorGpuView<FT> &time_mix, const TensorGpuView<float> &state,
+                                const TensorGpu<F0> &input, const TensorGpu<F1> &output, bool reversed) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), i = input.c(), o = output.c();
+            const wrq_tensor_view t = time_mix.c(), st = state.c();
+            return wrq_token_shift(s, &c, &t, &st, &i, (wrq_dtype)dtype_of<F0>::value, &o, (wrq_dtype)dtype_of<F1>::value, reversed ? 1 : 0);
+        });
+    }
+    template <typename F>
+    static TensorOp channel_mix(const TensorGpu<uint32_t> &cursors, const TensorGpuView<float> &state, const TensorGpu<F> &r, const TensorGpu<F> &v,
+                                const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), tr = r.c(), tv = v.c(), tx = x.c();
+            const wrq_tensor_view st = state.c();
+            return wrq_channel_mix(s, &c, &st, &tr, &tv, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+    template <typename F>
+    static TensorOp time_mix_v6(const TensorGpu<uint32_t> &cursors, const TensorGpu<float> &time_decay, const TensorGpu<float> &time_first,
+                                const TensorGpuView<float> &state, const TensorGpu<F> &k, const TensorGpu<F> &v, const TensorGpu<F> &r, const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), td = time_decay.c(), tf = time_first.c(), tk = k.c(), tv = v.c(), tr = r.c(), tx = x.c();
+            const wrq_tensor_view st = state.c();
+            return wrq_time_mix_v6(s, &c, &td, &tf, &st, &tk, &tv, &tr, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+
     Kind kind() const { return kind_; }
     const std::vector<TensorOp> &list() const { return list_; }
     const Payload &payload() const { return payload_; }
@@ -374,6 +463,8 @@ class TensorOp {
             throw TensorError(WRQ_ERR_SHAPE, "tensor shape not match: " + v.shape().to_string() + " vs. " + want.to_string());
     }
     static void precheck_vec(const VecInt8 &) {}
+    // an op whose shapes the library checks when it runs (the Queue turns a failed status into TensorError)
+    static TensorOp checked(std::function<int(wrq_stream)> f) { return atom(std::move(f)); }
     static TensorOp atom(std::function<int(wrq_stream)> f) {
         TensorOp op;
         op.kind_ = Kind::Atom;

@@ -256,6 +256,60 @@ static void test_gpu_head() {
     EXPECT(threw);
 }
 
+// The ops between the products through the same Queue: layer norm against its closed form, the
+// literal buffer of the reference's test_blit (src/tensor/ops.rs:3302-3336), a rejected shape.
+static void test_gpu_layer_ops() {
+    check(wrq_init());
+    const uint32_t C = 1000, T = 3;
+    std::mt19937 rng(11);
+    std::uniform_real_distribution<float> ux(-5.0f, 5.0f), uw(-0.5f, 0.5f);
+    std::vector<float> xh((size_t)C * T);
+    std::vector<f16> wh(C), bh(C);
+    for (auto &e : xh) e = ux(rng);
+    for (auto &e : wh) e.bits = to_h(uw(rng));
+    for (auto &e : bh) e.bits = to_h(uw(rng));
+    Queue queue;
+    auto x = TensorGpu<float>::from_data(Shape(C, T, 1, 1), xh);
+    auto w = TensorGpu<f16>::from_data(Shape(C, 1, 1, 1), wh);
+    auto b = TensorGpu<f16>::from_data(Shape(C, 1, 1, 1), bh);
+    queue.submit(TensorOp::layer_norm(w, b, x, 1.0e-5f));
+    queue.sync();
+    const auto got = x.back();
+    int bad = 0;
+    for (uint32_t t = 0; t < T; t++) {
+        double mean = 0, var = 0;
+        for (uint32_t i = 0; i < C; i++) mean += xh[t * C + i];
+        mean /= C;
+        for (uint32_t i = 0; i < C; i++) var += (xh[t * C + i] - mean) * (xh[t * C + i] - mean);
+        var /= C;
+        for (uint32_t i = 0; i < C; i++) {
+            const double want = (xh[t * C + i] - mean) / std::sqrt(var + 1.0e-5) * from_h(wh[i].bits) + from_h(bh[i].bits);
+            bad += std::fabs(want - got[t * C + i]) > std::max(1e-3, 1e-3 * std::fabs(want));
+        }
+    }
+    EXPECT(bad == 0);
+
+    auto out = TensorGpu<float>::from_data(Shape(4, 3, 2, 1), std::vector<float>(24, 0.0f));
+    std::vector<float> a(8), c(4);
+    for (int i = 0; i < 8; i++) a[i] = (float)i;
+    for (int i = 0; i < 4; i++) c[i] = (float)(8 + i);
+    auto in0 = TensorGpu<float>::from_data(Shape(4, 1, 2, 1), a);
+    auto in1 = TensorGpu<float>::from_data(Shape(4, 1, 1, 1), c);
+    queue.submit(TensorOp::blit(TensorGpuView<float>(in0), view_of(out, {{{0, 4}, {1, 2}, {0, 2}, {0, 1}}})));
+    queue.submit(TensorOp::blit(TensorGpuView<float>(in1), view_of(out, {{{0, 4}, {2, 3}, {1, 2}, {0, 1}}})));
+    queue.sync();
+    const std::vector<float> want = {0, 0, 0, 0, 0, 1, 2, 3, 0, 0, 0, 0, 0, 0, 0, 0, 4, 5, 6, 7, 8, 9, 10, 11};
+    EXPECT(out.back() == want);
+
+    bool threw = false;
+    try {
+        queue.submit(TensorOp::transpose(TensorGpuView<float>(in0), TensorGpuView<float>(out)));
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_SHAPE;
+    }
+    EXPECT(threw);
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     test_run_iter();
@@ -267,6 +321,7 @@ int main(int argc, char **argv) {
         try {
             test_gpu_layer();
             test_gpu_head();
+            test_gpu_layer_ops();
         } catch (const TensorError &e) {
             std::printf("FAIL: TensorError %d: %s\n", e.status, e.what());
             failures++;
