@@ -405,11 +405,34 @@ def full_layers(wrq, torch, args, C, H):
     # one request in slot 0 whose A tokens fill the stack (the reference packs the count into 8 bits)
     cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
     x0 = buf.x.clone()
+    model = args.full_model
+    if model:
+        # the ends of the model (src/runtime/v6.rs:625-640, :960-1000): embedding + its layer norm in front,
+        # layer norm + f16 head (65536 x C) on the run's last token + softmax behind
+        V = 65536
+        g = torch.Generator(device="cuda").manual_seed(SEED + 8)
+        embed = (torch.randn((V, C), generator=g, device="cuda") * 0.5).half()
+        head = wrq.Matrix.fp16((torch.randn((V, C), generator=g, device="cuda") * 0.02).half())
+        ln = [(1.0 + 0.1 * torch.randn(C, generator=g, device="cuda")).half(), (0.1 * torch.randn(C, generator=g, device="cuda")).half()]
+        ids = torch.randint(0, V, (1, A), generator=g, device="cuda", dtype=torch.int32)
+        inp = torch.zeros((1, A, C), dtype=torch.float16, device="cuda")
+        head_x = torch.zeros((1, 1, C), dtype=torch.float16, device="cuda")
+        logits = torch.zeros((1, 1, V), dtype=torch.float32, device="cuda")
 
     def step():
-        buf.x.copy_(x0)  # the embedding of the next token would land here
+        if model:
+            wrq.LayerOp.embed(ids, embed, inp)
+            wrq.LayerOp.layer_norm(ln[0], ln[1], inp, v6.LN_EPS)
+            wrq.LayerOp.blit(inp, buf.x)
+        else:
+            buf.x.copy_(x0)  # the embedding of the next token would land here
         for i, (layer, st) in enumerate(zip(layers, states)):
             v6.dispatch_layer(layer, buf, st, cursors, A, heads, S, rescale_now=(i + 1) % 6 == 0)
+        if model:
+            wrq.LayerOp.blit(buf.x, head_x, input_view=((C, 1, 1), (C, A, 1), (0, A - 1, 0)))
+            wrq.LayerOp.layer_norm(ln[0], ln[1], head_x, v6.LN_EPS)
+            head.matmul_op(head_x, logits, turbo=False)
+            wrq.LayerOp.softmax(logits)
 
     step()
     torch.cuda.synchronize()
@@ -422,7 +445,9 @@ def full_layers(wrq, torch, args, C, H):
         fn = graph.replay
     ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
     assert torch.isfinite(buf.x.float()).all()
-    print(json.dumps({"metric": "RWKV-v6 7B-shape layers, every op (no embedding, no head), tokens/s", "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
+    what = "RWKV-v6 7B-shape model step, every op (embedding, layers, head on the last token, softmax), tokens/s" if model else \
+        "RWKV-v6 7B-shape layers, every op (no embedding, no head), tokens/s"
+    print(json.dumps({"metric": what, "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
                       "config": {"workload": f"{args.layers} v6 layers ({C} x {H}, {heads} heads), {args.quant}, {A} token(s) of one request per step, 35 ops per layer",
                                  "hip_graph": not args.no_graph}, "data": "synthetic"}))
@@ -501,6 +526,7 @@ def main():
     ap.add_argument("--slots", type=int, default=32)
     ap.add_argument("--full-layers", action="store_true", help="every op of the v6 layers (35 per layer), not only the quantized products")
     ap.add_argument("--ops", action="store_true", help="time of every layer op alone at the 7B layer shape")
+    ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
@@ -521,7 +547,7 @@ def main():
     if args.ops:
         ops_table(wrq, torch, args, C)
         return
-    if args.full_layers:
+    if args.full_layers or args.full_model:
         full_layers(wrq, torch, args, C, H)
         return
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)

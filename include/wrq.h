@@ -235,6 +235,8 @@ int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_
                      int act_x, int act_y, int act_out);
 
 /*
+ * TensorOp::embed(tokens, input, output)    src/tensor/ops.rs:350-405, src/shaders/embed.wgsl
+ *   tokens u32 [T, B, 1, 1]; input f16 [C, V, 1, 1]; output [C, T, B, 1] <- the tokens' rows.
  * TensorOp::blit(input, output)             src/tensor/ops.rs:2015-2068, src/shaders/blit.wgsl
  *   copies a view into a view of the same shape, converting the element type.
  * TensorOp::transpose(input, output)        src/tensor/ops.rs:2121-2169, src/shaders/reshape.wgsl:58-77
@@ -245,6 +247,8 @@ int wrq_mul_activate(wrq_stream stream, const wrq_tensor_view *input, const wrq_
  * TensorOp::lerp(input, output, factor, reversed)   src/tensor/ops.rs:2284-2350, src/shaders/lerp.wgsl
  *   output <- input (1 - f) + output f (reversed: the two swapped); factor [C, T|1, B|1, 1].
  */
+int wrq_embed(wrq_stream stream, const wrq_tensor *tokens, const wrq_tensor *input, const wrq_tensor *output,
+              wrq_dtype dtype);
 int wrq_blit(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output);
 int wrq_transpose(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output);
 int wrq_activate(wrq_stream stream, const wrq_tensor_view *x, int act);

@@ -398,6 +398,11 @@ class TensorOp {
     static TensorOp mul(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
         return mul_activate(input, output, Activation::None, Activation::None, Activation::None);
     }
+    // src/tensor/ops.rs:350-405
+    template <typename F>
+    static TensorOp embed(const TensorGpu<uint32_t> &tokens, const TensorGpu<f16> &input, const TensorGpu<F> &output) {
+        return checked([=](wrq_stream s) { const wrq_tensor t = tokens.c(), i = input.c(), o = output.c(); return wrq_embed(s, &t, &i, &o, (wrq_dtype)dtype_of<F>::value); });
+    }
     // src/tensor/ops.rs:2015-2068, :2121-2169, :1973-2013, :2352-2391, :2284-2350
     template <typename F0, typename F1>
     static TensorOp blit(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {

@@ -335,6 +335,23 @@ def test_gpu_data_movement_kats(gpu):
 
 
 @pytest.mark.gpu
+def test_gpu_embed(gpu):
+    import torch
+
+    print("embed on the GPU", flush=True)
+    rng = np.random.default_rng(SEED + 45)
+    V, C, T, B = 300, 128, 5, 2
+    table = rng.standard_normal((V, C)).astype(np.float16)
+    ids = rng.integers(0, V, size=(B, T)).astype(np.int32)
+    for dt in (torch.float16, torch.float32):
+        out = torch.zeros((B, T, C), dtype=dt, device="cuda")
+        gpu.LayerOp.embed(torch.from_numpy(ids).cuda(), torch.from_numpy(table).cuda(), out)
+        assert np.array_equal(out.cpu().numpy(), table[ids].astype(out.cpu().numpy().dtype))  # a gather: exact
+    with pytest.raises(gpu.TensorError):
+        gpu.LayerOp.embed(torch.from_numpy(ids).cuda(), torch.from_numpy(table).cuda(), torch.zeros((B, T + 1, C), dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.gpu
 def test_gpu_lerp_activate_affine(gpu, lop):
     import torch
 

@@ -43,7 +43,7 @@ EXPORTS = [
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
-    "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v6",
+    "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v6", "wrq_embed",
 ]
 MAX_GROUP = 8
 
@@ -197,6 +197,7 @@ def lib():
         L.wrq_token_shift.argtypes = [vp, T, V, V, T, i, T, i, i]
         L.wrq_channel_mix.argtypes = [vp, T, V, T, T, T, i]
         L.wrq_time_mix_v6.argtypes = [vp, T, T, T, V, T, T, T, T, i]
+        L.wrq_embed.argtypes = [vp, T, T, T, i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -319,6 +320,10 @@ class LayerOp:
 
     add = add_activate
     mul = mul_activate
+
+    @staticmethod
+    def embed(tokens, input, output):
+        _check(lib().wrq_embed(_stream(), C.byref(as_tensor(tokens)), C.byref(as_tensor(input)), C.byref(as_tensor(output)), _dtype(output)))
 
     @staticmethod
     def blit(input, output, input_view=None, output_view=None):

@@ -194,6 +194,16 @@ __global__ __launch_bounds__(256) void lerp_kernel(const FT *f, const IT *x, OT 
     store_vec4(out, make_float4(mix(a.x, c.x, ff.x), mix(a.y, c.y, ff.y), mix(a.z, c.z, ff.z), mix(a.w, c.w, ff.w)));
 }
 
+// output[batch][token] <- row tokens[batch][token] of the f16 table (src/shaders/embed.wgsl:22-38); an
+// id beyond the table reads its last row (the host cannot check ids that live in device memory)
+template <typename OT>
+__global__ __launch_bounds__(256) void embed_kernel(const uint32_t *tokens, const uint16_t *table, OT *output, uint32_t C, uint32_t T, uint32_t vocab) {
+    const uint32_t index = blockIdx.x * 256 + threadIdx.x, token = blockIdx.y, batch = blockIdx.z;
+    if (index >= C / 4) return;
+    const uint32_t id = min(tokens[batch * T + token], vocab - 1);
+    store_vec4(output + ((uint64_t)(batch * T + token) * C + 4 * index), load_vec4(table + ((uint64_t)id * C + 4 * index)));
+}
+
 int check_row_tensor(const wrq_tensor *x, int dtype, const char *what) {
     if (!x || !x->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, dtype);
@@ -209,7 +219,11 @@ int launch_rows(hipStream_t stream, void *x, int dtype, const void *w, const voi
     if (rows > 0x7fffffffull) return fail(WRQ_ERR_SIZE, "%s: data size not match", what);
     const uint16_t *wp = static_cast<const uint16_t *>(w), *bp = static_cast<const uint16_t *>(b);
     // short rows (a head of a group norm) take one wave, no LDS exchange
-    if (n <= 1024) {
+    if (n > 16384) {
+        // a vocabulary-sized row (softmax over the logits): 1024 threads
+        if (dtype == WRQ_F16) hipLaunchKernelGGL((row_kernel<uint16_t, MODE, 1024>), dim3((uint32_t)rows), dim3(1024), 0, stream, static_cast<uint16_t *>(x), wp, bp, n, heads, eps);
+        else hipLaunchKernelGGL((row_kernel<float, MODE, 1024>), dim3((uint32_t)rows), dim3(1024), 0, stream, static_cast<float *>(x), wp, bp, n, heads, eps);
+    } else if (n <= 1024) {
         if (dtype == WRQ_F16) hipLaunchKernelGGL((row_kernel<uint16_t, MODE, 64>), dim3((uint32_t)rows), dim3(64), 0, stream, static_cast<uint16_t *>(x), wp, bp, n, heads, eps);
         else hipLaunchKernelGGL((row_kernel<float, MODE, 64>), dim3((uint32_t)rows), dim3(64), 0, stream, static_cast<float *>(x), wp, bp, n, heads, eps);
     } else {
@@ -396,4 +410,25 @@ int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_v
     return lerp_out<float, float>(st, factor, input, output, grid, reversed);
 }
 
+int wrq_embed(wrq_stream stream, const wrq_tensor *tokens, const wrq_tensor *input, const wrq_tensor *output, wrq_dtype dtype) {
+    const int s = check_row_tensor(output, dtype, "embed");
+    if (s != WRQ_OK) return s;
+    if (!tokens || !input || !tokens->data || !input->data) return fail(WRQ_ERR_NULL, "embed: null tensor");
+    const uint32_t *o = output->shape, *t = tokens->shape, *i = input->shape;
+    // src/tensor/ops.rs:357-364
+    if (t[0] != o[1] || t[1] != o[2] || t[2] != 1 || t[3] != 1 || i[0] != o[0] || i[2] != 1 || i[3] != 1 || i[1] == 0)
+        return fail(WRQ_ERR_SHAPE, "embed: data shape not match [%u, %u, %u, %u]", o[0], o[1], o[2], o[3]);
+    if ((uintptr_t)input->data % 8) return fail(WRQ_ERR_ALIGNMENT, "embed: device pointers must be 8-byte aligned");
+    if (o[0] == 0 || o[1] == 0 || o[2] == 0) return WRQ_OK;
+    if (o[1] > 65535u || o[2] > 65535u) return fail(WRQ_ERR_SIZE, "embed: data size not match");
+    const dim3 grid((o[0] / 4 + 255) / 256, o[1], o[2]);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    if (dtype == WRQ_F16)
+        hipLaunchKernelGGL((embed_kernel<uint16_t>), grid, dim3(256), 0, hs, static_cast<const uint32_t *>(tokens->data), static_cast<const uint16_t *>(input->data), static_cast<uint16_t *>(output->data), o[0], o[1], i[1]);
+    else
+        hipLaunchKernelGGL((embed_kernel<float>), grid, dim3(256), 0, hs, static_cast<const uint32_t *>(tokens->data), static_cast<const uint16_t *>(input->data), static_cast<float *>(output->data), o[0], o[1], i[1]);
+    return check_launch("embed");
+}
+
 } // extern "C"
+
