@@ -405,6 +405,7 @@ def full_layers(wrq, torch, args, C, H):
     # one request in slot 0 whose A tokens fill the stack (the reference packs the count into 8 bits)
     cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
     x0 = buf.x.clone()
+    dispatch = v6.dispatch_layer_fused if args.fused else v6.dispatch_layer
     model = args.full_model
     if model:
         # the ends of the model (src/runtime/v6.rs:625-640, :960-1000): embedding + its layer norm in front,
@@ -427,7 +428,7 @@ def full_layers(wrq, torch, args, C, H):
         else:
             buf.x.copy_(x0)  # the embedding of the next token would land here
         for i, (layer, st) in enumerate(zip(layers, states)):
-            v6.dispatch_layer(layer, buf, st, cursors, A, heads, S, rescale_now=(i + 1) % 6 == 0)
+            dispatch(layer, buf, st, cursors, A, heads, S, rescale_now=(i + 1) % 6 == 0)
         if model:
             wrq.LayerOp.blit(buf.x, head_x, input_view=((C, 1, 1), (C, A, 1), (0, A - 1, 0)))
             wrq.LayerOp.layer_norm(ln[0], ln[1], head_x, v6.LN_EPS)
@@ -449,7 +450,8 @@ def full_layers(wrq, torch, args, C, H):
         "RWKV-v6 7B-shape layers, every op (no embedding, no head), tokens/s"
     print(json.dumps({"metric": what, "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
-                      "config": {"workload": f"{args.layers} v6 layers ({C} x {H}, {heads} heads), {args.quant}, {A} token(s) of one request per step, 35 ops per layer",
+                      "config": {"workload": f"{args.layers} v6 layers ({C} x {H}, {heads} heads), {args.quant}, {A} token(s) of one request per step, "
+                                             + ("12 launches per layer (fused small ops)" if args.fused else "35 ops per layer"),
                                  "hip_graph": not args.no_graph}, "data": "synthetic"}))
 
 
@@ -526,6 +528,7 @@ def main():
     ap.add_argument("--slots", type=int, default=32)
     ap.add_argument("--full-layers", action="store_true", help="every op of the v6 layers (35 per layer), not only the quantized products")
     ap.add_argument("--ops", action="store_true", help="time of every layer op alone at the 7B layer shape")
+    ap.add_argument("--fused", action="store_true", help="with --full-layers / --full-model: the fused small ops (12 launches per layer instead of 35)")
     ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -285,6 +285,38 @@ int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
                     const wrq_tensor *time_first, const wrq_tensor_view *state, const wrq_tensor *k,
                     const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype);
 
+/*
+ * Fused forms of consecutive small ops of an RWKV-v6 layer (src/runtime/v6.rs:758-955).  They have no
+ * counterpart among the reference's constructors; they are for callers that run a layer without hooks
+ * between its ops: at batch 1 every op costs its launch, and these bring a layer from 35 launches to 12.
+ * Each computes what the listed ops compute, rounding to f16 where the list stores an f16 buffer.
+ * Buffers are contiguous device arrays of `Runtime<f16>` (v6.rs:270-303): C channels x A tokens.
+ *
+ * wrq_v6_pre: [add(add, x) ->] blit + layer_norm + token_shift x `shifts` (reversed)   v6.rs:759-777, :906-933
+ *   x_out (f16, only with `add`, must differ from x) <- add + x;  ln_out <- LN(row);  shift_s <- mix(ln, previous, factor_s).
+ * wrq_v6_time_mix: transpose + time_mix_w2 + add(time_mix) + token_shift(5)           v6.rs:785-805
+ *   lora f16 [lora_size, 5, A]; w2 f16 [lora_size, C, 5]; time_mix f16 [C, 1, 5]; att_sx f16 [C, A, 5].
+ * wrq_v6_decay: time_decay_w2 + add(time_decay) + activate(StableExp)                 v6.rs:839-848
+ *   lora f16 [lora_size, A]; w2 f16 [lora_size, C]; out f32 [C, A].
+ * wrq_v6_wkv_gate: blit + time_mix_v6 + group_norm + blit + mul_activate(Silu)        v6.rs:851-887
+ *   k, v, r, time_decay f32 [C, A]; g f16; att_x f16 in (the normalised layer input) and out. Head size 64.
+ * wrq_v6_post_ffn: channel_mix + add (+ affine(0.5) when `rescale`)                   v6.rs:942-955
+ */
+int wrq_v6_pre(wrq_stream stream, uint32_t C, uint32_t A, const void *cursors, const void *x, const void *add,
+               void *x_out, const void *ln_w, const void *ln_b, float eps, const wrq_tensor_view *state, int shifts,
+               const void *factor0, const void *factor1, void *ln_out, void *shift0, void *shift1);
+int wrq_v6_time_mix(wrq_stream stream, uint32_t C, uint32_t A, uint32_t lora_size, const void *cursors,
+                    const void *lora, const void *w2, const void *time_mix, const wrq_tensor_view *state,
+                    const void *att_x, void *att_sx);
+int wrq_v6_decay(wrq_stream stream, uint32_t C, uint32_t A, uint32_t lora_size, const void *lora, const void *w2,
+                 const void *time_decay, void *out);
+int wrq_v6_wkv_gate(wrq_stream stream, uint32_t S, uint32_t H, uint32_t A, const void *cursors,
+                    const void *time_decay, const void *time_first, const wrq_tensor_view *state, const void *k,
+                    const void *v, const void *r, const void *g, const void *gn_w, const void *gn_b, float eps,
+                    void *att_x);
+int wrq_v6_post_ffn(wrq_stream stream, uint32_t C, uint32_t A, const void *cursors, const wrq_tensor_view *state,
+                    const void *r, const void *v, const void *ffn_x, const void *x_in, void *x_out, int rescale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -91,3 +91,37 @@ def test_v6_layer_against_numpy(gpu, oracle, quant, runs):
     assert_close(sd.cpu().numpy(), want_state, 1e-2, "state after the run")
     untouched = [b for b in range(B) if b not in [s for s, _ in runs]]
     assert np.array_equal(sd.cpu().numpy()[untouched], state[untouched])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quant", ["int8", "nf4"])
+@pytest.mark.parametrize("runs", [[(2, 3), (0, 1), (5, 4)], [(1, 20), (3, 12)], [(4, 1)]], ids=["8 tokens", "32 tokens (chunk kernels)", "1 token"])
+def test_v6_layer_fused_equals_op_list(gpu, oracle, quant, runs):
+    # the 12-launch form of the layer against the op list: same buffers, same roundings
+    import torch
+
+    sys.path.insert(0, ROOT)
+    lop = importlib.import_module("oracle.layer_ops")
+    v6 = importlib.import_module(gpu.__name__ + ".v6")
+    print("v6 layer, fused, on the GPU", quant, runs, flush=True)
+    H, S, hidden, B = 4, 64, 512, 6
+    C = H * S
+    rng = np.random.default_rng(SEED + 100 + len(runs))
+    layer = v6.Layer(torch, v6.random_layer_weights(rng, C, H, S, hidden, layer=3), quant)
+    cursors = lop.pack_cursors(runs)
+    A = len(cursors)
+    curd = torch.from_numpy(cursors.view(np.int32)).cuda()
+    x = rng.standard_normal((A, C)).astype(np.float16)
+    state = (0.1 * rng.standard_normal((B, S + 2, C))).astype(np.float32)
+    outs = []
+    for fused in (False, True):
+        buf = v6.Runtime(torch, C, hidden, A)
+        buf.x.copy_(torch.from_numpy(x).cuda().reshape(1, A, C))
+        sd = torch.from_numpy(state.copy()).cuda()
+        (v6.dispatch_layer_fused if fused else v6.dispatch_layer)(layer, buf, sd, curd, A, H, S, rescale_now=True)
+        torch.cuda.synchronize()
+        outs.append((buf.x.cpu().numpy()[0].astype(np.float32), sd.cpu().numpy()))
+    # f32 sums in another order flip an f16 rounding here and there: a few f16 ulps after 35 ops
+    assert_close(outs[1][0], outs[0][0], 4e-3, "layer output, fused vs op list")
+    assert_close(outs[1][1], outs[0][1], 4e-3, "state, fused vs op list")
+    assert np.mean(outs[1][0] == outs[0][0]) > 0.9  # and most outputs are the same f16 value

@@ -44,6 +44,7 @@ EXPORTS = [
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
     "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v6", "wrq_embed",
+    "wrq_v6_pre", "wrq_v6_time_mix", "wrq_v6_decay", "wrq_v6_wkv_gate", "wrq_v6_post_ffn",
 ]
 MAX_GROUP = 8
 
@@ -198,6 +199,12 @@ def lib():
         L.wrq_channel_mix.argtypes = [vp, T, V, T, T, T, i]
         L.wrq_time_mix_v6.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         L.wrq_embed.argtypes = [vp, T, T, T, i]
+        u = C.c_uint32
+        L.wrq_v6_pre.argtypes = [vp, u, u, vp, vp, vp, vp, vp, vp, C.c_float, V, i, vp, vp, vp, vp, vp]
+        L.wrq_v6_time_mix.argtypes = [vp, u, u, u, vp, vp, vp, vp, V, vp, vp]
+        L.wrq_v6_decay.argtypes = [vp, u, u, u, vp, vp, vp, vp]
+        L.wrq_v6_wkv_gate.argtypes = [vp, u, u, u, vp, vp, vp, V, vp, vp, vp, vp, vp, vp, C.c_float, vp]
+        L.wrq_v6_post_ffn.argtypes = [vp, u, u, vp, V, vp, vp, vp, vp, vp, i]
         for name in EXPORTS[4:]:
             getattr(L, name).restype = i
         _lib = L
@@ -361,6 +368,41 @@ class LayerOp:
     def lerp(input, output, factor, reversed=False, input_view=None, output_view=None, factor_view=None):
         _check(lib().wrq_lerp(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)),
                               C.byref(as_view(factor, factor_view)), int(reversed)))
+
+
+class FusedV6:
+    """The fused forms of a v6 layer's small ops (`wrq_v6_*`); arguments are contiguous torch tensors."""
+
+    @staticmethod
+    def _p(t):
+        return None if t is None else C.c_void_p(t.data_ptr())
+
+    @staticmethod
+    def pre(Cn, A, cursors, x, add, x_out, ln_w, ln_b, eps, state, state_view, factors, ln_out, shifts):
+        p = FusedV6._p
+        _check(lib().wrq_v6_pre(_stream(), Cn, A, p(cursors), p(x), p(add), p(x_out), p(ln_w), p(ln_b), eps, C.byref(as_view(state, state_view)), len(factors),
+                                p(factors[0]), p(factors[1] if len(factors) > 1 else None), p(ln_out), p(shifts[0]), p(shifts[1] if len(shifts) > 1 else None)))
+
+    @staticmethod
+    def time_mix(Cn, A, lora_size, cursors, lora, w2, time_mix, state, state_view, att_x, att_sx):
+        p = FusedV6._p
+        _check(lib().wrq_v6_time_mix(_stream(), Cn, A, lora_size, p(cursors), p(lora), p(w2), p(time_mix), C.byref(as_view(state, state_view)), p(att_x), p(att_sx)))
+
+    @staticmethod
+    def decay(Cn, A, lora_size, lora, w2, time_decay, out):
+        p = FusedV6._p
+        _check(lib().wrq_v6_decay(_stream(), Cn, A, lora_size, p(lora), p(w2), p(time_decay), p(out)))
+
+    @staticmethod
+    def wkv_gate(S, H, A, cursors, time_decay, time_first, state, state_view, k, v, r, g, gn_w, gn_b, eps, att_x):
+        p = FusedV6._p
+        _check(lib().wrq_v6_wkv_gate(_stream(), S, H, A, p(cursors), p(time_decay), p(time_first), C.byref(as_view(state, state_view)), p(k), p(v), p(r), p(g),
+                                     p(gn_w), p(gn_b), eps, p(att_x)))
+
+    @staticmethod
+    def post_ffn(Cn, A, cursors, state, state_view, r, v, ffn_x, x_in, x_out, rescale):
+        p = FusedV6._p
+        _check(lib().wrq_v6_post_ffn(_stream(), Cn, A, p(cursors), C.byref(as_view(state, state_view)), p(r), p(v), p(ffn_x), p(x_in), p(x_out), int(rescale)))
 
 
 def matmul_vec_group(ops):

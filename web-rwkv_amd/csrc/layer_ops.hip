@@ -9,8 +9,7 @@
 // one LDS exchange, every access is a whole 8- or 16-byte vector of 4 elements as in the shaders.
 // The statistics are two-pass (mean, then the sum of squared deviations) in f32: the shaders merge
 // per-lane Welford states; both agree with the exact value far inside the reference's 1e-3 test bar.
-#include "wrq_device.h"
-#include "wrq_host.h"
+#include "layer_device.h"
 
 namespace wrq {
 
@@ -18,51 +17,6 @@ namespace {
 
 constexpr int kRowThreads = 256;
 constexpr int kRowCache = 8; // vectors of 4 elements a thread keeps: rows up to 8192 elements stay in registers
-
-template <typename XT>
-__device__ __forceinline__ float4 load_vec4(const XT *p) {
-    if constexpr (sizeof(XT) == 2) {
-        const uint2 v = *reinterpret_cast<const uint2 *>(p);
-        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
-    } else {
-        return *reinterpret_cast<const float4 *>(p);
-    }
-}
-
-template <typename XT>
-__device__ __forceinline__ void store_vec4(XT *p, float4 v) {
-    if constexpr (sizeof(XT) == 2) {
-        *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f2h(v.x) | ((uint32_t)f2h(v.y) << 16), (uint32_t)f2h(v.z) | ((uint32_t)f2h(v.w) << 16));
-    } else {
-        *reinterpret_cast<float4 *>(p) = v;
-    }
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
-}
-
-// sum or maximum over the workgroup, the same value in every thread
-template <bool MAX, int THREADS>
-__device__ __forceinline__ float block_reduce(float v, float *red) {
-    v = MAX ? wave_max(v) : wave_sum(v);
-    if constexpr (THREADS == 64) return v;
-    const uint32_t wave = threadIdx.x >> 6;
-    __syncthreads(); // `red` may still be read from the previous reduction
-    if ((threadIdx.x & 63) == 0) red[wave] = v;
-    __syncthreads();
-    float r = red[0];
-#pragma unroll
-    for (int w = 1; w < THREADS / 64; w++) r = MAX ? fmaxf(r, red[w]) : r + red[w];
-    return r;
-}
 
 // One workgroup per row of `n` elements (n % 4 == 0).  MODE 0: softmax; 1: layer norm (w, b of the
 // row's length); 2: group norm (w, b indexed by head * n, the row index modulo `heads`).
@@ -131,17 +85,6 @@ __global__ __launch_bounds__(THREADS) void row_kernel(XT *x, const uint16_t *w, 
     } else {
         for (uint32_t i = threadIdx.x; i < nv; i += THREADS) finish(i, load_vec4(row + 4 * i));
     }
-}
-
-struct ViewArgs {
-    uint32_t shape[4], stride[4], offset[4];
-};
-
-// element index of vector `index` of (batch, token) in a view, in units of 4 elements
-// (compute_index of the shaders: src/shaders/binary.wgsl:30-34)
-__device__ __forceinline__ uint64_t view_index(const ViewArgs &v, uint32_t batch, uint32_t token, uint32_t index) {
-    const uint64_t stride = v.stride[0] >> 2;
-    return ((uint64_t)(batch + v.offset[2]) * v.stride[1] + (token + v.offset[1])) * stride + index + (v.offset[0] >> 2);
 }
 
 // output = ACT_OUT(ACT_X(input) op ACT_Y(output)); input broadcast over tokens / batches of extent 1
@@ -233,29 +176,12 @@ int launch_rows(hipStream_t stream, void *x, int dtype, const void *w, const voi
     return check_launch(what);
 }
 
-ViewArgs view_args(const wrq_view &v) {
-    ViewArgs a;
-    for (int i = 0; i < 4; i++) a.shape[i] = v.shape[i], a.stride[i] = v.stride[i], a.offset[i] = v.offset[i];
-    return a;
-}
-
-int check_view(const wrq_tensor_view *t, const char *what) {
-    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
-    if (t->dtype != WRQ_F16 && t->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, (int)t->dtype);
-    for (int i = 0; i < 4; i++)
-        if ((uint64_t)t->view.offset[i] + t->view.shape[i] > t->view.stride[i])
-            return fail(WRQ_ERR_SHAPE, "%s: slice out of range", what);
-    if (t->view.shape[0] % 4 || t->view.stride[0] % 4 || t->view.offset[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "%s: rows not in units of 4 elements", what);
-    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
-    return WRQ_OK;
-}
-
 template <bool MUL>
 int binary(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_view *output, int act_x, int act_y, int act_out) {
     const char *what = MUL ? "mul" : "add";
-    int s = check_view(input, what);
+    int s = check_layer_view(input, what);
     if (s != WRQ_OK) return s;
-    s = check_view(output, what);
+    s = check_layer_view(output, what);
     if (s != WRQ_OK) return s;
     for (int a : {act_x, act_y, act_out})
         if (a < 0 || a > WRQ_ACT_SILU) return fail(WRQ_ERR_UNSUPPORTED, "%s: unknown activation %d", what, a);
@@ -280,9 +206,9 @@ int binary(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_vi
 template <int MODE>
 int copy(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_view *output) {
     const char *what = MODE == 1 ? "transpose" : "blit";
-    int s = check_view(input, what);
+    int s = check_layer_view(input, what);
     if (s != WRQ_OK) return s;
-    s = check_view(output, what);
+    s = check_layer_view(output, what);
     if (s != WRQ_OK) return s;
     const uint32_t *i = input->view.shape, *o = output->view.shape;
     const bool ok = MODE == 1 ? (o[0] == i[0] && o[1] == i[2] && o[2] == i[1] && o[3] == 1 && i[3] == 1) : (o[0] == i[0] && o[1] == i[1] && o[2] == i[2] && o[3] == i[3]);
@@ -302,7 +228,7 @@ int copy(hipStream_t stream, const wrq_tensor_view *input, const wrq_tensor_view
 template <bool AFFINE>
 int unary(hipStream_t stream, const wrq_tensor_view *x, int act, float scale, float bias) {
     const char *what = AFFINE ? "affine" : "activate";
-    const int s = check_view(x, what);
+    const int s = check_layer_view(x, what);
     if (s != WRQ_OK) return s;
     if (!AFFINE && (act < 0 || act > WRQ_ACT_SILU)) return fail(WRQ_ERR_UNSUPPORTED, "%s: unknown activation %d", what, act);
     const uint32_t *v = x->view.shape;
@@ -390,9 +316,9 @@ int wrq_affine(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype, float sc
 }
 
 int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output, const wrq_tensor_view *factor, int reversed) {
-    int s = check_view(input, "lerp");
-    if (s == WRQ_OK) s = check_view(output, "lerp");
-    if (s == WRQ_OK) s = check_view(factor, "lerp");
+    int s = check_layer_view(input, "lerp");
+    if (s == WRQ_OK) s = check_layer_view(output, "lerp");
+    if (s == WRQ_OK) s = check_layer_view(factor, "lerp");
     if (s != WRQ_OK) return s;
     const uint32_t *o = output->view.shape, *i = input->view.shape, *f = factor->view.shape;
     // src/tensor/ops.rs:2298-2307

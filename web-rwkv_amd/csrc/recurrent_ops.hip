@@ -14,66 +14,11 @@
 // per token, no LDS and no barrier; S is read when a request's tokens begin and written when they
 // end.  The sum over j is therefore taken in four interleaved partial sums instead of one chain
 // (a difference of rounding order only).
-#include "wrq_device.h"
-#include "wrq_host.h"
+#include "layer_device.h"
 
 namespace wrq {
 
 namespace {
-
-struct ViewArgs {
-    uint32_t shape[4], stride[4], offset[4];
-};
-
-ViewArgs view_args(const wrq_view &v) {
-    ViewArgs a;
-    for (int i = 0; i < 4; i++) a.shape[i] = v.shape[i], a.stride[i] = v.stride[i], a.offset[i] = v.offset[i];
-    return a;
-}
-
-// element index (units of 1 element) of (batch, token, element) in a view: compute_index of the shaders
-__device__ __forceinline__ uint64_t view_elem(const ViewArgs &v, uint32_t batch, uint32_t token, uint32_t elem) {
-    return ((uint64_t)(batch + v.offset[2]) * v.stride[1] + (token + v.offset[1])) * v.stride[0] + elem + v.offset[0];
-}
-
-template <typename XT>
-__device__ __forceinline__ float4 load_vec4(const XT *p) {
-    if constexpr (sizeof(XT) == 2) {
-        const uint2 v = *reinterpret_cast<const uint2 *>(p);
-        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
-    } else {
-        return *reinterpret_cast<const float4 *>(p);
-    }
-}
-
-template <typename XT>
-__device__ __forceinline__ void store_vec4(XT *p, float4 v) {
-    if constexpr (sizeof(XT) == 2) {
-        *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f2h(v.x) | ((uint32_t)f2h(v.y) << 16), (uint32_t)f2h(v.z) | ((uint32_t)f2h(v.w) << 16));
-    } else {
-        *reinterpret_cast<float4 *>(p) = v;
-    }
-}
-
-template <typename XT>
-__device__ __forceinline__ float load_one(const XT *p) {
-    if constexpr (sizeof(XT) == 2) return h2f(*p);
-    else return *p;
-}
-
-struct Cursor {
-    uint32_t batch, token, len;
-};
-__device__ __forceinline__ Cursor unpack_cursor(uint32_t x) { return Cursor{x & 0xffu, (x >> 8) & 0xffffu, (x >> 24) & 0xffu}; }
-// Cursors live in device memory, the host cannot check them: a state slot beyond the view is clamped
-// to its last slot and a first token beyond the token itself counts as the token itself, so that a
-// malformed cursor reads and writes inside the tensors (the shaders rely on WebGPU's bounds clamping).
-__device__ __forceinline__ Cursor read_cursor(const uint32_t *cursors, uint32_t stack, const ViewArgs &vs) {
-    Cursor c = unpack_cursor(cursors[stack]);
-    c.batch = min(c.batch, vs.shape[2] - 1);
-    c.token = min(c.token, stack);
-    return c;
-}
 
 // output[count][stack] = mix(previous token, this token, time_mix) (reversed: the two swapped); the
 // previous token of a request's first token in the stack is its state row
@@ -213,24 +158,6 @@ __global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursor
     }
 }
 
-int check_view(const wrq_tensor_view *t, const char *what) {
-    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
-    if (t->dtype != WRQ_F16 && t->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", what, (int)t->dtype);
-    for (int i = 0; i < 4; i++)
-        if ((uint64_t)t->view.offset[i] + t->view.shape[i] > t->view.stride[i]) return fail(WRQ_ERR_SHAPE, "%s: slice out of range", what);
-    if (t->view.shape[0] % 4 || t->view.stride[0] % 4 || t->view.offset[0] % 4) return fail(WRQ_ERR_ALIGNMENT, "%s: rows not in units of 4 elements", what);
-    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
-    return WRQ_OK;
-}
-
-int check_tensor(const wrq_tensor *t, const char *what) {
-    if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
-    if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);
-    return WRQ_OK;
-}
-
-bool same_shape(const uint32_t *a, const uint32_t *b) { return a[0] == b[0] && a[1] == b[1] && a[2] == b[2] && a[3] == b[3]; }
-
 template <typename FT, typename IT>
 int token_shift_out(hipStream_t stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix, const wrq_tensor_view *state, const wrq_tensor *input,
                     const wrq_tensor *output, int out_dtype, dim3 grid, int reversed) {
@@ -256,11 +183,11 @@ extern "C" {
 
 int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix, const wrq_tensor_view *state, const wrq_tensor *input,
                     wrq_dtype input_dtype, const wrq_tensor *output, wrq_dtype output_dtype, int reversed) {
-    int s = check_tensor(cursors, "token_shift");
-    if (s == WRQ_OK) s = check_tensor(input, "token_shift");
-    if (s == WRQ_OK) s = check_tensor(output, "token_shift");
-    if (s == WRQ_OK) s = check_view(time_mix, "token_shift");
-    if (s == WRQ_OK) s = check_view(state, "token_shift");
+    int s = check_layer_tensor(cursors, "token_shift");
+    if (s == WRQ_OK) s = check_layer_tensor(input, "token_shift");
+    if (s == WRQ_OK) s = check_layer_tensor(output, "token_shift");
+    if (s == WRQ_OK) s = check_layer_view(time_mix, "token_shift");
+    if (s == WRQ_OK) s = check_layer_view(state, "token_shift");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "token_shift: the state is f32");
     for (int d : {(int)input_dtype, (int)output_dtype})
@@ -285,10 +212,10 @@ int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
 
 int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state, const wrq_tensor *r, const wrq_tensor *v, const wrq_tensor *x,
                     wrq_dtype dtype) {
-    int s = check_tensor(cursors, "channel_mix");
+    int s = check_layer_tensor(cursors, "channel_mix");
     for (const wrq_tensor *t : {r, v, x})
-        if (s == WRQ_OK) s = check_tensor(t, "channel_mix");
-    if (s == WRQ_OK) s = check_view(state, "channel_mix");
+        if (s == WRQ_OK) s = check_layer_tensor(t, "channel_mix");
+    if (s == WRQ_OK) s = check_layer_view(state, "channel_mix");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: the state is f32");
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: unsupported element type %d", (int)dtype);
@@ -315,10 +242,10 @@ int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
 
 int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
                     const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
-    int s = check_tensor(cursors, "time_mix_v6");
+    int s = check_layer_tensor(cursors, "time_mix_v6");
     for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
-        if (s == WRQ_OK) s = check_tensor(t, "time_mix_v6");
-    if (s == WRQ_OK) s = check_view(state, "time_mix_v6");
+        if (s == WRQ_OK) s = check_layer_tensor(t, "time_mix_v6");
+    if (s == WRQ_OK) s = check_layer_view(state, "time_mix_v6");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: the state is f32");
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: unsupported element type %d", (int)dtype);

@@ -7,7 +7,7 @@ import importlib
 import numpy as np
 
 _pkg = importlib.import_module(__name__.rsplit(".", 1)[0])
-LayerOp, Matrix, turbo, matmul_vec_group = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo, _pkg.matmul_vec_group
+LayerOp, Matrix, turbo, matmul_vec_group, FusedV6 = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo, _pkg.matmul_vec_group, _pkg.FusedV6
 ACT_NONE, ACT_SQUARED_RELU, ACT_TANH, ACT_STABLE_EXP, ACT_SILU = _pkg.ACT_NONE, _pkg.ACT_SQUARED_RELU, _pkg.ACT_TANH, _pkg.ACT_STABLE_EXP, _pkg.ACT_SILU
 
 LN_EPS = 1.0e-5   # Model::LN_EPS, src/runtime/v6.rs:46
@@ -69,6 +69,7 @@ class Runtime:
         self.time_mix_x, self.time_mix_t = z(A, 5, TIME_MIX_LORA), z(5, A, TIME_MIX_LORA)
         self.ffn_x, self.ffn_kx, self.ffn_rx, self.ffn_v, self.ffn_r = (z(1, A, C) for _ in range(5))
         self.ffn_k = z(1, A, hidden)
+        self.x2 = z(1, A, C)  # the residual between the two halves of a layer on the fused path
 
 
 def dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now=False):
@@ -116,3 +117,31 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now=False):
     LayerOp.add(buf.ffn_x, buf.x)
     if rescale_now:
         LayerOp.affine(buf.x, 0.5, 0.0)
+
+
+def dispatch_layer_fused(layer, buf, state, cursors, A, H, S, rescale_now=False):
+    """The same layer in 12 launches: the 8 quantized products (3 launches for the independent ones, 2
+    alone), the first halves of the two adapters, and 5 fused launches for the 27 small ops
+    (`wrq_v6_*`).  Same buffers and results as `dispatch_layer` up to f32 summation order."""
+    t, m, C = layer.t, layer.m, H * S
+    B = state.shape[0]
+    fast = turbo(A)
+    att_state = ((C, S + 1, B), (C, S + 2, B), (0, 0, 0))
+    ffn_state = ((C, 1, B), (C, S + 2, B), (0, S + 1, 0))
+    slice_of = lambda i: ((C, A, 1), (C, A, 5), (0, 0, i))
+
+    FusedV6.pre(C, A, cursors, buf.x, None, None, t["att_ln_w"], t["att_ln_b"], LN_EPS, state, att_state, [t["time_mix_x"]], buf.att_x, [buf.att_xx])
+    m["time_mix_w1"].matmul_op(buf.att_xx, buf.time_mix_x.view(1, A, 5 * TIME_MIX_LORA), ACT_TANH, fast)
+    FusedV6.time_mix(C, A, TIME_MIX_LORA, cursors, buf.time_mix_x, t["time_mix_w2"], t["time_mix"], state, att_state, buf.att_x, buf.att_sx)
+    matmul_vec_group([(m[n], buf.att_sx, out, ACT_NONE, False, dict(input_view=slice_of(i)))
+                      for n, out, i in (("att_w_k", buf.att_k, 1), ("att_w_v", buf.att_v, 2), ("att_w_r", buf.att_r, 3), ("att_w_g", buf.att_g, 4))])
+    m["time_decay_w1"].matmul_op(buf.att_sx, buf.att_w, ACT_TANH, fast, input_view=slice_of(0))
+    FusedV6.decay(C, A, TIME_DECAY_LORA, buf.att_w, t["time_decay_w2"], t["time_decay"], buf.time_decay)
+    FusedV6.wkv_gate(S, H, A, cursors, buf.time_decay, t["time_first"], state, att_state, buf.att_k, buf.att_v, buf.att_r, buf.att_g, t["gn_w"], t["gn_b"],
+                     GN_EPS, buf.att_x)
+    m["att_w_o"].matmul_op(buf.att_x, buf.att_o, ACT_NONE, fast)
+    FusedV6.pre(C, A, cursors, buf.x, buf.att_o, buf.x2, t["ffn_ln_w"], t["ffn_ln_b"], LN_EPS, state, ffn_state, [t["ffn_time_mix_k"], t["ffn_time_mix_r"]],
+                buf.ffn_x, [buf.ffn_kx, buf.ffn_rx])
+    matmul_vec_group([(m["ffn_w_k"], buf.ffn_kx, buf.ffn_k, ACT_SQUARED_RELU, False, {}), (m["ffn_w_r"], buf.ffn_rx, buf.ffn_r, ACT_NONE, False, {})])
+    m["ffn_w_v"].matmul_op_sparse(buf.ffn_k, buf.ffn_v, ACT_NONE, fast)
+    FusedV6.post_ffn(C, A, cursors, state, ffn_state, buf.ffn_r, buf.ffn_v, buf.ffn_x, buf.x2, buf.x, rescale_now)
