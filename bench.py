@@ -405,7 +405,7 @@ def full_layers(wrq, torch, args, C, H):
     # one request in slot 0 whose A tokens fill the stack (the reference packs the count into 8 bits)
     cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
     x0 = buf.x.clone()
-    dispatch = v6.dispatch_layer_fused if args.fused else v6.dispatch_layer
+    dispatch = v6.dispatch_layer_auto if args.fused else v6.dispatch_layer
     model = args.full_model
     if model:
         # the ends of the model (src/runtime/v6.rs:625-640, :960-1000): embedding + its layer norm in front,
@@ -451,7 +451,7 @@ def full_layers(wrq, torch, args, C, H):
     print(json.dumps({"metric": what, "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
                       "config": {"workload": f"{args.layers} v6 layers ({C} x {H}, {heads} heads), {args.quant}, {A} token(s) of one request per step, "
-                                             + ("12 launches per layer (fused small ops)" if args.fused else "35 ops per layer"),
+                                             + ("12 launches per layer (fused small ops)" if args.fused and A <= v6.FUSED_MAX_TOKENS else "35 ops per layer"),
                                  "hip_graph": not args.no_graph}, "data": "synthetic"}))
 
 

@@ -157,11 +157,24 @@ __global__ __launch_bounds__(64) void v6_wkv_gate_kernel(const uint32_t *cursors
     const float gw = h2f(gn_w[chan]), gb = h2f(gn_b[chan]);
     float s[S];
     uint32_t held = 0xffffffffu;
+    // the operands of the next token are fetched while this one is worked on (clamped at the end)
+    float nk = k[chan], nr = r[chan], nw = decay[chan], nv = v[chan];
+    uint16_t ng = g[chan], nx = att_x[chan];
+    uint32_t ncur = cursors[0];
     for (uint32_t t = 0; t < A; t++) {
-        const Cursor cur = read_cursor(cursors, t, vs);
+        const float ck = nk, cr = nr, cw = nw, vv = nv;
+        const uint16_t cg = ng, cx = nx;
+        Cursor cur = unpack_cursor(ncur);
+        cur.batch = min(cur.batch, vs.shape[2] - 1); // as read_cursor
+        cur.token = min(cur.token, t);
         const uint64_t ti = (uint64_t)t * C + chan;
+        {
+            const uint64_t tn = (uint64_t)min(t + 1, A - 1) * C + chan;
+            nk = k[tn], nr = r[tn], nw = decay[tn], nv = v[tn], ng = g[tn], nx = att_x[tn];
+            ncur = cursors[min(t + 1, A - 1)];
+        }
         __syncthreads(); // the previous token's reads of ks / rs / ws are done
-        ks[i] = k[ti], rs[i] = r[ti], ws[i] = decay[ti];
+        ks[i] = ck, rs[i] = cr, ws[i] = cw;
         if (cur.batch != held) {
             if (held != 0xffffffffu) {
 #pragma unroll
@@ -172,8 +185,7 @@ __global__ __launch_bounds__(64) void v6_wkv_gate_kernel(const uint32_t *cursors
             for (int j = 0; j < S; j++) s[j] = state[view_elem(vs, held, j + 1, chan)];
         }
         // row 0 of the request's state keeps the layer's normalised input at its last token
-        if (t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = h2f(att_x[ti]);
-        const float vv = v[ti];
+        if (t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = h2f(cx);
         __syncthreads();
         float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -192,7 +204,7 @@ __global__ __launch_bounds__(64) void v6_wkv_gate_kernel(const uint32_t *cursors
         const float mean = wave_sum(y) * (1.0f / S);
         const float dev = rsqrtf(wave_sum((y - mean) * (y - mean)) * (1.0f / S) + eps);
         const float gn = round_h(fmaf((y - mean) * dev, gw, gb));
-        att_x[ti] = f2h(act_one<WRQ_ACT_SILU>(h2f(g[ti])) * gn);
+        att_x[ti] = f2h(act_one<WRQ_ACT_SILU>(h2f(cg)) * gn);
     }
     if (held != 0xffffffffu) {
 #pragma unroll

@@ -11,9 +11,8 @@
 // per head, token after token.  The shader re-reads and re-writes the head's S (64 x 64 f32) in memory
 // for every token; here a request's S stays in registers for all its tokens of the run: four lanes
 // share an output element i and hold a quarter of j each (16 values of S), one DPP quad reduction
-// per token, no LDS and no barrier; S is read when a request's tokens begin and written when they
-// end.  The sum over j is therefore taken in four interleaved partial sums instead of one chain
-// (a difference of rounding order only).
+// per token; S is read when a request's tokens begin and written when they end.  The sum over j is
+// therefore taken in interleaved partial sums instead of one chain (a difference of rounding order only).
 #include "layer_device.h"
 
 namespace wrq {
@@ -55,8 +54,6 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
-// One workgroup per head: thread = (output element i of the head, quarter q of the j range), four
-// waves of 16 i x 4 q.  S = head size (a multiple of 16, at most 256: JQ = S / 4 values of S per lane).
 // One workgroup per head: thread = (output element i of the head, quarter q of the j range), four
 // waves of 16 i x 4 q; JQ = S / 4 values of S[.][i] per lane.  The operands of the head (k, r, w, v:
 // S values each per token) come in chunks of 1024 / S tokens: every thread fetches one 4-element

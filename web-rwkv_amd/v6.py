@@ -145,3 +145,14 @@ def dispatch_layer_fused(layer, buf, state, cursors, A, H, S, rescale_now=False)
     matmul_vec_group([(m["ffn_w_k"], buf.ffn_kx, buf.ffn_k, ACT_SQUARED_RELU, False, {}), (m["ffn_w_r"], buf.ffn_rx, buf.ffn_r, ACT_NONE, False, {})])
     m["ffn_w_v"].matmul_op_sparse(buf.ffn_k, buf.ffn_v, ACT_NONE, fast)
     FusedV6.post_ffn(C, A, cursors, state, ffn_state, buf.ffn_r, buf.ffn_v, buf.ffn_x, buf.x2, buf.x, rescale_now)
+
+
+FUSED_MAX_TOKENS = 16  # measured: beyond this the op list's chunked kernels win (the fused ones walk tokens one by one)
+
+
+def dispatch_layer_auto(layer, buf, state, cursors, A, H, S, rescale_now=False):
+    """The fused form for short runs (decode and the tail of a schedule), the op list beyond."""
+    if A <= FUSED_MAX_TOKENS and S == 64:
+        dispatch_layer_fused(layer, buf, state, cursors, A, H, S, rescale_now)
+    else:
+        dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now)
