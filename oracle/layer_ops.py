@@ -242,3 +242,25 @@ def time_mix_v6(cursors, time_decay, time_first, state, k, v, r, x):
             state[slot, 1 + j] = _fma(np.broadcast_to(w32[t, :, j:j + 1], (H, S)), ss, kv).reshape(-1)
         out[t] = y
     return out.astype(x.dtype)
+
+
+def time_mix_v5(cursors, time_decay, time_first, state, k, v, r, x):
+    """src/shaders/time_mix_v5.wgsl:86-155.  k, v, r, x (A, H, S); time_decay, time_first (H, S): the
+    decay is a constant of the channel; state (B, S + 1, H * S) f32 updated in place (row 0: x at a
+    request's last token; row 1 + j: S[j][.]); the sum over j in the shader's order.  Returns the new x."""
+    x = np.asarray(x)
+    A, H, S = x.shape
+    k32, v32, r32, w32, u32 = (np.asarray(t).astype(F) for t in (k, v, r, time_decay, time_first))
+    out = np.empty((A, H, S), dtype=F)
+    for t in range(A):
+        slot, first, n = _cursor(cursors[t])
+        if t - first + 1 == n:
+            state[slot, 0] = x[first + n - 1].astype(F).reshape(-1)
+        y = np.zeros((H, S), dtype=F)
+        for j in range(S):
+            ss = state[slot, 1 + j].reshape(H, S)
+            kv = k32[t, :, j:j + 1] * v32[t]
+            y = y + r32[t, :, j:j + 1] * _fma(np.broadcast_to(u32[:, j:j + 1], (H, S)), kv, ss)
+            state[slot, 1 + j] = _fma(np.broadcast_to(w32[:, j:j + 1], (H, S)), ss, kv).reshape(-1)
+        out[t] = y
+    return out.astype(x.dtype)

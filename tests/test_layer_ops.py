@@ -313,6 +313,72 @@ def test_gpu_time_mix_v6(gpu, lop, dtype, H, S, runs):
 
 
 # ---------------------------------------------------------------------------------------------
+def test_oracle_time_mix_v5(lop):
+    # v5 is the recurrence with one decay per channel (src/shaders/time_mix_v5.wgsl:120-152): the
+    # float64 textbook form with that decay repeated for every token, and bit equality with the v6
+    # restatement on the repeated decay (the shaders differ only in where w comes from)
+    rng = np.random.default_rng(SEED + 8)
+    H, S, B = 3, 16, 6
+    cur = lop.pack_cursors(RUNS)
+    A = len(cur)
+    k, v, r, x, w, u, state = wkv6_inputs(rng, A, H, S, B, np.float32)
+    w5 = w[0]
+    wrep = np.broadcast_to(w5, (A, H, S))
+    st = state.copy()
+    got = lop.time_mix_v5(cur, w5, u, st, k, v, r, x)
+    want, want_state = wkv6_float64(cur, wrep, u, state, k, v, r, x)
+    assert_close(got, want, 1e-5, "y vs float64")
+    assert_close(st, want_state, 1e-5, "state vs float64")
+    st6 = state.copy()
+    assert np.array_equal(got, lop.time_mix_v6(cur, wrep, u, st6, k, v, r, x)) and np.array_equal(st, st6)
+    # n tokens of one request from a zero state with r = 1, u = 0: y_t[i] = sum_j sum_{s<t} w_j^(t-1-s) k_s[j] v_s[i]
+    n = 5
+    z = np.zeros_like(state)
+    ones = np.ones((n, H, S), dtype=np.float32)
+    y = lop.time_mix_v5(lop.pack_cursors([(2, n)]), w5, np.zeros_like(u), z, k[:n], v[:n], ones, x[:n])
+    w64, k64, v64 = w5.astype(np.float64), k[:n].astype(np.float64), v[:n].astype(np.float64)
+    for t in range(n):
+        closed = sum(((w64 ** (t - 1 - s)) * k64[s]).sum(axis=-1, keepdims=True) * v64[s] for s in range(t)) if t else np.zeros((H, S))
+        assert_close(y[t], closed, 1e-5, f"geometric closed form, token {t}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("H,S,runs", [(3, 16, RUNS), (12, 64, RUNS), (12, 64, [(0, 1)]), (2, 128, [(1, 2), (3, 2)]), (2, 64, [(4, 100)])])
+def test_gpu_time_mix_v5(gpu, lop, dtype, H, S, runs):
+    import torch
+
+    print("time mix v5 on the GPU", dtype.__name__, H, S, runs[:3], flush=True)
+    rng = np.random.default_rng(SEED + 80 + H + S)
+    B = 6
+    cur = lop.pack_cursors(runs)
+    A = len(cur)
+    k, v, r, x, w, u, state = wkv6_inputs(rng, A, H, S, B, dtype)
+    w5 = np.ascontiguousarray(w[0])
+    full = np.concatenate([np.zeros_like(state), state], axis=1)
+    sview = ((H * S, S + 1, B), (H * S, 2 * (S + 1), B), (0, S + 1, 0))
+    sd = torch.from_numpy(full.copy()).cuda()
+    xd = torch.from_numpy(x.copy()).cuda()
+    gpu.LayerOp.time_mix_v5(torch.from_numpy(cur.view(np.int32)).cuda(), torch.from_numpy(w5).cuda(), torch.from_numpy(u).cuda(), sd,
+                            torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), torch.from_numpy(r).cuda(), xd, state_view=sview)
+    want, want_state = wkv6_float64(cur, np.broadcast_to(w5, (A, H, S)), u, state, k, v, r, x)
+    eps = 2e-3 if dtype == np.float16 else 2e-5
+    assert_close(xd.cpu().numpy(), want, eps, "y vs float64")
+    got_state = sd.cpu().numpy()
+    assert_close(got_state[:, S + 1:], want_state, 2e-5, "state vs float64")
+    assert np.array_equal(got_state[:, :S + 1], full[:, :S + 1])  # the other layer's rows are untouched
+    if A * H * S * S <= 2000000:
+        st = state.copy()
+        assert_close(xd.cpu().numpy(), lop.time_mix_v5(cur, w5, u, st, k, v, r, x), eps, "y vs oracle")
+        assert_close(got_state[:, S + 1:], st, 2e-5, "state vs oracle")
+    # a per-token decay tensor is the v6 op's operand, not this one's
+    if A > 1:
+        with pytest.raises(gpu.TensorError):
+            gpu.LayerOp.time_mix_v5(torch.from_numpy(cur.view(np.int32)).cuda(), torch.from_numpy(w).cuda(), torch.from_numpy(u).cuda(), sd,
+                                    torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), torch.from_numpy(r).cuda(), xd, state_view=sview)
+
+
+# ---------------------------------------------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_data_movement_kats(gpu):
     import torch

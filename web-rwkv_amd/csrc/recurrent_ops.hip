@@ -1,6 +1,7 @@
-// The ops of a v6 layer that carry state from token to token:
+// The ops of a v5 / v6 layer that carry state from token to token:
 //   token_shift   src/tensor/ops.rs:1393-1462, src/shaders/token_shift.wgsl
 //   channel_mix   src/tensor/ops.rs:1860-1915, src/shaders/channel_mix.wgsl
+//   time_mix_v5   src/tensor/ops.rs:1530-1599, src/shaders/time_mix_v5.wgsl
 //   time_mix_v6   src/tensor/ops.rs:1601-1677, src/shaders/time_mix_v6.wgsl
 //
 // A run is a stack of A tokens from several requests; `cursors[a]` packs, for the request of token
@@ -8,7 +9,8 @@
 // of its tokens in the stack (8 bits) (`compute_cursor` of the shaders).
 //
 // time_mix_v6 is the recurrence  y[i] = sum_j r[j] (u[j] k[j] v[i] + S[j][i]),  S[j][i] <- w[j] S[j][i] + k[j] v[i]
-// per head, token after token.  The shader re-reads and re-writes the head's S (64 x 64 f32) in memory
+// per head, token after token; time_mix_v5 is the same recurrence with a decay w that is a constant of
+// the channel instead of a value per token (one kernel, TOKEN_DECAY tells them apart).  The shader re-reads and re-writes the head's S (64 x 64 f32) in memory
 // for every token; here a request's S stays in registers for all its tokens of the run: four lanes
 // share an output element i and hold a quarter of j each (16 values of S), one DPP quad reduction
 // per token; S is read when a request's tokens begin and written when they end.  The sum over j is
@@ -59,8 +61,8 @@ __device__ __forceinline__ float quad_sum(float v) {
 // S values each per token) come in chunks of 1024 / S tokens: every thread fetches one 4-element
 // vector of each while the previous chunk is worked on, and the chunk is passed round through LDS
 // (two buffers), from where the lanes of a quarter read their j range as broadcasts.
-template <typename XT, int JQ>
-__global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursors, const float *time_decay, const float *time_first, float *state, const XT *k,
+template <typename XT, int JQ, bool TOKEN_DECAY>
+__global__ __launch_bounds__(256) void time_mix_kernel(const uint32_t *cursors, const float *time_decay, const float *time_first, float *state, const XT *k,
                                                           const XT *v, const XT *r, XT *x, ViewArgs vs, uint32_t S, uint32_t H, uint32_t A) {
     constexpr int SZ = 4 * JQ;      // head size
     constexpr int TB = 1024 / SZ;   // tokens per chunk
@@ -77,13 +79,14 @@ __global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursor
     auto fetch = [&](uint32_t chunk) {
         const uint32_t t = min(chunk * TB + lt, A - 1); // clamped: tokens past the run are never used
         const uint64_t g = (uint64_t)t * C + head * SZ + le;
-        fk = load_vec4(k + g), fr = load_vec4(r + g), fw = load_vec4(time_decay + g), fv = load_vec4(v + g);
+        fk = load_vec4(k + g), fr = load_vec4(r + g), fv = load_vec4(v + g);
+        if constexpr (TOKEN_DECAY) fw = load_vec4(time_decay + g);
         if (tid < (uint32_t)TB) fc = cursors[min(chunk * TB + tid, A - 1)];
     };
     auto stage = [&](int buf) {
         *reinterpret_cast<float4 *>(&ks[buf][4 * tid]) = fk;
         *reinterpret_cast<float4 *>(&rs[buf][4 * tid]) = fr;
-        *reinterpret_cast<float4 *>(&ws[buf][4 * tid]) = fw;
+        if constexpr (TOKEN_DECAY) *reinterpret_cast<float4 *>(&ws[buf][4 * tid]) = fw;
         *reinterpret_cast<float4 *>(&vsh[buf][4 * tid]) = fv;
         if (tid < (uint32_t)TB) csh[buf][tid] = fc;
     };
@@ -91,11 +94,15 @@ __global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursor
         const uint32_t i = i0 + (tid >> 2);
         const bool live = i < SZ; // head sizes below 64 leave waves without an output element
         const uint32_t chan = head * SZ + min(i, (uint32_t)SZ - 1);
-        float u[JQ], s[JQ];
+        float u[JQ], s[JQ], wc[TOKEN_DECAY ? 1 : JQ]; // wc: the constant decay of this lane's j range
 #pragma unroll
         for (int c = 0; c < JQ / 4; c++) {
             const float4 t4 = *reinterpret_cast<const float4 *>(time_first + head * SZ + q * JQ + 4 * c);
             u[4 * c] = t4.x, u[4 * c + 1] = t4.y, u[4 * c + 2] = t4.z, u[4 * c + 3] = t4.w;
+            if constexpr (!TOKEN_DECAY) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(time_decay + head * SZ + q * JQ + 4 * c);
+                wc[4 * c] = d4.x, wc[4 * c + 1] = d4.y, wc[4 * c + 2] = d4.z, wc[4 * c + 3] = d4.w;
+            }
         }
         uint32_t held = 0xffffffffu; // request whose S is in registers
         fetch(0);
@@ -129,9 +136,15 @@ __global__ __launch_bounds__(256) void time_mix_v6_kernel(const uint32_t *cursor
                     float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // four chains instead of one of JQ dependent adds
 #pragma unroll
                     for (int c = 0; c < JQ / 4; c++) {
-                        const float4 k4 = *reinterpret_cast<const float4 *>(kp + 4 * c), r4 = *reinterpret_cast<const float4 *>(rp + 4 * c),
-                                     w4 = *reinterpret_cast<const float4 *>(wp + 4 * c);
-                        const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, rr[4] = {r4.x, r4.y, r4.z, r4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+                        const float4 k4 = *reinterpret_cast<const float4 *>(kp + 4 * c), r4 = *reinterpret_cast<const float4 *>(rp + 4 * c);
+                        const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, rr[4] = {r4.x, r4.y, r4.z, r4.w};
+                        float ww[4];
+                        if constexpr (TOKEN_DECAY) {
+                            const float4 w4 = *reinterpret_cast<const float4 *>(wp + 4 * c);
+                            ww[0] = w4.x, ww[1] = w4.y, ww[2] = w4.z, ww[3] = w4.w;
+                        } else {
+                            ww[0] = wc[4 * c], ww[1] = wc[4 * c + 1], ww[2] = wc[4 * c + 2], ww[3] = wc[4 * c + 3];
+                        }
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const float kv = kk[e] * vv;
@@ -237,43 +250,66 @@ int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
     return check_launch("channel_mix");
 }
 
-int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
-                    const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
-    int s = check_layer_tensor(cursors, "time_mix_v6");
+} // extern "C"
+
+namespace {
+
+// time_mix_v5 (token_decay == false: time_decay [S, H, 1, 1]) and time_mix_v6 (time_decay [S, H, A, 1])
+int time_mix(const char *name, bool token_decay, wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first,
+             const wrq_tensor_view *state, const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
+    int s = check_layer_tensor(cursors, name);
     for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
-        if (s == WRQ_OK) s = check_layer_tensor(t, "time_mix_v6");
-    if (s == WRQ_OK) s = check_layer_view(state, "time_mix_v6");
+        if (s == WRQ_OK) s = check_layer_tensor(t, name);
+    if (s == WRQ_OK) s = check_layer_view(state, name);
     if (s != WRQ_OK) return s;
-    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: the state is f32");
-    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v6: unsupported element type %d", (int)dtype);
+    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: the state is f32", name);
+    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", name, (int)dtype);
     const uint32_t *sh = x->shape, *st = state->view.shape; // [S, H, A, 1]
     const uint32_t S = sh[0], H = sh[1], A = sh[2];
-    // src/tensor/ops.rs:1620-1625
+    // src/tensor/ops.rs:1546-1553 (v5), 1620-1625 (v6)
     const uint32_t tf[4] = {S, H, 1, 1};
-    if (sh[3] != 1 || !same_shape(k->shape, sh) || !same_shape(v->shape, sh) || !same_shape(r->shape, sh) || !same_shape(time_decay->shape, sh) ||
+    if (sh[3] != 1 || !same_shape(k->shape, sh) || !same_shape(v->shape, sh) || !same_shape(r->shape, sh) || !same_shape(time_decay->shape, token_decay ? sh : tf) ||
         !same_shape(time_first->shape, tf) || st[0] != S * H || st[1] != S + 1 || st[3] != 1)
-        return fail(WRQ_ERR_SHAPE, "time_mix_v6: data shape not match [%u, %u, %u, %u]", sh[0], sh[1], sh[2], sh[3]);
-    if (cursors->shape[0] < A) return fail(WRQ_ERR_SHAPE, "time_mix_v6: %u cursors for %u tokens", cursors->shape[0], A);
+        return fail(WRQ_ERR_SHAPE, "%s: data shape not match [%u, %u, %u, %u]", name, sh[0], sh[1], sh[2], sh[3]);
+    if (cursors->shape[0] < A) return fail(WRQ_ERR_SHAPE, "%s: %u cursors for %u tokens", name, cursors->shape[0], A);
     if (S == 0 || H == 0 || A == 0) return WRQ_OK;
-    if (S % 16 || S > 256) return fail(WRQ_ERR_UNSUPPORTED, "time_mix_v6: head size %u (a multiple of 16 up to 256 is built)", S);
     const ViewArgs vs = view_args(state->view);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     const uint32_t *cur = static_cast<const uint32_t *>(cursors->data);
     const float *td = static_cast<const float *>(time_decay->data), *tfp = static_cast<const float *>(time_first->data);
     float *sp = static_cast<float *>(state->data);
-#define WRQ_TM(JQ)                                                                                                                                           \
-    if (S == 4 * JQ) {                                                                                                                                       \
-        if (dtype == WRQ_F16)                                                                                                                                \
-            hipLaunchKernelGGL((time_mix_v6_kernel<uint16_t, JQ>), dim3(H), dim3(256), 0, hs, cur, td, tfp, sp, static_cast<const uint16_t *>(k->data),      \
-                               static_cast<const uint16_t *>(v->data), static_cast<const uint16_t *>(r->data), static_cast<uint16_t *>(x->data), vs, S, H, A); \
-        else                                                                                                                                                 \
-            hipLaunchKernelGGL((time_mix_v6_kernel<float, JQ>), dim3(H), dim3(256), 0, hs, cur, td, tfp, sp, static_cast<const float *>(k->data),            \
-                               static_cast<const float *>(v->data), static_cast<const float *>(r->data), static_cast<float *>(x->data), vs, S, H, A);        \
-        return check_launch("time_mix_v6");                                                                                                                  \
+#define WRQ_TM_LAUNCH(XT, JQ, TD)                                                                                                                \
+    hipLaunchKernelGGL((time_mix_kernel<XT, JQ, TD>), dim3(H), dim3(256), 0, hs, cur, td, tfp, sp, static_cast<const XT *>(k->data),               \
+                       static_cast<const XT *>(v->data), static_cast<const XT *>(r->data), static_cast<XT *>(x->data), vs, S, H, A)
+#define WRQ_TM(JQ)                                                                                                                               \
+    if (S == 4 * JQ) {                                                                                                                           \
+        if (dtype == WRQ_F16) {                                                                                                                  \
+            if (token_decay) WRQ_TM_LAUNCH(uint16_t, JQ, true);                                                                                  \
+            else WRQ_TM_LAUNCH(uint16_t, JQ, false);                                                                                             \
+        } else {                                                                                                                                 \
+            if (token_decay) WRQ_TM_LAUNCH(float, JQ, true);                                                                                     \
+            else WRQ_TM_LAUNCH(float, JQ, false);                                                                                                \
+        }                                                                                                                                        \
+        return check_launch(name);                                                                                                               \
     }
     WRQ_TM(4) WRQ_TM(8) WRQ_TM(16) WRQ_TM(32) WRQ_TM(64)
 #undef WRQ_TM
-    return fail(WRQ_ERR_UNSUPPORTED, "time_mix_v6: head size %u (16, 32, 64, 128 or 256 is built)", S);
+#undef WRQ_TM_LAUNCH
+    return fail(WRQ_ERR_UNSUPPORTED, "%s: head size %u (16, 32, 64, 128 or 256 is built)", name, S);
+}
+
+} // namespace
+
+extern "C" {
+
+int wrq_time_mix_v5(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
+                    const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
+    return time_mix("time_mix_v5", false, stream, cursors, time_decay, time_first, state, k, v, r, x, dtype);
+}
+
+int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
+                    const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
+    return time_mix("time_mix_v6", true, stream, cursors, time_decay, time_first, state, k, v, r, x, dtype);
 }
 
 } // extern "C"

@@ -1,0 +1,101 @@
+"""Host-side mirror of one RWKV-v5 layer as the reference dispatches it (src/runtime/v5.rs:651-890):
+the same ops in the same order on the same buffers, every op one library call on torch's current
+stream.  Weights are random-init tensors of the reference's shapes (src/runtime/v5.rs:60-105,
+:945-1036); nothing here loads a checkpoint."""
+import importlib
+
+import numpy as np
+
+_pkg = importlib.import_module(__name__.rsplit(".", 1)[0])
+LayerOp, Matrix, turbo, matmul_vec_group = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo, _pkg.matmul_vec_group
+ACT_NONE, ACT_SQUARED_RELU, ACT_SILU = _pkg.ACT_NONE, _pkg.ACT_SQUARED_RELU, _pkg.ACT_SILU
+
+LN_EPS = 1.0e-5   # Model::LN_EPS, src/runtime/v5.rs:45
+GN_EPS = 64.0e-5  # Model::GN_EPS, src/runtime/v5.rs:46
+
+QUANTIZED = ("att_w_k", "att_w_v", "att_w_r", "att_w_g", "att_w_o", "ffn_w_k", "ffn_w_v", "ffn_w_r")
+
+
+def random_layer_weights(rng, C, H, S, hidden, layer=0):
+    """numpy weights of one layer: matrices [out, in] f16 ~ N(0, 0.02) (att.output and ffn.value with the
+    loader's 2^-(layer / 6) discount, src/runtime/loader.rs:660-661), vectors of plausible ranges;
+    time_decay as the loader leaves it, exp(-exp(w)) (src/runtime/loader.rs:472-520)."""
+    h16 = lambda *s, std=0.02: (rng.standard_normal(s, dtype=np.float32) * np.float32(std)).astype(np.float16)
+    disc = np.float32(2.0 ** -(layer // 6))
+    w = {
+        "att_ln_w": (1.0 + 0.1 * rng.standard_normal(C)).astype(np.float16), "att_ln_b": h16(C, std=0.1),
+        "ffn_ln_w": (1.0 + 0.1 * rng.standard_normal(C)).astype(np.float16), "ffn_ln_b": h16(C, std=0.1),
+        "time_decay": np.exp(-np.exp((-1.0 + 0.5 * rng.standard_normal((H, S))).astype(np.float32))).astype(np.float32),
+        "time_first": (0.3 * rng.standard_normal((H, S))).astype(np.float32),
+        "gn_w": (1.0 + 0.1 * rng.standard_normal((H, S))).astype(np.float16), "gn_b": h16(H, S, std=0.1),
+    }
+    for name in ("time_mix_k", "time_mix_v", "time_mix_r", "time_mix_g", "ffn_time_mix_k", "ffn_time_mix_r"):
+        w[name] = rng.random(C).astype(np.float16)
+    for name, (R, K) in {"att_w_k": (C, C), "att_w_v": (C, C), "att_w_r": (C, C), "att_w_g": (C, C), "att_w_o": (C, C),
+                         "ffn_w_k": (hidden, C), "ffn_w_v": (C, hidden), "ffn_w_r": (C, C)}.items():
+        m = rng.standard_normal((R, K), dtype=np.float32) * np.float32(0.02)
+        if name in ("att_w_o", "ffn_w_v"):
+            m = m * disc
+        w[name] = m.astype(np.float16)
+    return w
+
+
+class Layer:
+    """Device weights of one layer: the eight matrices quantised (`quant`: "int8" or "nf4"), vectors
+    as the reference keeps them."""
+
+    def __init__(self, torch, weights, quant):
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        self.t = {k: dev(v) for k, v in weights.items() if k not in QUANTIZED}
+        pack = Matrix.quant_u8 if quant == "int8" else Matrix.quant_nf4
+        self.m = {k: pack(dev(weights[k])) for k in QUANTIZED}
+
+
+class Runtime:
+    """The buffers of a run of `A` tokens (`Runtime<F>`, src/runtime/v5.rs:258-313), F = f16."""
+
+    def __init__(self, torch, C, hidden, A):
+        z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device="cuda")
+        f32 = torch.float32
+        self.x, self.att_x, self.att_kx, self.att_vx, self.att_rx, self.att_gx, self.att_g, self.att_o = (z(1, A, C) for _ in range(8))
+        self.aux_x, self.att_k, self.att_v, self.att_r = (z(1, A, C, dt=f32) for _ in range(4))
+        self.ffn_x, self.ffn_kx, self.ffn_rx, self.ffn_v, self.ffn_r = (z(1, A, C) for _ in range(5))
+        self.ffn_k = z(1, A, hidden)
+
+
+def dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now=False):
+    """src/runtime/v5.rs:651-890.  `state`: this layer's f32 tensor (B, S + 2, C): rows 0..S the
+    attention state (`State::att`, :175-179), row S + 1 the feed-forward one (`State::ffn`, :181-185)."""
+    t, m, C = layer.t, layer.m, H * S
+    B = state.shape[0]
+    fast = turbo(A)
+    att_state = ((C, S + 1, B), (C, S + 2, B), (0, 0, 0))
+    ffn_state = ((C, 1, B), (C, S + 2, B), (0, S + 1, 0))
+    heads = lambda x: x.view(A, H, S)
+
+    LayerOp.blit(buf.x, buf.att_x)
+    LayerOp.layer_norm(t["att_ln_w"], t["att_ln_b"], buf.att_x, LN_EPS)
+    for name, out in (("time_mix_k", buf.att_kx), ("time_mix_v", buf.att_vx), ("time_mix_r", buf.att_rx), ("time_mix_g", buf.att_gx)):
+        LayerOp.token_shift(cursors, t[name], state, buf.att_x, out, False, state_view=att_state)
+    # the four independent projections in one call: the library's form of a `TensorOp::List` of them
+    matmul_vec_group([(m["att_w_k"], buf.att_kx, buf.att_k, ACT_NONE, False, {}), (m["att_w_v"], buf.att_vx, buf.att_v, ACT_NONE, False, {}),
+                      (m["att_w_r"], buf.att_rx, buf.att_r, ACT_NONE, False, {}), (m["att_w_g"], buf.att_gx, buf.att_g, ACT_NONE, False, {})])
+    LayerOp.blit(buf.att_x, buf.aux_x)
+    LayerOp.time_mix_v5(cursors, t["time_decay"], t["time_first"], state, heads(buf.att_k), heads(buf.att_v), heads(buf.att_r), heads(buf.aux_x),
+                        state_view=att_state)
+    LayerOp.group_norm(t["gn_w"], t["gn_b"], heads(buf.aux_x), GN_EPS)
+    LayerOp.blit(buf.aux_x, buf.att_x)
+    LayerOp.mul_activate(buf.att_g, buf.att_x, ACT_SILU, ACT_NONE, ACT_NONE)
+    m["att_w_o"].matmul_op(buf.att_x, buf.att_o, ACT_NONE, fast)
+    LayerOp.add(buf.att_o, buf.x)
+
+    LayerOp.blit(buf.x, buf.ffn_x)
+    LayerOp.layer_norm(t["ffn_ln_w"], t["ffn_ln_b"], buf.ffn_x, LN_EPS)
+    LayerOp.token_shift(cursors, t["ffn_time_mix_k"], state, buf.ffn_x, buf.ffn_kx, False, state_view=ffn_state)
+    LayerOp.token_shift(cursors, t["ffn_time_mix_r"], state, buf.ffn_x, buf.ffn_rx, False, state_view=ffn_state)
+    matmul_vec_group([(m["ffn_w_k"], buf.ffn_kx, buf.ffn_k, ACT_SQUARED_RELU, False, {}), (m["ffn_w_r"], buf.ffn_rx, buf.ffn_r, ACT_NONE, False, {})])
+    m["ffn_w_v"].matmul_op_sparse(buf.ffn_k, buf.ffn_v, ACT_NONE, fast)
+    LayerOp.channel_mix(cursors, state, buf.ffn_r, buf.ffn_v, buf.ffn_x, state_view=ffn_state)
+    LayerOp.add(buf.ffn_x, buf.x)
+    if rescale_now:
+        LayerOp.affine(buf.x, 0.5, 0.0)
