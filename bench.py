@@ -455,6 +455,36 @@ def full_layers(wrq, torch, args, C, H):
                                  "hip_graph": not args.no_graph}, "data": "synthetic"}))
 
 
+def v5_model(wrq, torch, args):
+    """Config 1 on the GPU: the v5-shape model, every op of a run through the library
+    (src/runtime/v5.rs:541-930), one request; the 32-token prompt run and the one-token decode run,
+    each a HIP graph."""
+    v5 = importlib.import_module("web-rwkv_amd.v5")
+    L, heads, S, hidden, V = 12, 12, 64, 2688, 65536
+    rng = np.random.default_rng(SEED + 1)
+    model = v5.Model(torch, v5.random_model_weights(rng, L, heads * S, heads, S, hidden, V), args.quant, heads, S, hidden, 1)
+    out = {}
+    for A in (32, 1):
+        model.run([int(t) for t in rng.integers(0, V, A)], 0)
+        torch.cuda.synchronize()
+        if args.no_graph:
+            fn = lambda A=A: model.dispatch(A)
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                model.dispatch(A)
+            fn = graph.replay
+        ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
+        out[A] = (ms, wall_ms)
+        assert torch.isfinite(model.buffers(A)[5]).all()
+    packed = sum(m.w.numel() * m.w.element_size() + m.m.numel() * 2 for layer in model.layers for m in layer.m.values())
+    print(json.dumps({"metric": "RWKV-v5-shape model (config 1), every op, decode tokens/s, batch 1", "value": round(1e3 / out[1][1], 2), "unit": "tok/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(out[1][1], 4), "gpu_ms_per_step": round(out[1][0], 4),
+                      "prompt_32_tokens_ms": round(out[32][1], 4), "prompt_tok_s": round(32e3 / out[32][1], 1),
+                      "config": {"workload": f"{L} v5 layers (768 x {hidden}, {heads} heads), {args.quant}, embedding, head 65536 x 768 f16 on the last token; "
+                                             "27 ops per layer", "hip_graph": not args.no_graph, "packed_bytes": packed}, "data": "synthetic"}))
+
+
 def ops_table(wrq, torch, args, C):
     """Time of every layer op alone at the 7B layer shape, A tokens (HIP graph of 20 calls)."""
     LayerOp = wrq.LayerOp
@@ -530,6 +560,8 @@ def main():
     ap.add_argument("--ops", action="store_true", help="time of every layer op alone at the 7B layer shape")
     ap.add_argument("--fused", action="store_true", help="with --full-layers / --full-model: the fused small ops (12 launches per layer instead of 35)")
     ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
+    ap.add_argument("--v5-model", action="store_true",
+                    help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
@@ -552,6 +584,9 @@ def main():
         return
     if args.full_layers or args.full_model:
         full_layers(wrq, torch, args, C, H)
+        return
+    if args.v5_model:
+        v5_model(wrq, torch, args)
         return
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
     if args.schedule:

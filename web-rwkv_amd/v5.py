@@ -126,22 +126,36 @@ class Model:
         self.layers = [Layer(torch, w, quant) for w in weights["layers"]]
         self.state = [torch.zeros((slots, S + 2, self.C), dtype=torch.float32, device="cuda") for _ in self.layers]
         self.vocab = weights["head"].shape[0]
+        self._buffers = {}
 
-    def run(self, tokens, slot):
-        """One run: `tokens` (up to 255) of the request in `slot`; returns the f32 logits after the last one."""
-        torch, C, A = self.torch, self.C, len(tokens)
-        buf = Runtime(torch, C, self.hidden, A)
-        ids = torch.tensor([list(tokens)], dtype=torch.int32, device="cuda")
-        cursors = torch.from_numpy(np.full(A, slot | (A << 24), dtype=np.uint32).view(np.int32)).cuda()
-        inp = torch.zeros((1, A, C), dtype=torch.float16, device="cuda")
+    def buffers(self, A):
+        """The buffers of runs of `A` tokens, made once per run length (`checkout_buffer`, src/runtime/v5.rs:497-510)."""
+        if A not in self._buffers:
+            torch, C = self.torch, self.C
+            z = lambda *s, dt: torch.zeros(s, dtype=dt, device="cuda")
+            self._buffers[A] = (Runtime(torch, C, self.hidden, A), z(1, A, dt=torch.int32), z(A, dt=torch.int32), z(1, A, C, dt=torch.float16),
+                                z(1, 1, C, dt=torch.float16), z(1, 1, self.vocab, dt=torch.float32))
+        return self._buffers[A]
+
+    def dispatch(self, A):
+        """The op list of one run of `A` tokens of one request on the buffers of that run length: nothing but
+        library calls on the current stream (a HIP graph can record it)."""
+        C = self.C
+        buf, ids, cursors, inp, head_x, logits = self.buffers(A)
         LayerOp.embed(ids, self.t["embed"], inp)
         LayerOp.layer_norm(self.t["embed_ln_w"], self.t["embed_ln_b"], inp, LN_EPS)
         LayerOp.blit(inp, buf.x)
         for i, (layer, st) in enumerate(zip(self.layers, self.state)):
             dispatch_layer(layer, buf, st, cursors, A, self.H, self.S, rescale_now=(i + 1) % self.rescale == 0)
-        head_x = torch.zeros((1, 1, C), dtype=torch.float16, device="cuda")
-        logits = torch.zeros((1, 1, self.vocab), dtype=torch.float32, device="cuda")
         LayerOp.blit(buf.x, head_x, input_view=((C, 1, 1), (C, A, 1), (0, A - 1, 0)))
         LayerOp.layer_norm(self.t["head_ln_w"], self.t["head_ln_b"], head_x, LN_EPS)
         self.head.matmul_op(head_x, logits, ACT_NONE, turbo(1))
         return logits.view(-1)
+
+    def run(self, tokens, slot):
+        """One run: `tokens` (up to 255) of the request in `slot`; returns the f32 logits after the last one."""
+        torch, A = self.torch, len(tokens)
+        _, ids, cursors, _, _, _ = self.buffers(A)
+        ids.copy_(torch.tensor([list(tokens)], dtype=torch.int32))
+        cursors.copy_(torch.from_numpy(np.full(A, slot | (A << 24), dtype=np.uint32).view(np.int32)))
+        return self.dispatch(A)
