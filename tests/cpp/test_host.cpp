@@ -1,6 +1,6 @@
 // Tests of the C++ host mirror (include/wrq.hpp).  `--cpu`: everything that needs no device
 // (token schedule against the literal expectations of src/runtime/infer/rnn.rs:362-569,
-// op-build shape errors).  Without flag: the same API driving the GPU, checked against a
+// op-build shape errors, the on-disk form of packed matrices against RFC 8949's examples).  Without flag: the same API driving the GPU, checked against a
 // float64 product on host-dequantised weights.
 #include <cmath>
 #include <cstdio>
@@ -8,6 +8,7 @@
 #include <random>
 
 #include "../../include/wrq.hpp"
+#include "../../include/wrq_serde.hpp"
 
 using namespace wrq;
 
@@ -310,6 +311,160 @@ static void test_gpu_layer_ops() {
     EXPECT(threw);
 }
 
+
+// ---------------------------------------------------------------- on-disk form of a Matrix
+
+static std::vector<uint8_t> hex(const char *s) {
+    std::vector<uint8_t> out;
+    for (; s[0] && s[1]; s += 2) {
+        unsigned v = 0;
+        std::sscanf(s, "%2x", &v);
+        out.push_back((uint8_t)v);
+    }
+    return out;
+}
+
+// The items the format is made of, against the examples of RFC 8949, Appendix A.
+static void test_cbor_items() {
+    const std::pair<uint64_t, const char *> ints[] = {{0, "00"}, {1, "01"}, {10, "0a"}, {23, "17"}, {24, "1818"}, {25, "1819"}, {100, "1864"},
+                                                      {1000, "1903e8"}, {1000000, "1a000f4240"}, {1000000000000ull, "1b000000e8d4a51000"},
+                                                      {18446744073709551615ull, "1bffffffffffffffff"}};
+    for (const auto &kv : ints) {
+        serde::Writer w;
+        w.uint(kv.first);
+        EXPECT(w.out == hex(kv.second));
+        const auto bytes = hex(kv.second);
+        serde::Reader r(bytes.data(), bytes.size());
+        EXPECT(r.uint() == kv.first && r.remaining() == 0);
+    }
+    {
+        serde::Writer w;
+        const uint8_t b[4] = {1, 2, 3, 4};
+        w.bytes(b, 4); // h'01020304'
+        EXPECT(w.out == hex("4401020304"));
+        serde::Writer e;
+        e.bytes(b, 0); // h''
+        EXPECT(e.out == hex("40"));
+    }
+    {
+        serde::Writer w;
+        w.text("IETF");
+        EXPECT(w.out == hex("6449455446"));
+        serde::Writer e;
+        e.text("");
+        EXPECT(e.out == hex("60"));
+    }
+    {
+        serde::Writer w; // [1, 2, 3]
+        w.array(3), w.uint(1), w.uint(2), w.uint(3);
+        EXPECT(w.out == hex("83010203"));
+        serde::Writer l; // [1 .. 25]
+        l.array(25);
+        for (int i = 1; i <= 25; i++) l.uint(i);
+        EXPECT(l.out == hex("98190102030405060708090a0b0c0d0e0f101112131415161718181819"));
+    }
+    {
+        serde::Writer w; // {"a": 1, "b": [2, 3]}
+        w.map(2), w.text("a"), w.uint(1), w.text("b"), w.array(2), w.uint(2), w.uint(3);
+        EXPECT(w.out == hex("a26161016162820203"));
+        // the same value with open-ended containers: {_ "a": 1, "b": [_ 2, 3]}
+        for (const char *form : {"a26161016162820203", "bf61610161629f0203ffff"}) {
+            const auto bytes = hex(form);
+            serde::Reader r(bytes.data(), bytes.size());
+            std::vector<uint64_t> seen;
+            std::string keys;
+            r.each(5, "a map", [&](uint64_t) {
+                keys += r.text();
+                if (keys == "a") seen.push_back(r.uint());
+                else r.each(4, "an array", [&](uint64_t) { seen.push_back(r.uint()); });
+            });
+            EXPECT(keys == "ab" && seen == (std::vector<uint64_t>{1, 2, 3}) && r.remaining() == 0);
+        }
+    }
+}
+
+static void test_matrix_blob() {
+    using serde::MatrixBlob;
+    using serde::TensorBlob;
+    // one tensor, written out by hand from the rules: map(2) "shape" [2, 300, 1, 1] "data" h'0a0b'
+    {
+        serde::Writer w;
+        serde::write(w, TensorBlob{Shape(2, 300, 1, 1), {0x0a, 0x0b}});
+        EXPECT(w.out == hex("a2" "657368617065" "84" "02" "19012c" "01" "01" "6464617461" "42" "0a0b"));
+    }
+    std::mt19937 rng(3);
+    auto blob = [&](Shape s, size_t elem) {
+        TensorBlob t{s, std::vector<uint8_t>(s.len() * elem)};
+        for (auto &b : t.data) b = (uint8_t)rng();
+        return t;
+    };
+    MatrixBlob i8{Matrix::Kind::Int8, blob(Shape(128, 2, 1, 1), 1), blob(Shape(4, 1, 1, 1), 2), {}};
+    MatrixBlob f4{Matrix::Kind::Fp4, blob(Shape(64, 2, 1, 1), 1), blob(Shape(4, 1, 1, 1), 2), blob(Shape(16, 1, 1, 1), 4)};
+    MatrixBlob h{Matrix::Kind::Fp16, blob(Shape(8, 3, 1, 1), 2), {}, {}};
+    for (const MatrixBlob *mb : {&i8, &f4, &h}) {
+        const auto bytes = serde::to_vec(*mb);
+        EXPECT(serde::from_slice(bytes.data(), bytes.size()) == *mb);
+    }
+    // the head of an Int8 matrix: {"Int8": {"w": {"shape": [128, 2, 1, 1], "data": h'(256 bytes)...
+    const auto bytes = serde::to_vec(i8);
+    const auto head = hex("a1" "64496e7438" "a2" "6177" "a2" "657368617065" "84" "1880" "02" "01" "01" "6464617461" "590100");
+    EXPECT(bytes.size() > head.size() && std::equal(head.begin(), head.end(), bytes.begin()));
+    EXPECT(bytes.size() == head.size() + 256 + hex("616d" "a2" "657368617065" "84" "04" "01" "01" "01" "6464617461" "48").size() + 8);
+    // `Nf4` is read as `Fp4` (src/tensor/matrix.rs:88)
+    auto alias = serde::to_vec(f4);
+    EXPECT(alias[1] == 0x63 && alias[2] == 'F' && alias[3] == 'p' && alias[4] == '4');
+    alias[2] = 'N', alias[3] = 'f';
+    EXPECT(serde::from_slice(alias.data(), alias.size()) == f4);
+    // what must be refused: a cut file, another variant, scales that do not fit the weights, trailing bytes
+    auto refused = [](const std::vector<uint8_t> &b) {
+        try {
+            serde::from_slice(b.data(), b.size());
+        } catch (const serde::Error &) {
+            return true;
+        }
+        return false;
+    };
+    EXPECT(refused(std::vector<uint8_t>(bytes.begin(), bytes.end() - 1)));
+    EXPECT(refused(std::vector<uint8_t>(bytes.begin(), bytes.begin() + 40)));
+    auto other = bytes;
+    other[2] = 'J';
+    EXPECT(refused(other));
+    MatrixBlob wrong = i8;
+    wrong.m = blob(Shape(6, 1, 1, 1), 2);
+    EXPECT(refused(serde::to_vec(wrong)));
+    auto longer = bytes;
+    longer.push_back(0);
+    EXPECT(refused(longer));
+    EXPECT(!refused(bytes));
+}
+
+// A packed matrix written to its on-disk form and read back gives the same bytes and the same product.
+static void test_gpu_matrix_round_trip() {
+    check(wrq_init());
+    const uint32_t C = 256, R = 384;
+    std::mt19937 rng(5);
+    std::normal_distribution<float> nw(0.0f, 0.02f), nx(0.0f, 1.0f);
+    std::vector<f16> wh((size_t)C * R), xh(C);
+    for (auto &e : wh) e.bits = to_h(nw(rng));
+    for (auto &e : xh) e.bits = to_h(nx(rng));
+    Queue queue;
+    auto src = TensorGpu<f16>::from_data(Shape(C, R, 1, 1), wh);
+    auto x = TensorGpu<f16>::from_data(Shape(C, 1, 1, 1), xh);
+    const Matrix mats[3] = {Matrix::quant_u8(src, queue), Matrix::quant_nf4(src, queue), Matrix::fp16(src)};
+    queue.sync();
+    for (const Matrix &mx : mats) {
+        const auto bytes = serde::to_vec(mx);
+        const Matrix back = serde::matrix_from_slice(bytes.data(), bytes.size());
+        EXPECT(back.kind == mx.kind);
+        EXPECT(serde::to_blob(back) == serde::to_blob(mx));
+        auto o0 = TensorGpu<float>::init(Shape(R, 1, 1, 1)), o1 = TensorGpu<float>::init(Shape(R, 1, 1, 1));
+        queue.submit(mx.matmul_op(TensorGpuView<f16>(x), TensorGpuView<float>(o0), Activation::None, false));
+        queue.submit(back.matmul_op(TensorGpuView<f16>(x), TensorGpuView<float>(o1), Activation::None, false));
+        queue.sync();
+        EXPECT(o0.back() == o1.back());
+    }
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     test_run_iter();
@@ -317,11 +472,14 @@ int main(int argc, char **argv) {
     test_redirect();
     test_schedule_of_the_configs();
     test_build_time_errors();
+    test_cbor_items();
+    test_matrix_blob();
     if (!cpu_only) {
         try {
             test_gpu_layer();
             test_gpu_head();
             test_gpu_layer_ops();
+            test_gpu_matrix_round_trip();
         } catch (const TensorError &e) {
             std::printf("FAIL: TensorError %d: %s\n", e.status, e.what());
             failures++;
