@@ -5,10 +5,12 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <fstream>
 #include <random>
 
 #include "../../include/wrq.hpp"
 #include "../../include/wrq_serde.hpp"
+#include "../../include/wrq_loader.hpp"
 
 using namespace wrq;
 
@@ -465,8 +467,119 @@ static void test_gpu_matrix_round_trip() {
     }
 }
 
+// ------------------------------------------------------------------------- the loader
+
+static std::vector<uint8_t> file_bytes(const std::string &path) {
+    std::ifstream f(path, std::ios::binary);
+    return std::vector<uint8_t>(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+}
+
+// every f16 value survives the trip through f32, and the rounding of f32 -> f16 at its critical points
+static void test_f16_conversions() {
+    int bad = 0;
+    for (uint32_t b = 0; b < 65536; b++) {
+        f16 h;
+        h.bits = (uint16_t)b;
+        const bool nan = (b & 0x7c00) == 0x7c00 && (b & 0x3ff);
+        const f16 r = f16_from_f32(f16_to_f32(h));
+        bad += nan ? ((r.bits & 0x7c00) != 0x7c00 || !(r.bits & 0x3ff)) : r.bits != h.bits;
+    }
+    EXPECT(bad == 0);
+    EXPECT(f16_to_f32(f16{0x3c00}) == 1.0f && f16_to_f32(f16{0x0001}) == 5.9604644775390625e-8f && f16_to_f32(f16{0xfbff}) == -65504.0f);
+    EXPECT(f16_from_f32(1.0f + 0x1p-11f).bits == 0x3c00);          // tie: to even (down)
+    EXPECT(f16_from_f32(1.0f + 0x1p-10f + 0x1p-11f).bits == 0x3c02); // tie: to even (up)
+    EXPECT(f16_from_f32(1.0f + 0x1p-11f + 0x1p-20f).bits == 0x3c01); // above the tie
+    EXPECT(f16_from_f32(65519.0f).bits == 0x7bff && f16_from_f32(65520.0f).bits == 0x7c00);
+    EXPECT(f16_from_f32(0x1p-25f).bits == 0x0000 && f16_from_f32(0x1.000002p-25f).bits == 0x0001); // smallest subnormal's tie
+    EXPECT(f16_from_f32(0x1.8p-24f).bits == 0x0002 && f16_from_f32(-0x1p-14f).bits == 0x8400);
+    EXPECT(f16_from_f32(0x1.ffcp-15f).bits == 0x0400); // largest subnormal's upper neighbour rounds into the normal range
+}
+
+// argv: the model file and the folder of what a numpy reading of the same file expects
+static void test_loader_host(const std::string &model_path, const std::string &dir) {
+    SafeTensors model(model_path);
+    Queue queue; // holds a stream handle only; the host-side functions never launch
+    Loader loader(model, queue);
+    EXPECT(model.contains("blocks.6.att.output.weight") && model.contains("blocks.6.ffn.value.weight") && model.contains("blocks.6.att.time_first"));
+    EXPECT(!model.contains("blocks.7.att.output.weight") && model.names().size() == 3);
+    EXPECT(model.shape("blocks.6.ffn.value.weight") == (std::vector<uint64_t>{256, 384}));
+    EXPECT(loader.tensor_shape("blocks.6.ffn.value.weight") == Shape(384, 256, 1, 1)); // [out, in] -> x = in
+    EXPECT(loader.tensor_shape("blocks.6.att.time_first") == Shape(64, 4, 1, 1));
+    EXPECT(model.metadata().count("note") && model.metadata().at("note") == "a \"quoted\" word");
+    for (const char *name : {"blocks.6.att.output.weight", "blocks.6.ffn.value.weight"}) {
+        const auto got = loader.discounted(name, 0.5f);
+        const auto want = file_bytes(dir + "/" + name + ".half.f16");
+        EXPECT(want.size() == got.size() * 2 && std::memcmp(want.data(), got.data(), want.size()) == 0);
+        const auto got3 = loader.discounted(name, 0.3f);
+        const auto want3 = file_bytes(dir + "/" + name + ".x03.f16");
+        EXPECT(want3.size() == got3.size() * 2 && std::memcmp(want3.data(), got3.data(), want3.size()) == 0);
+    }
+    bool threw = false;
+    try {
+        loader.discounted("blocks.6.att.time_first", 1.0f); // an f32 tensor
+    } catch (const TensorError &e) {
+        threw = e.status == WRQ_ERR_TYPE;
+    }
+    EXPECT(threw);
+    threw = false;
+    try {
+        model.tensor("blocks.0.nothing");
+    } catch (const LoaderError &) {
+        threw = true;
+    }
+    EXPECT(threw);
+    threw = false;
+    try {
+        SafeTensors cut(dir + "/cut.st"); // the same file without its last bytes
+    } catch (const LoaderError &) {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
+// file -> discount -> pack on the device, against the packed bytes the CPU restatement gives for numpy's discount
+static void test_loader_gpu(const std::string &model_path, const std::string &dir) {
+    check(wrq_init());
+    SafeTensors model(model_path);
+    Queue queue;
+    Loader loader(model, queue);
+    const std::string name = "blocks.6.ffn.value.weight";
+    struct Case {
+        Quant quant;
+        const char *tag;
+    };
+    for (const Case &c : {Case{Quant::Int8, "int8"}, Case{Quant::NF4, "nf4"}}) {
+        const Matrix mx = loader.load_matrix_discount(name, c.quant, 0.5f);
+        queue.sync();
+        const serde::MatrixBlob blob = serde::to_blob(mx);
+        EXPECT(blob.w.data == file_bytes(dir + "/" + name + "." + c.tag + ".w"));
+        EXPECT(blob.m.data == file_bytes(dir + "/" + name + "." + c.tag + ".m"));
+        EXPECT(blob.w.shape == (c.quant == Quant::Int8 ? Shape(384, 256, 1, 1) : Shape(192, 256, 1, 1)));
+    }
+    const Matrix plain = loader.load_matrix(name, Quant::None);
+    const auto bytes = model.tensor(name);
+    const auto back = plain.h.back();
+    EXPECT(plain.kind == Matrix::Kind::Fp16 && back.size() * 2 == bytes.second && std::memcmp(back.data(), bytes.first, bytes.second) == 0);
+    const Matrix sf4 = loader.load_matrix(name, Quant::SF4);
+    queue.sync();
+    EXPECT(sf4.kind == Matrix::Kind::Fp4 && sf4.q.back() == float4_quant_student(5.0));
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
+    if (argc > 3 && (std::string(argv[1]) == "--loader" || std::string(argv[1]) == "--loader-gpu")) {
+        // the loader against a model file and its expectations, both written by tests/test_loader.py
+        try {
+            test_f16_conversions();
+            test_loader_host(argv[2], argv[3]);
+            if (std::string(argv[1]) == "--loader-gpu") test_loader_gpu(argv[2], argv[3]);
+        } catch (const std::exception &e) {
+            std::printf("FAIL: %s\n", e.what());
+            failures++;
+        }
+        std::printf(failures ? "%d FAILED\n" : "host tests ok%.0d\n", failures);
+        return failures ? 1 : 0;
+    }
     test_run_iter();
     test_advance();
     test_redirect();
