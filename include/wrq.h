@@ -292,6 +292,34 @@ int wrq_time_mix_v6(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
                     const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype);
 
 /*
+ * The ops an RWKV-v7 layer adds (src/runtime/v7.rs:757-1006).
+ * TensorOp::l2_norm(x, eps)                 src/tensor/ops.rs:642-700, src/shaders/normalize.wgsl:118-152
+ *   x [C, T, B, 1] <- x / sqrt(sum of squares over the row + eps).
+ * TensorOp::control_k_v7(p, a, k)           src/tensor/ops.rs:1800-1858, src/shaders/control_k_v7.wgsl
+ *   k [C, T, B, 1] <- k (1 + (a - 1) p); p f16 [C, 1, 1, 1]; a, k views of f16 or f32 tensors.
+ * TensorOp::time_mix_v7(cursors, state, r, w, n, x)
+ *                                           src/tensor/ops.rs:1679-1741, src/shaders/time_mix_v7.wgsl:137-212
+ *   x, r, w [S, H, A, 1]; n [S, H, A, 4] holds k, v, a, kk; state [S H, S + 1, B, 1] as for time_mix_v6.
+ *   With a' = -kk, b = kk a, w' = exp(-exp(-0.5) sigmoid(w)):  sa[i] = sum_j S[j][i] a'[j],
+ *   S[j][i] <- S[j][i] w'[j] + k[j] v[i] + sa[i] b[j],  x[i] <- sum_j r[j] S[j][i].  Head sizes 32, 64, 128.
+ * TensorOp::time_first_v7(u, r, n, x)       src/tensor/ops.rs:1743-1798, src/shaders/time_mix_v7.wgsl:214-255
+ *   x[i] <- x[i] + (sum_j u[j] k[j] r[j]) v[i] per head and token; u f16 [S, H, 1, 1].
+ * TensorOp::channel_mix_v7(cursors, state, v, x)
+ *                                           src/tensor/ops.rs:1917-1970, src/shaders/channel_mix.wgsl (V7)
+ *   state [C, 1, B, 1] <- x at every request's last token; x [C, A, 1, 1] <- v.
+ */
+int wrq_l2_norm(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype, float eps);
+int wrq_control_k_v7(wrq_stream stream, const wrq_tensor *p, const wrq_tensor_view *a,
+                     const wrq_tensor_view *k);
+int wrq_time_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state,
+                    const wrq_tensor *r, const wrq_tensor *w, const wrq_tensor *n, const wrq_tensor *x,
+                    wrq_dtype dtype);
+int wrq_time_first_v7(wrq_stream stream, const wrq_tensor *u, const wrq_tensor *r, const wrq_tensor *n,
+                      const wrq_tensor *x, wrq_dtype dtype);
+int wrq_channel_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state,
+                       const wrq_tensor *v, const wrq_tensor *x, wrq_dtype dtype);
+
+/*
  * Fused forms of consecutive small ops of an RWKV-v6 layer (src/runtime/v6.rs:758-955).  They have no
  * counterpart among the reference's constructors; they are for callers that run a layer without hooks
  * between its ops: at batch 1 every op costs its launch, and these bring a layer from 35 launches to 12.

@@ -7,6 +7,7 @@ Each function follows its shader lane by lane: a workgroup of BLOCK_SIZE threads
   softmax                 src/shaders/softmax.wgsl:52-110           (BLOCK_SIZE 128, ops.rs:301)
   layer_norm, group_norm  src/shaders/layer_norm.wgsl:27-120        (128 / 32, ops.rs:415, :468)
   add / mul + activations src/shaders/binary.wgsl:36-77, activations src/tensor/ops.rs:205-233
+  token_shift, channel_mix(_v7), time_mix_v5 / v6 / v7, time_first_v7, l2_norm, control_k_v7: cited at each function
 What pins them: the closed forms of the reference's own tests (softmax ops.rs:2655-2662, layer
 norm ops.rs:2726-2746: sequential Welford) and float64 textbook forms, in tests/test_layer_ops.py.
 Parity unpinned: group_norm's tree starts at a stride (64) beyond its 32 threads; the reads past
@@ -264,3 +265,83 @@ def time_mix_v5(cursors, time_decay, time_first, state, k, v, r, x):
             state[slot, 1 + j] = _fma(np.broadcast_to(w32[:, j:j + 1], (H, S)), ss, kv).reshape(-1)
         out[t] = y
     return out.astype(x.dtype)
+
+
+def l2_norm(x, eps, block=128):
+    """src/shaders/normalize.wgsl:118-152: rows of the last axis; squares summed per lane vector over the
+    row's stride, then the shader's tree over the threads; x / sqrt(sum + eps)."""
+    rows, shape, dtype = _rows(x)
+    out = np.empty_like(rows)
+    for i, row in enumerate(rows):
+        vec, valid = _lanes(row, block)
+        acc = np.zeros((block, 4), dtype=F)
+        for it in range(vec.shape[0]):
+            acc = np.where(valid[it][:, None], acc + vec[it] * vec[it], acc)
+        step = block >> 1
+        while step:
+            acc[:step] = acc[:step] + acc[step:2 * step]
+            step >>= 1
+        total = F(F(acc[0, 0] + acc[0, 1]) + acc[0, 2]) + acc[0, 3]
+        out[i] = row * (F(1) / np.sqrt(F(total + F(eps)), dtype=F))
+    return out.reshape(shape).astype(dtype)
+
+
+def control_k_v7(p, a, k):
+    """src/shaders/control_k_v7.wgsl:64-79: k (1 + (a - 1) p), p (C,) broadcast over tokens."""
+    k = np.asarray(k)
+    p32, a32, k32 = np.asarray(p).astype(F), np.asarray(a).astype(F), k.astype(F)
+    return (k32 * (F(1) + (a32 - F(1)) * p32)).astype(k.dtype)
+
+
+def time_mix_v7(cursors, state, r, w, n, x):
+    """src/shaders/time_mix_v7.wgsl:137-212.  r, w, x (A, H, S); n (4, A, H, S) = k, v, a, kk; state
+    (B, S + 1, H * S) f32 updated in place (row 0: x at a request's last token; row 1 + j: S[j][.]);
+    both sums over j in the shader's order.  Returns the new x."""
+    x = np.asarray(x)
+    A, H, S = x.shape
+    r32, w32, n32 = (np.asarray(t).astype(F) for t in (r, w, n))
+    k32, v32, a32, kk32 = n32
+    out = np.empty((A, H, S), dtype=F)
+    for t in range(A):
+        slot, first, cnt = _cursor(cursors[t])
+        if t - first + 1 == cnt:
+            state[slot, 0] = x[first + cnt - 1].astype(F).reshape(-1)
+        ww = np.exp(F(-0.606531) * (F(1) / (F(1) + np.exp(-w32[t], dtype=F))), dtype=F)
+        aa, bb = -kk32[t], kk32[t] * a32[t]
+        sa = np.zeros((H, S), dtype=F)
+        for j in range(S):
+            sa = sa + state[slot, 1 + j].reshape(H, S) * aa[:, j:j + 1]
+        y = np.zeros((H, S), dtype=F)
+        for j in range(S):
+            ss = state[slot, 1 + j].reshape(H, S)
+            ss = ss * ww[:, j:j + 1] + k32[t, :, j:j + 1] * v32[t] + sa * bb[:, j:j + 1]
+            y = y + r32[t, :, j:j + 1] * ss
+            state[slot, 1 + j] = ss.reshape(-1)
+        out[t] = y
+    return out.astype(x.dtype)
+
+
+def time_first_v7(u, r, n, x):
+    """src/shaders/time_mix_v7.wgsl:214-255: x + (sum_j u[j] k[j] r[j]) v per head and token; the sum
+    runs over 4-lane vectors with the shader's tree, then over the four lanes."""
+    x = np.asarray(x)
+    A, H, S = x.shape
+    n32 = np.asarray(n).astype(F)
+    prod = np.asarray(u).astype(F)[None] * n32[0] * np.asarray(r).astype(F)  # (A, H, S)
+    vec = prod.reshape(A, H, S // 4, 4).copy()
+    step = (S // 4) >> 1
+    while step:
+        vec[:, :, :step] = vec[:, :, :step] + vec[:, :, step:2 * step]
+        step >>= 1
+    xx = (vec[:, :, 0, 0] + vec[:, :, 0, 1]) + vec[:, :, 0, 2] + vec[:, :, 0, 3]
+    return (x.astype(F) + xx[..., None] * n32[1]).astype(x.dtype)
+
+
+def channel_mix_v7(cursors, state_row, v, x):
+    """src/shaders/channel_mix.wgsl:83-106 with V7: state_row (B, C) f32 updated in place; returns v as the new x."""
+    x = np.asarray(x)
+    for a in range(x.shape[0]):
+        slot, first, cnt = _cursor(cursors[a])
+        if a - first + 1 == cnt:
+            state_row[slot] = x[a].astype(F)
+    return np.asarray(v).astype(x.dtype)

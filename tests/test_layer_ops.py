@@ -379,6 +379,194 @@ def test_gpu_time_mix_v5(gpu, lop, dtype, H, S, runs):
 
 
 # ---------------------------------------------------------------------------------------------
+# the ops an RWKV-v7 layer adds.  The reference has no test of them: the restatements are pinned by
+# float64 textbook forms, closed forms of special cases and invariants only (parity unpinned).
+def wkv7_float64(cursors, state, r, w, n, x):
+    """per request and head in float64, matrices indexed [j, i]:  sa = S^T a,  S <- diag(w) S + k v^T + b sa^T,  y = S^T r
+    with a = -kk, b = kk * a_in, w = exp(-exp(-1/2) sigmoid(w_in))"""
+    A, H, S = x.shape
+    f = np.float64
+    st = state.astype(f).copy()
+    out = np.zeros((A, H, S))
+    k, v, a_in, kk = (t.astype(f) for t in n)
+    for t in range(A):
+        c = int(cursors[t])
+        slot, first, cnt = c & 0xff, (c >> 8) & 0xffff, (c >> 24) & 0xff
+        if t - first + 1 == cnt:
+            st[slot, 0] = x[t].astype(f).reshape(-1)
+        for h in range(H):
+            Sm = st[slot, 1:, h * S:(h + 1) * S]
+            ww = np.exp(-np.exp(-0.5) / (1.0 + np.exp(-w[t, h].astype(f))))
+            sa = Sm.T @ (-kk[t, h])
+            Sn = ww[:, None] * Sm + np.outer(k[t, h], v[t, h]) + np.outer(kk[t, h] * a_in[t, h], sa)
+            out[t, h] = Sn.T @ r[t, h].astype(f)
+            st[slot, 1:, h * S:(h + 1) * S] = Sn
+    return out, st
+
+
+def wkv7_inputs(rng, A, H, S, B, dtype):
+    r = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    w = rng.standard_normal((A, H, S)).astype(dtype)
+    k = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    v = (0.5 * rng.standard_normal((A, H, S))).astype(dtype)
+    a = rng.random((A, H, S)).astype(dtype)  # a sigmoid's output
+    kk = rng.standard_normal((A, H, S))
+    kk = (kk / np.sqrt((kk * kk).sum(axis=-1, keepdims=True))).astype(dtype)  # rows of unit length, as after l2_norm
+    x = rng.standard_normal((A, H, S)).astype(dtype)
+    state = (0.1 * rng.standard_normal((B, S + 1, H * S))).astype(np.float32)
+    return r, w, np.stack([k, v, a, kk]), x, state
+
+
+def test_oracle_v7_ops(lop):
+    rng = np.random.default_rng(SEED + 9)
+    H, S, B = 3, 16, 6
+    cur = lop.pack_cursors(RUNS)
+    A = len(cur)
+    r, w, n, x, state = wkv7_inputs(rng, A, H, S, B, np.float32)
+    st = state.copy()
+    got = lop.time_mix_v7(cur, st, r, w, n, x)
+    want, want_state = wkv7_float64(cur, state, r, w, n, x)
+    assert_close(got, want, 1e-5, "y vs float64")
+    assert_close(st, want_state, 1e-5, "state vs float64")
+    assert np.array_equal(st[[1, 3, 4]], state[[1, 3, 4]])
+    # one token from a zero state: S = k v^T, so y = (r . k) v whatever a and kk are
+    z = np.zeros_like(state)
+    y1 = lop.time_mix_v7(lop.pack_cursors([(1, 1)]), z, r[:1], w[:1], n[:, :1], x[:1])
+    assert_close(y1[0], (r[0] * n[0, 0]).sum(axis=-1, keepdims=True).astype(np.float64) * n[1, 0], 1e-5, "first token")
+    # kk = 0 switches the correction off: tokens of one request from a zero state give
+    # y_t = sum_{s <= t} (r_t . (prod_{s < q <= t} w_q) k_s) v_s
+    n0 = n.copy()
+    n0[3] = 0
+    z = np.zeros_like(state)
+    y = lop.time_mix_v7(lop.pack_cursors([(2, 4)]), z, r[:4], w[:4], n0[:, :4], x[:4])
+    wd = np.exp(-np.exp(-0.5) / (1.0 + np.exp(-w[:4].astype(np.float64))))
+    for t in range(4):
+        closed = np.zeros((H, S))
+        for s_ in range(t + 1):
+            decay = np.prod(wd[s_ + 1:t + 1], axis=0) if s_ < t else np.ones((H, S))
+            closed += (r[t] * decay * n[0, s_]).sum(axis=-1, keepdims=True) * n[1, s_]
+        assert_close(y[t], closed, 1e-5, f"decay-only closed form, token {t}")
+    # a run of 2 tokens equals two runs of 1 token
+    s_a, s_b = state.copy(), state.copy()
+    two = lop.time_mix_v7(lop.pack_cursors([(4, 2)]), s_a, r[:2], w[:2], n[:, :2], x[:2])
+    first = lop.time_mix_v7(lop.pack_cursors([(4, 1)]), s_b, r[:1], w[:1], n[:, :1], x[:1])
+    second = lop.time_mix_v7(lop.pack_cursors([(4, 1)]), s_b, r[1:2], w[1:2], n[:, 1:2], x[1:2])
+    assert np.array_equal(two, np.concatenate([first, second])) and np.array_equal(s_a, s_b)
+
+    u = (0.3 * rng.standard_normal((H, S))).astype(np.float16)
+    got = lop.time_first_v7(u, r, n, x)
+    f = np.float64
+    want = x.astype(f) + (u.astype(f) * n[0].astype(f) * r.astype(f)).sum(axis=-1, keepdims=True) * n[1].astype(f)
+    assert_close(got, want, 1e-5, "time_first_v7 vs float64")
+
+    rows = rng.standard_normal((5, 7, 64)).astype(np.float32)
+    got = lop.l2_norm(rows, 1e-12)
+    assert_close(got, rows / np.sqrt((rows.astype(f) ** 2).sum(axis=-1, keepdims=True)), 1e-6, "l2_norm vs float64")
+    assert_close((got.astype(f) ** 2).sum(axis=-1), np.ones((5, 7)), 1e-6, "unit length")
+    assert np.array_equal(lop.l2_norm(np.zeros((1, 8), dtype=np.float32), 1e-12), np.zeros((1, 8), dtype=np.float32))  # eps keeps 0 / 0 away
+
+    p = rng.random(64).astype(np.float16)
+    a, k = rng.random((3, 64)).astype(np.float32), rng.standard_normal((3, 64)).astype(np.float32)
+    assert_close(lop.control_k_v7(p, a, k), k.astype(f) * (1 + (a.astype(f) - 1) * p.astype(f)), 1e-6, "control_k_v7 vs float64")
+    assert np.array_equal(lop.control_k_v7(np.zeros(64, dtype=np.float16), a, k), k)  # p = 0: k unchanged
+    assert_close(lop.control_k_v7(np.ones(64, dtype=np.float16), a, k), k * a, 1e-6, "p = 1: k a")
+
+    cm_state = rng.standard_normal((B, 64)).astype(np.float32)
+    keep = cm_state.copy()
+    xs, vs_ = rng.standard_normal((A, 64)).astype(np.float16), rng.standard_normal((A, 64)).astype(np.float16)
+    out = lop.channel_mix_v7(cur, cm_state, vs_, xs)
+    assert np.array_equal(out, vs_)
+    first = 0
+    for slot, cnt in RUNS:
+        assert np.array_equal(cm_state[slot], xs[first + cnt - 1].astype(np.float32))
+        first += cnt
+    assert np.array_equal(cm_state[[1, 3, 4]], keep[[1, 3, 4]])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("H,S,runs", [(3, 32, RUNS), (4, 64, RUNS), (64, 64, [(0, 1)]), (2, 128, [(1, 2), (3, 2)]), (2, 64, [(4, 100)])])
+def test_gpu_time_mix_v7(gpu, lop, dtype, H, S, runs):
+    import torch
+
+    print("time mix v7 on the GPU", dtype.__name__, H, S, runs[:3], flush=True)
+    rng = np.random.default_rng(SEED + 90 + H + S)
+    B = 6
+    cur = lop.pack_cursors(runs)
+    A = len(cur)
+    r, w, n, x, state = wkv7_inputs(rng, A, H, S, B, dtype)
+    full = np.concatenate([np.zeros_like(state), state], axis=1)
+    sview = ((H * S, S + 1, B), (H * S, 2 * (S + 1), B), (0, S + 1, 0))
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    sd, xd, rd, nd = dev(full), dev(x), dev(r), dev(n)
+    gpu.LayerOp.time_mix_v7(dev(cur.view(np.int32)), sd, rd, dev(w), nd, xd, state_view=sview)
+    want, want_state = wkv7_float64(cur, state, r, w, n, x)
+    eps = 2e-3 if dtype == np.float16 else 5e-5
+    assert_close(xd.cpu().numpy(), want, eps, "y vs float64")
+    got_state = sd.cpu().numpy()
+    assert_close(got_state[:, S + 1:], want_state, 5e-5, "state vs float64")
+    assert np.array_equal(got_state[:, :S + 1], full[:, :S + 1])  # the other layer's rows are untouched
+    if A * H * S * S <= 2000000:
+        st = state.copy()
+        assert_close(xd.cpu().numpy(), lop.time_mix_v7(cur, st, r, w, n, x), eps, "y vs oracle")
+        assert_close(got_state[:, S + 1:], st, 5e-5, "state vs oracle")
+    # time_first_v7 on top of the result
+    u = (0.3 * rng.standard_normal((H, S))).astype(np.float16)
+    y = xd.cpu().numpy()
+    gpu.LayerOp.time_first_v7(dev(u), rd, nd, xd)
+    assert_close(xd.cpu().numpy(), lop.time_first_v7(u, r, n, y), eps, "time_first_v7 vs oracle")
+    f = np.float64
+    assert_close(xd.cpu().numpy(), y.astype(f) + (u.astype(f) * n[0].astype(f) * r.astype(f)).sum(axis=-1, keepdims=True) * n[1].astype(f), eps, "time_first_v7 vs float64")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_gpu_v7_small_ops(gpu, lop, dtype):
+    import torch
+
+    print("l2 norm / control k / channel mix v7 on the GPU", dtype.__name__, flush=True)
+    rng = np.random.default_rng(SEED + 95)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    eps = 2e-3 if dtype == np.float16 else 1e-6
+    f = np.float64
+    for shape in ((9, 12, 64), (3, 1, 1000), (1, 2, 2048)):
+        rows = rng.standard_normal(shape).astype(dtype)
+        xd = dev(rows)
+        gpu.LayerOp.l2_norm(xd, 1e-12)
+        assert_close(xd.cpu().numpy(), lop.l2_norm(rows, 1e-12), eps, f"l2_norm vs oracle {shape}")
+        assert_close(xd.cpu().numpy(), rows.astype(f) / np.sqrt((rows.astype(f) ** 2).sum(axis=-1, keepdims=True)), eps, f"l2_norm vs float64 {shape}")
+    C, A, B = 256, 8, 6
+    p = rng.random(C).astype(np.float16)
+    for adt in (np.float16, np.float32):
+        a, k = rng.random((1, A, C)).astype(adt), rng.standard_normal((1, A, C)).astype(dtype)
+        kd = dev(k)
+        gpu.LayerOp.control_k_v7(dev(p), dev(a), kd)
+        assert_close(kd.cpu().numpy(), lop.control_k_v7(p, a, k), eps, "control_k_v7 vs oracle")
+    # k as one slice of a larger tensor
+    big = rng.standard_normal((3, A, C)).astype(dtype)
+    a = rng.random((1, A, C)).astype(dtype)
+    bd = dev(big)
+    gpu.LayerOp.control_k_v7(dev(p), dev(a), bd, k_view=((C, A, 1), (C, A, 3), (0, 0, 2)))
+    want = big.copy()
+    want[2] = lop.control_k_v7(p, a[0], big[2])
+    assert_close(bd.cpu().numpy(), want, eps, "control_k_v7 on a slice")
+    assert np.array_equal(bd.cpu().numpy()[:2], big[:2])
+    cur = lop.pack_cursors(RUNS)
+    A = len(cur)
+    rows_, row = 4, 3
+    state = rng.standard_normal((B, rows_, C)).astype(np.float32)
+    sview = ((C, 1, B), (C, rows_, B), (0, row, 0))
+    x, v = rng.standard_normal((A, C)).astype(dtype), rng.standard_normal((A, C)).astype(dtype)
+    sd, xd = dev(state), dev(x.reshape(1, A, C))
+    gpu.LayerOp.channel_mix_v7(dev(cur.view(np.int32)), sd, dev(v.reshape(1, A, C)), xd, state_view=sview)
+    st = state[:, row].copy()
+    assert np.array_equal(xd.cpu().numpy()[0], lop.channel_mix_v7(cur, st, v, x))
+    want_state = state.copy()
+    want_state[:, row] = st
+    assert np.array_equal(sd.cpu().numpy(), want_state)
+
+
+# ---------------------------------------------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_data_movement_kats(gpu):
     import torch

@@ -44,6 +44,7 @@ EXPORTS = [
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
     "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v5", "wrq_time_mix_v6", "wrq_embed",
+    "wrq_l2_norm", "wrq_control_k_v7", "wrq_time_mix_v7", "wrq_time_first_v7", "wrq_channel_mix_v7",
     "wrq_v6_pre", "wrq_v6_time_mix", "wrq_v6_decay", "wrq_v6_wkv_gate", "wrq_v6_post_ffn",
 ]
 MAX_GROUP = 8
@@ -199,6 +200,11 @@ def lib():
         L.wrq_channel_mix.argtypes = [vp, T, V, T, T, T, i]
         L.wrq_time_mix_v5.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         L.wrq_time_mix_v6.argtypes = [vp, T, T, T, V, T, T, T, T, i]
+        L.wrq_l2_norm.argtypes = [vp, T, i, C.c_float]
+        L.wrq_control_k_v7.argtypes = [vp, T, V, V]
+        L.wrq_time_mix_v7.argtypes = [vp, T, V, T, T, T, T, i]
+        L.wrq_time_first_v7.argtypes = [vp, T, T, T, T, i]
+        L.wrq_channel_mix_v7.argtypes = [vp, T, V, T, T, i]
         L.wrq_embed.argtypes = [vp, T, T, T, i]
         u = C.c_uint32
         L.wrq_v6_pre.argtypes = [vp, u, u, vp, vp, vp, vp, vp, vp, C.c_float, V, i, vp, vp, vp, vp, vp]
@@ -370,6 +376,28 @@ class LayerOp:
         _check(lib().wrq_time_mix_v6(_stream(), C.byref(as_tensor(cursors)), C.byref(as_tensor(time_decay)), C.byref(as_tensor(time_first)),
                                      C.byref(as_view(state, state_view)), C.byref(as_tensor(k)), C.byref(as_tensor(v)), C.byref(as_tensor(r)),
                                      C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def l2_norm(x, eps):
+        _check(lib().wrq_l2_norm(_stream(), C.byref(as_tensor(x)), _dtype(x), eps))
+
+    @staticmethod
+    def control_k_v7(p, a, k, a_view=None, k_view=None):
+        _check(lib().wrq_control_k_v7(_stream(), C.byref(as_tensor(p)), C.byref(as_view(a, a_view)), C.byref(as_view(k, k_view))))
+
+    @staticmethod
+    def time_mix_v7(cursors, state, r, w, n, x, state_view=None):
+        _check(lib().wrq_time_mix_v7(_stream(), C.byref(as_tensor(cursors)), C.byref(as_view(state, state_view)), C.byref(as_tensor(r)),
+                                     C.byref(as_tensor(w)), C.byref(as_tensor(n)), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def time_first_v7(u, r, n, x):
+        _check(lib().wrq_time_first_v7(_stream(), C.byref(as_tensor(u)), C.byref(as_tensor(r)), C.byref(as_tensor(n)), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def channel_mix_v7(cursors, state, v, x, state_view=None):
+        _check(lib().wrq_channel_mix_v7(_stream(), C.byref(as_tensor(cursors)), C.byref(as_view(state, state_view)), C.byref(as_tensor(v)),
+                                        C.byref(as_tensor(x)), _dtype(x)))
 
     @staticmethod
     def lerp(input, output, factor, reversed=False, input_view=None, output_view=None, factor_view=None):
