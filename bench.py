@@ -499,6 +499,7 @@ def ops_table(wrq, torch, args, C):
     x, y, w, b, x5, tm5 = h(1, A, C), h(1, A, C), h(C), h(C), h(5, A, C), h(5, A, C)
     k, v, r, aux, decay, u = f(A, heads, S), f(A, heads, S), f(A, heads, S), f(A, heads, S), torch.rand((A, heads, S), device="cuda"), f(heads, S)
     gw, gb = h(heads, S), h(heads, S)
+    r16, w16, n16, u16 = h(A, heads, S), h(A, heads, S), 0.1 * h(4, A, heads, S), h(heads, S)  # the v7 operands are f16
     cases = {
         "layer_norm": (lambda: LayerOp.layer_norm(w, b, x, 1e-5), 2 * A * C * 2),
         "group_norm": (lambda: LayerOp.group_norm(gw, gb, aux, 64e-5), 2 * A * C * 4),
@@ -510,6 +511,12 @@ def ops_table(wrq, torch, args, C):
         "activate stable_exp": (lambda: LayerOp.activate(decay.view(1, A, C), wrq.ACT_STABLE_EXP), 2 * A * C * 4),
         "channel_mix": (lambda: LayerOp.channel_mix(cur, state, x, y, x5[0:1], state_view=ffn), 4 * A * C * 2),
         "time_mix_v6": (lambda: LayerOp.time_mix_v6(cur, decay, u, state, k, v, r, aux, state_view=att), 5 * A * C * 4 + 2 * S * C * 4),
+        "time_mix_v5": (lambda: LayerOp.time_mix_v5(cur, decay[0], u, state, k, v, r, aux, state_view=att), 4 * A * C * 4 + 2 * S * C * 4),
+        "time_mix_v7": (lambda: LayerOp.time_mix_v7(cur, state, r16, w16, n16, x.view(A, heads, S), state_view=att), 7 * A * C * 2 + 2 * S * C * 4),
+        "time_first_v7": (lambda: LayerOp.time_first_v7(u16, r16, n16, x.view(A, heads, S)), 5 * A * C * 2),
+        "l2_norm (heads)": (lambda: LayerOp.l2_norm(x.view(A, heads, S), 1e-12), 2 * A * C * 2),
+        "control_k_v7": (lambda: LayerOp.control_k_v7(w, x, y), 3 * A * C * 2),
+        "channel_mix_v7": (lambda: LayerOp.channel_mix_v7(cur, state, x, y, state_view=ffn), 2 * A * C * 2),
         "softmax (65536)": (lambda: LayerOp.softmax(f(1, 1, 65536)), 0),
     }
     for name, (fn, nbytes) in cases.items():

@@ -463,6 +463,44 @@ class TensorOp {
         });
     }
 
+    // the ops an RWKV-v7 layer adds: src/tensor/ops.rs:642-700, :1800-1858, :1679-1741, :1743-1798, :1917-1970
+    template <typename F>
+    static TensorOp l2_norm(const TensorGpu<F> &x, float eps) {
+        return checked([=](wrq_stream s) { const wrq_tensor tx = x.c(); return wrq_l2_norm(s, &tx, (wrq_dtype)dtype_of<F>::value, eps); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp control_k_v7(const TensorGpu<f16> &p, const TensorGpuView<F0> &a, const TensorGpuView<F1> &k) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor tp = p.c();
+            const wrq_tensor_view ta = a.c(), tk = k.c();
+            return wrq_control_k_v7(s, &tp, &ta, &tk);
+        });
+    }
+    template <typename F>
+    static TensorOp time_mix_v7(const TensorGpu<uint32_t> &cursors, const TensorGpuView<float> &state, const TensorGpu<F> &r, const TensorGpu<F> &w,
+                                const TensorGpu<F> &n, const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), tr = r.c(), tw = w.c(), tn = n.c(), tx = x.c();
+            const wrq_tensor_view st = state.c();
+            return wrq_time_mix_v7(s, &c, &st, &tr, &tw, &tn, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+    template <typename F>
+    static TensorOp time_first_v7(const TensorGpu<f16> &u, const TensorGpu<F> &r, const TensorGpu<F> &n, const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor tu = u.c(), tr = r.c(), tn = n.c(), tx = x.c();
+            return wrq_time_first_v7(s, &tu, &tr, &tn, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+    template <typename F>
+    static TensorOp channel_mix_v7(const TensorGpu<uint32_t> &cursors, const TensorGpuView<float> &state, const TensorGpu<F> &v, const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), tv = v.c(), tx = x.c();
+            const wrq_tensor_view st = state.c();
+            return wrq_channel_mix_v7(s, &c, &st, &tv, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+
     Kind kind() const { return kind_; }
     const std::vector<TensorOp> &list() const { return list_; }
     const Payload &payload() const { return payload_; }

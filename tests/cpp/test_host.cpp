@@ -304,6 +304,31 @@ static void test_gpu_layer_ops() {
     const std::vector<float> want = {0, 0, 0, 0, 0, 1, 2, 3, 0, 0, 0, 0, 0, 0, 0, 0, 4, 5, 6, 7, 8, 9, 10, 11};
     EXPECT(out.back() == want);
 
+    // rows of unit length after l2_norm (src/tensor/ops.rs:642-700), k (1 + (a - 1) p) after control_k_v7 (:1800-1858)
+    {
+        std::vector<float> rows(64 * 5), av(64 * 5, 0.25f);
+        for (auto &e : rows) e = ux(rng);
+        std::vector<f16> ph(64);
+        for (auto &e : ph) e.bits = to_h(0.5f);
+        auto xr = TensorGpu<float>::from_data(Shape(64, 5, 1, 1), rows);
+        auto kr = TensorGpu<float>::from_data(Shape(64, 5, 1, 1), rows);
+        auto ar = TensorGpu<float>::from_data(Shape(64, 5, 1, 1), av);
+        auto pr = TensorGpu<f16>::from_data(Shape(64, 1, 1, 1), ph);
+        queue.submit(TensorOp::l2_norm(xr, 1.0e-12f));
+        queue.submit(TensorOp::control_k_v7(pr, TensorGpuView<float>(ar), TensorGpuView<float>(kr)));
+        queue.sync();
+        const auto unit = xr.back(), kc = kr.back();
+        int off = 0;
+        for (int t = 0; t < 5; t++) {
+            double sq = 0, in = 0;
+            for (int i = 0; i < 64; i++) sq += (double)unit[t * 64 + i] * unit[t * 64 + i], in += (double)rows[t * 64 + i] * rows[t * 64 + i];
+            off += std::fabs(sq - 1.0) > 1e-5;
+            for (int i = 0; i < 64; i++) off += std::fabs(unit[t * 64 + i] - rows[t * 64 + i] / std::sqrt(in)) > 1e-6;
+            for (int i = 0; i < 64; i++) off += std::fabs(kc[t * 64 + i] - rows[t * 64 + i] * 0.625) > 1e-6 * std::max(1.0, (double)std::fabs(rows[t * 64 + i]));
+        }
+        EXPECT(off == 0);
+    }
+
     bool threw = false;
     try {
         queue.submit(TensorOp::transpose(TensorGpuView<float>(in0), TensorGpuView<float>(out)));

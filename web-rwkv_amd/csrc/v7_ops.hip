@@ -8,9 +8,10 @@
 // time_mix_v7 is, per head and token, with S[j][i] the head's state, a = -kk, b = kk * a_in and
 // w = exp(-exp(-0.5) sigmoid(w_in)):
 //   sa[i] = sum_j S[j][i] a[j];   S[j][i] <- S[j][i] w[j] + k[j] v[i] + sa[i] b[j];   y[i] = sum_j r[j] S[j][i]
-// The shader walks the state in memory twice per token; here a lane owns column i of S (one register
-// per j) for all tokens of a request in the run, and the five vectors over j of a token are passed
-// round through LDS as broadcasts.  One workgroup of S lanes per head.
+// The shader walks the state in memory twice per token; here four lanes share column i of S and hold a
+// quarter of its j range each in registers for all tokens of a request in the run (two quad reductions
+// per token, for sa and for y); the five vectors over j of a token are fetched one token ahead and
+// passed round through LDS (two buffers, one barrier per token).  One workgroup of 4 S lanes per head.
 #include "layer_device.h"
 
 namespace wrq {
@@ -44,55 +45,84 @@ __global__ __launch_bounds__(256) void control_k_kernel(const uint16_t *p, const
     store_vec4(kp, make_float4(f(kk.x, aa.x, pp.x), f(kk.y, aa.y, pp.y), f(kk.z, aa.z, pp.z), f(kk.w, aa.w, pp.w)));
 }
 
+__device__ __forceinline__ float quad_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true)); // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true)); // quad_perm [2,3,0,1]
+    return v;
+}
+
+// thread = (column i of S, quarter q of the j range): 4 SZ threads per head, JQ = SZ / 4 values of S per lane
 template <typename XT, int SZ>
-__global__ __launch_bounds__(SZ) void time_mix_v7_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *w, const XT *n, XT *x, ViewArgs vs, uint32_t H,
-                                                         uint32_t A) {
-    __shared__ float rs[SZ], ws[SZ], ks[SZ], as[SZ], bs[SZ];
-    const uint32_t head = blockIdx.x, i = threadIdx.x;
+__global__ __launch_bounds__(4 * SZ) void time_mix_v7_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *w, const XT *n, XT *x, ViewArgs vs,
+                                                             uint32_t H, uint32_t A) {
+    constexpr int JQ = SZ / 4;
+    // the vectors over j of a token and its v, two buffers: token t + 1 is written while token t may still be read
+    __shared__ __align__(16) float rs[2][SZ], ws[2][SZ], ks[2][SZ], as[2][SZ], bs[2][SZ], vsh[2][SZ];
+    const uint32_t head = blockIdx.x, tid = threadIdx.x, i = tid >> 2, q = tid & 3;
     const uint32_t C = SZ * H, chan = head * SZ + i;
     const uint64_t plane = (uint64_t)A * C; // n holds k, v, a, kk one after the other
-    float s[SZ];
+    const bool stager = tid < (uint32_t)SZ; // the first SZ threads fetch element `tid` of a token's operands, one token ahead
+    float s[JQ];
     uint32_t held = 0xffffffffu; // request whose S is in registers
+    float fr = 0, fw = 0, fk = 0, fv = 0, fa = 0, fkk = 0;
+    uint32_t fc;
+    auto fetch = [&](uint32_t t) {
+        fc = cursors[t];
+        if (stager) {
+            const uint64_t ti = (uint64_t)t * C + head * SZ + tid;
+            fr = load_one(r + ti), fw = load_one(w + ti), fk = load_one(n + ti), fv = load_one(n + plane + ti);
+            fa = load_one(n + 2 * plane + ti), fkk = load_one(n + 3 * plane + ti);
+        }
+    };
+    fetch(0);
     for (uint32_t t = 0; t < A; t++) {
-        const Cursor cur = read_cursor(cursors, t, vs);
+        const int buf = t & 1;
+        Cursor cur = unpack_cursor(fc);
+        cur.batch = min(cur.batch, vs.shape[2] - 1); // as read_cursor
+        cur.token = min(cur.token, t);
+        if (stager) {
+            rs[buf][tid] = fr;
+            ws[buf][tid] = expf(-0.606531f / (1.0f + expf(-fw))); // exp(-exp(-0.5) sigmoid(w))
+            ks[buf][tid] = fk;
+            as[buf][tid] = -fkk;
+            bs[buf][tid] = fkk * fa;
+            vsh[buf][tid] = fv;
+        }
+        __syncthreads(); // token t is in LDS; the other buffer was last read before the previous barrier
+        if (t + 1 < A) fetch(t + 1);
         if (cur.batch != held) {
             if (held != 0xffffffffu) {
 #pragma unroll
-                for (int j = 0; j < SZ; j++) state[view_elem(vs, held, j + 1, chan)] = s[j];
+                for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
             }
             held = cur.batch;
 #pragma unroll
-            for (int j = 0; j < SZ; j++) s[j] = state[view_elem(vs, held, j + 1, chan)];
+            for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
         }
         const uint64_t ti = (uint64_t)t * C + chan;
         // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
-        if (t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti);
-        const float ww = load_one(w + ti), aa = load_one(n + 2 * plane + ti), kk = load_one(n + 3 * plane + ti);
-        __syncthreads(); // the previous token's vectors have been read
-        rs[i] = load_one(r + ti);
-        ws[i] = expf(-0.606531f / (1.0f + expf(-ww))); // exp(-exp(-0.5) sigmoid(w))
-        ks[i] = load_one(n + ti);
-        as[i] = -kk;
-        bs[i] = kk * aa;
-        __syncthreads();
-        const float vv = load_one(n + plane + ti);
+        if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti);
+        const float vv = vsh[buf][i];
+        const float *ap = &as[buf][q * JQ], *wp = &ws[buf][q * JQ], *kp = &ks[buf][q * JQ], *bp = &bs[buf][q * JQ], *rp = &rs[buf][q * JQ];
         float sa4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int j = 0; j < SZ; j++) sa4[j & 3] += s[j] * as[j];
-        const float sa = (sa4[0] + sa4[1]) + (sa4[2] + sa4[3]);
+        for (int jj = 0; jj < JQ; jj++) sa4[jj & 3] += s[jj] * ap[jj];
+        const float sa = quad_sum((sa4[0] + sa4[1]) + (sa4[2] + sa4[3]));
         float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int j = 0; j < SZ; j++) {
-            s[j] = s[j] * ws[j] + ks[j] * vv + sa * bs[j];
-            y4[j & 3] += rs[j] * s[j];
+        for (int jj = 0; jj < JQ; jj++) {
+            s[jj] = s[jj] * wp[jj] + kp[jj] * vv + sa * bp[jj];
+            y4[jj & 3] += rp[jj] * s[jj];
         }
-        const float y = (y4[0] + y4[1]) + (y4[2] + y4[3]);
-        if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
-        else x[ti] = y;
+        const float y = quad_sum((y4[0] + y4[1]) + (y4[2] + y4[3]));
+        if (q == 0) {
+            if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
+            else x[ti] = y;
+        }
     }
     if (held != 0xffffffffu) {
 #pragma unroll
-        for (int j = 0; j < SZ; j++) state[view_elem(vs, held, j + 1, chan)] = s[j];
+        for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
     }
 }
 
@@ -200,10 +230,10 @@ int wrq_time_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
 #define WRQ_TM7(SZ)                                                                                                                                  \
     if (S == SZ) {                                                                                                                                   \
         if (dtype == WRQ_F16)                                                                                                                        \
-            hipLaunchKernelGGL((time_mix_v7_kernel<uint16_t, SZ>), dim3(H), dim3(SZ), 0, hs, cur, sp, static_cast<const uint16_t *>(r->data),        \
+            hipLaunchKernelGGL((time_mix_v7_kernel<uint16_t, SZ>), dim3(H), dim3(4 * SZ), 0, hs, cur, sp, static_cast<const uint16_t *>(r->data),        \
                                static_cast<const uint16_t *>(w->data), static_cast<const uint16_t *>(n->data), static_cast<uint16_t *>(x->data), vs, H, A); \
         else                                                                                                                                         \
-            hipLaunchKernelGGL((time_mix_v7_kernel<float, SZ>), dim3(H), dim3(SZ), 0, hs, cur, sp, static_cast<const float *>(r->data),              \
+            hipLaunchKernelGGL((time_mix_v7_kernel<float, SZ>), dim3(H), dim3(4 * SZ), 0, hs, cur, sp, static_cast<const float *>(r->data),              \
                                static_cast<const float *>(w->data), static_cast<const float *>(n->data), static_cast<float *>(x->data), vs, H, A);   \
         return check_launch("time_mix_v7");                                                                                                          \
     }
