@@ -269,6 +269,11 @@ int wrq_lerp(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_v
  * TensorOp::channel_mix(cursors, state, r, v, x)
  *                                           src/tensor/ops.rs:1860-1915, src/shaders/channel_mix.wgsl
  *   state [C, 1, B, 1] <- x at every request's last token; x [C, A, 1, 1] <- sigmoid(r) * v.
+ * TensorOp::time_mix_v4(cursors, time_decay, time_first, state, k, v, r, x)
+ *                                           src/tensor/ops.rs:1464-1528, src/shaders/time_mix_v4.wgsl
+ *   x, k, v, r [C, A, 1, 1]; time_decay, time_first f32 [C, 1, 1, 1]; state [C, 4, B, 1]: row 0 <- x at
+ *   every request's last token, rows 1..3 the numerator, the denominator and their common exponent;
+ *   x <- sigmoid(r) * wkv, the exponent-shifted weighted average of v over the request's past.
  * TensorOp::time_mix_v5(cursors, time_decay, time_first, state, k, v, r, x)
  *                                           src/tensor/ops.rs:1530-1599, src/shaders/time_mix_v5.wgsl
  *   as time_mix_v6 below with time_decay f32 [S, H, 1, 1]: one decay per channel for every token.
@@ -284,6 +289,9 @@ int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
                     const wrq_tensor *output, wrq_dtype output_dtype, int reversed);
 int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor_view *state,
                     const wrq_tensor *r, const wrq_tensor *v, const wrq_tensor *x, wrq_dtype dtype);
+int wrq_time_mix_v4(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay,
+                    const wrq_tensor *time_first, const wrq_tensor_view *state, const wrq_tensor *k,
+                    const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype);
 int wrq_time_mix_v5(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay,
                     const wrq_tensor *time_first, const wrq_tensor_view *state, const wrq_tensor *k,
                     const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype);

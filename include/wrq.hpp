@@ -444,6 +444,16 @@ class TensorOp {
         });
     }
     template <typename F>
+    static TensorOp time_mix_v4(const TensorGpu<uint32_t> &cursors, const TensorGpu<float> &time_decay, const TensorGpu<float> &time_first,
+                                const TensorGpuView<float> &state, const TensorGpu<F> &k, const TensorGpu<F> &v, const TensorGpu<F> &r, const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor c = cursors.c(), td = time_decay.c(), tf = time_first.c(), tk = k.c(), tv = v.c(), tr = r.c(), tx = x.c();
+            const wrq_tensor_view st = state.c();
+            return wrq_time_mix_v4(s, &c, &td, &tf, &st, &tk, &tv, &tr, &tx, (wrq_dtype)dtype_of<F>::value);
+        });
+    }
+
+    template <typename F>
     static TensorOp time_mix_v5(const TensorGpu<uint32_t> &cursors, const TensorGpu<float> &time_decay, const TensorGpu<float> &time_first,
                                 const TensorGpuView<float> &state, const TensorGpu<F> &k, const TensorGpu<F> &v, const TensorGpu<F> &r, const TensorGpu<F> &x) {
         return checked([=](wrq_stream s) {

@@ -345,3 +345,29 @@ def channel_mix_v7(cursors, state_row, v, x):
         if a - first + 1 == cnt:
             state_row[slot] = x[a].astype(F)
     return np.asarray(v).astype(x.dtype)
+
+
+def time_mix_v4(cursors, time_decay, time_first, state, k, v, r, x):
+    """src/shaders/time_mix_v4.wgsl:67-129.  k, v, r, x (A, C); time_decay, time_first (C,); state
+    (B, 4, C) f32 updated in place (row 0: x at a request's last token; rows 1..3: aa, bb, pp).
+    Returns the new x."""
+    x = np.asarray(x)
+    A = x.shape[0]
+    k32, v32, r32 = (np.asarray(t).astype(F) for t in (k, v, r))
+    u, w = np.asarray(time_first).astype(F), np.asarray(time_decay).astype(F)
+    out = np.empty(x.shape, dtype=F)
+    for t in range(A):
+        slot, first, cnt = _cursor(cursors[t])
+        aa, bb, pp = state[slot, 1].copy(), state[slot, 2].copy(), state[slot, 3].copy()
+        if t - first + 1 == cnt:  # the shader stores this row at every token of the request, always from its last token
+            state[slot, 0] = x[first + cnt - 1].astype(F)
+        rr = F(1) / (F(1) + np.exp(-r32[t], dtype=F))
+        ww = u + k32[t]
+        q = np.maximum(pp, ww)
+        e1, e2 = np.exp(pp - q, dtype=F), np.exp(ww - q, dtype=F)
+        out[t] = rr * (e1 * aa + e2 * v32[t]) / (e1 * bb + e2)
+        ww = w + pp
+        q = np.maximum(ww, k32[t])
+        e1, e2 = np.exp(ww - q, dtype=F), np.exp(k32[t] - q, dtype=F)
+        state[slot, 1], state[slot, 2], state[slot, 3] = e1 * aa + e2 * v32[t], e1 * bb + e2, q
+    return out.astype(x.dtype)

@@ -379,6 +379,98 @@ def test_gpu_time_mix_v5(gpu, lop, dtype, H, S, runs):
 
 
 # ---------------------------------------------------------------------------------------------
+def wkv4_float64(cursors, w, u, state, k, v, r, x):
+    """the v4 recurrence without the exponent shift, in float64 (inputs small enough not to overflow):
+    a <- e^w a + e^k v, b <- e^w b + e^k, y = sigmoid(r) (a + e^(u+k) v) / (b + e^(u+k)); a = aa e^pp, b = bb e^pp.
+    Returns y, the true (a, b) of every request, and row 0."""
+    f = np.float64
+    A, C = x.shape
+    a = state[:, 1].astype(f) * np.exp(state[:, 3].astype(f))
+    b = state[:, 2].astype(f) * np.exp(state[:, 3].astype(f))
+    row0 = state[:, 0].astype(f).copy()
+    out = np.zeros((A, C))
+    for t in range(A):
+        c = int(cursors[t])
+        slot, first, cnt = c & 0xff, (c >> 8) & 0xffff, (c >> 24) & 0xff
+        if t - first + 1 == cnt:
+            row0[slot] = x[t].astype(f)
+        ek, eu = np.exp(k[t].astype(f)), np.exp(u.astype(f) + k[t].astype(f))
+        out[t] = (a[slot] + eu * v[t].astype(f)) / (b[slot] + eu) / (1 + np.exp(-r[t].astype(f)))
+        a[slot] = np.exp(w.astype(f)) * a[slot] + ek * v[t].astype(f)
+        b[slot] = np.exp(w.astype(f)) * b[slot] + ek
+    return out, a, b, row0
+
+
+def wkv4_inputs(rng, A, C, B, dtype):
+    k, v, r, x = (rng.standard_normal((A, C)).astype(dtype) for _ in range(4))
+    w = -np.exp(rng.standard_normal(C).astype(np.float32))  # the decay as the loader leaves it: -exp(time_decay)
+    u = (0.3 * rng.standard_normal(C)).astype(np.float32)
+    state = rng.standard_normal((B, 4, C)).astype(np.float32)
+    state[:, 2] = np.abs(state[:, 2]) + 0.5  # a denominator
+    state[3] = [[0] * C, [0] * C, [0] * C, [-1e30] * C]  # a fresh request: nothing seen yet
+    return k, v, r, x, w, u, state
+
+
+def check_wkv4_state(got, want_a, want_b, eps):
+    f = np.float64
+    assert_close(got[:, 1].astype(f) * np.exp(got[:, 3].astype(f)), want_a, eps, "numerator vs float64")
+    assert_close(got[:, 2].astype(f) * np.exp(got[:, 3].astype(f)), want_b, eps, "denominator vs float64")
+
+
+def test_oracle_time_mix_v4(lop):
+    rng = np.random.default_rng(SEED + 10)
+    C, B = 64, 6
+    runs = [(2, 3), (3, 2), (5, 4)]  # slot 3 starts fresh
+    cur = lop.pack_cursors(runs)
+    k, v, r, x, w, u, state = wkv4_inputs(rng, len(cur), C, B, np.float32)
+    st = state.copy()
+    got = lop.time_mix_v4(cur, w, u, st, k, v, r, x)
+    want, a, b, row0 = wkv4_float64(cur, w, u, state, k, v, r, x)
+    assert_close(got, want, 1e-5, "y vs float64")
+    check_wkv4_state(st, a, b, 1e-5)
+    assert_close(st[:, 0], row0, 0, "row 0")
+    assert np.array_equal(st[[0, 1, 4]], state[[0, 1, 4]])
+    # the first token of a fresh request returns sigmoid(r) v: the average of one value
+    assert_close(got[3], v[3] / (1 + np.exp(-r[3].astype(np.float64))), 1e-6, "fresh request")
+    # a run of 2 tokens equals two runs of 1 token
+    s_a, s_b = state.copy(), state.copy()
+    two = lop.time_mix_v4(lop.pack_cursors([(4, 2)]), w, u, s_a, k[:2], v[:2], r[:2], x[:2])
+    first = lop.time_mix_v4(lop.pack_cursors([(4, 1)]), w, u, s_b, k[:1], v[:1], r[:1], x[:1])
+    second = lop.time_mix_v4(lop.pack_cursors([(4, 1)]), w, u, s_b, k[1:2], v[1:2], r[1:2], x[1:2])
+    assert np.array_equal(two, np.concatenate([first, second])) and np.array_equal(s_a[:, 1:], s_b[:, 1:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("C,runs", [(64, [(2, 3), (3, 2), (5, 4)]), (768, [(3, 1)]), (1000, [(3, 40), (1, 2)])])
+def test_gpu_time_mix_v4(gpu, lop, dtype, C, runs):
+    import torch
+
+    print("time mix v4 on the GPU", dtype.__name__, C, runs, flush=True)
+    rng = np.random.default_rng(SEED + 70 + C)
+    B = 6
+    cur = lop.pack_cursors(runs)
+    A = len(cur)
+    k, v, r, x, w, u, state = wkv4_inputs(rng, A, C, B, dtype)
+    # the model's state holds 5 rows per layer (4 attention rows, 1 feed-forward row); the view picks the first 4
+    full = np.concatenate([state, np.full((B, 1, C), 7.0, dtype=np.float32)], axis=1)
+    sview = ((C, 4, B), (C, 5, B), (0, 0, 0))
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    sd, xd = dev(full), dev(x.reshape(1, A, C))
+    gpu.LayerOp.time_mix_v4(dev(cur.view(np.int32)), dev(w), dev(u), sd, dev(k.reshape(1, A, C)), dev(v.reshape(1, A, C)), dev(r.reshape(1, A, C)), xd, state_view=sview)
+    want, a, b, row0 = wkv4_float64(cur, w, u, state, k, v, r, x)
+    eps = 2e-3 if dtype == np.float16 else 2e-5
+    assert_close(xd.cpu().numpy()[0], want, eps, "y vs float64")
+    got_state = sd.cpu().numpy()
+    check_wkv4_state(got_state[:, :4], a, b, 5e-5)
+    assert_close(got_state[:, 0], row0, 0, "row 0")
+    assert np.array_equal(got_state[:, 4], full[:, 4])  # the feed-forward row is untouched
+    st = state.copy()
+    assert_close(xd.cpu().numpy()[0], lop.time_mix_v4(cur, w, u, st, k, v, r, x), eps, "y vs oracle")
+    assert_close(got_state[:, 1:4], st[:, 1:], 5e-5, "state vs oracle")
+
+
+# ---------------------------------------------------------------------------------------------
 # the ops an RWKV-v7 layer adds.  The reference has no test of them: the restatements are pinned by
 # float64 textbook forms, closed forms of special cases and invariants only (parity unpinned).
 def wkv7_float64(cursors, state, r, w, n, x):

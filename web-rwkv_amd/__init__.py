@@ -43,7 +43,7 @@ EXPORTS = [
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
-    "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v5", "wrq_time_mix_v6", "wrq_embed",
+    "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v4", "wrq_time_mix_v5", "wrq_time_mix_v6", "wrq_embed",
     "wrq_l2_norm", "wrq_control_k_v7", "wrq_time_mix_v7", "wrq_time_first_v7", "wrq_channel_mix_v7",
     "wrq_v6_pre", "wrq_v6_time_mix", "wrq_v6_decay", "wrq_v6_wkv_gate", "wrq_v6_post_ffn",
 ]
@@ -198,6 +198,7 @@ def lib():
         L.wrq_lerp.argtypes = [vp, V, V, V, i]
         L.wrq_token_shift.argtypes = [vp, T, V, V, T, i, T, i, i]
         L.wrq_channel_mix.argtypes = [vp, T, V, T, T, T, i]
+        L.wrq_time_mix_v4.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         L.wrq_time_mix_v5.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         L.wrq_time_mix_v6.argtypes = [vp, T, T, T, V, T, T, T, T, i]
         L.wrq_l2_norm.argtypes = [vp, T, i, C.c_float]
@@ -364,6 +365,12 @@ class LayerOp:
     def channel_mix(cursors, state, r, v, x, state_view=None):
         _check(lib().wrq_channel_mix(_stream(), C.byref(as_tensor(cursors)), C.byref(as_view(state, state_view)), C.byref(as_tensor(r)),
                                      C.byref(as_tensor(v)), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def time_mix_v4(cursors, time_decay, time_first, state, k, v, r, x, state_view=None):
+        _check(lib().wrq_time_mix_v4(_stream(), C.byref(as_tensor(cursors)), C.byref(as_tensor(time_decay)), C.byref(as_tensor(time_first)),
+                                     C.byref(as_view(state, state_view)), C.byref(as_tensor(k)), C.byref(as_tensor(v)), C.byref(as_tensor(r)),
+                                     C.byref(as_tensor(x)), _dtype(x)))
 
     @staticmethod
     def time_mix_v5(cursors, time_decay, time_first, state, k, v, r, x, state_view=None):

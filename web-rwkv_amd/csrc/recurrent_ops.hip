@@ -1,6 +1,7 @@
 // The ops of a v5 / v6 layer that carry state from token to token:
 //   token_shift   src/tensor/ops.rs:1393-1462, src/shaders/token_shift.wgsl
 //   channel_mix   src/tensor/ops.rs:1860-1915, src/shaders/channel_mix.wgsl
+//   time_mix_v4   src/tensor/ops.rs:1464-1528, src/shaders/time_mix_v4.wgsl
 //   time_mix_v5   src/tensor/ops.rs:1530-1599, src/shaders/time_mix_v5.wgsl
 //   time_mix_v6   src/tensor/ops.rs:1601-1677, src/shaders/time_mix_v6.wgsl
 //
@@ -168,6 +169,52 @@ __global__ __launch_bounds__(256) void time_mix_kernel(const uint32_t *cursors, 
     }
 }
 
+// The v4 recurrence, per channel: a numerator aa, a denominator bb and their common exponent pp,
+//   x <- sigmoid(r) (e^(pp-q) aa + e^(u+k-q) v) / (e^(pp-q) bb + e^(u+k-q)),  q = max(pp, u + k)
+//   aa, bb <- e^(w+pp-q') (aa, bb) + e^(k-q') (v, 1),  pp <- q' = max(w + pp, k)
+// One thread per channel walks the tokens of the run; a request's three values stay in registers over
+// its tokens (the shader reads and writes them per token), the next token's operands are fetched ahead.
+template <typename XT>
+__global__ __launch_bounds__(256) void time_mix_v4_kernel(const uint32_t *cursors, const float *time_decay, const float *time_first, float *state, const XT *k,
+                                                          const XT *v, const XT *r, XT *x, ViewArgs vs, uint32_t C, uint32_t A) {
+    const uint32_t c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const float u = time_first[c], w = time_decay[c];
+    float aa = 0.0f, bb = 0.0f, pp = 0.0f;
+    uint32_t held = 0xffffffffu;
+    float fk = load_one(k + c), fv = load_one(v + c), fr = load_one(r + c);
+    for (uint32_t t = 0; t < A; t++) {
+        const Cursor cur = read_cursor(cursors, t, vs);
+        const float kk = fk, vv = fv, rr = 1.0f / (1.0f + expf(-fr));
+        if (t + 1 < A) {
+            const uint64_t nx = (uint64_t)(t + 1) * C + c;
+            fk = load_one(k + nx), fv = load_one(v + nx), fr = load_one(r + nx);
+        }
+        if (cur.batch != held) {
+            if (held != 0xffffffffu)
+                state[view_elem(vs, held, 1, c)] = aa, state[view_elem(vs, held, 2, c)] = bb, state[view_elem(vs, held, 3, c)] = pp;
+            held = cur.batch;
+            aa = state[view_elem(vs, held, 1, c)], bb = state[view_elem(vs, held, 2, c)], pp = state[view_elem(vs, held, 3, c)];
+        }
+        const uint64_t ti = (uint64_t)t * C + c;
+        // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
+        if (t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, c)] = load_one(x + ti);
+        float ww = u + kk;
+        float q = fmaxf(pp, ww);
+        float e1 = expf(pp - q), e2 = expf(ww - q);
+        const float y = rr * (e1 * aa + e2 * vv) / (e1 * bb + e2);
+        if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
+        else x[ti] = y;
+        ww = w + pp;
+        q = fmaxf(ww, kk);
+        e1 = expf(ww - q), e2 = expf(kk - q);
+        aa = e1 * aa + e2 * vv;
+        bb = e1 * bb + e2;
+        pp = q;
+    }
+    if (held != 0xffffffffu) state[view_elem(vs, held, 1, c)] = aa, state[view_elem(vs, held, 2, c)] = bb, state[view_elem(vs, held, 3, c)] = pp;
+}
+
 template <typename FT, typename IT>
 int token_shift_out(hipStream_t stream, const wrq_tensor *cursors, const wrq_tensor_view *time_mix, const wrq_tensor_view *state, const wrq_tensor *input,
                     const wrq_tensor *output, int out_dtype, dim3 grid, int reversed) {
@@ -301,6 +348,37 @@ int time_mix(const char *name, bool token_decay, wrq_stream stream, const wrq_te
 } // namespace
 
 extern "C" {
+
+int wrq_time_mix_v4(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
+                    const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
+    int s = check_layer_tensor(cursors, "time_mix_v4");
+    for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
+        if (s == WRQ_OK) s = check_layer_tensor(t, "time_mix_v4");
+    if (s == WRQ_OK) s = check_layer_view(state, "time_mix_v4");
+    if (s != WRQ_OK) return s;
+    if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v4: the state is f32");
+    if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v4: unsupported element type %d", (int)dtype);
+    const uint32_t *sh = x->shape, *st = state->view.shape; // [C, A, 1, 1]
+    // src/tensor/ops.rs:1480-1485
+    const uint32_t vec[4] = {sh[0], 1, 1, 1};
+    if (sh[2] != 1 || sh[3] != 1 || !same_shape(k->shape, sh) || !same_shape(v->shape, sh) || !same_shape(r->shape, sh) || !same_shape(time_decay->shape, vec) ||
+        !same_shape(time_first->shape, vec) || st[0] != sh[0] || st[1] != 4 || st[3] != 1)
+        return fail(WRQ_ERR_SHAPE, "time_mix_v4: data shape not match [%u, %u, %u, %u]", sh[0], sh[1], sh[2], sh[3]);
+    if (cursors->shape[0] < sh[1]) return fail(WRQ_ERR_SHAPE, "time_mix_v4: %u cursors for %u tokens", cursors->shape[0], sh[1]);
+    if (sh[0] == 0 || sh[1] == 0) return WRQ_OK;
+    const ViewArgs vs = view_args(state->view);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    const uint32_t *cur = static_cast<const uint32_t *>(cursors->data);
+    const float *td = static_cast<const float *>(time_decay->data), *tfp = static_cast<const float *>(time_first->data);
+    const dim3 grid((sh[0] + 255) / 256);
+    if (dtype == WRQ_F16)
+        hipLaunchKernelGGL((time_mix_v4_kernel<uint16_t>), grid, dim3(256), 0, hs, cur, td, tfp, static_cast<float *>(state->data), static_cast<const uint16_t *>(k->data),
+                           static_cast<const uint16_t *>(v->data), static_cast<const uint16_t *>(r->data), static_cast<uint16_t *>(x->data), vs, sh[0], sh[1]);
+    else
+        hipLaunchKernelGGL((time_mix_v4_kernel<float>), grid, dim3(256), 0, hs, cur, td, tfp, static_cast<float *>(state->data), static_cast<const float *>(k->data),
+                           static_cast<const float *>(v->data), static_cast<const float *>(r->data), static_cast<float *>(x->data), vs, sh[0], sh[1]);
+    return check_launch("time_mix_v4");
+}
 
 int wrq_time_mix_v5(wrq_stream stream, const wrq_tensor *cursors, const wrq_tensor *time_decay, const wrq_tensor *time_first, const wrq_tensor_view *state,
                     const wrq_tensor *k, const wrq_tensor *v, const wrq_tensor *r, const wrq_tensor *x, wrq_dtype dtype) {
