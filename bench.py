@@ -485,6 +485,40 @@ def v5_model(wrq, torch, args):
                                              "27 ops per layer", "hip_graph": not args.no_graph, "packed_bytes": packed}, "data": "synthetic"}))
 
 
+def v7_layers(wrq, torch, args):
+    """RWKV-v7 layers at the 7B shape, every op through the library (src/runtime/v7.rs:704-1006), one
+    request, one HIP graph per step."""
+    v7 = importlib.import_module("web-rwkv_amd.v7")
+    C, heads, S, hidden, A = 4096, 64, 64, 16384, args.tokens
+    rng = np.random.default_rng(SEED + 9)
+    layers = [v7.Layer(torch, v7.random_layer_weights(rng, C, heads, S, hidden), args.quant) for _ in range(args.layers)]
+    states = [torch.zeros((1, S + 2, C), dtype=torch.float32, device="cuda") for _ in layers]
+    buf = v7.Runtime(torch, C, hidden, A)
+    x0 = torch.randn((1, A, C), device="cuda").half()
+    cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
+
+    def step():
+        buf.x.copy_(x0)  # the embedding of the next token would land here
+        for i, (layer, st) in enumerate(zip(layers, states)):
+            v7.dispatch_layer(layer, buf, st, cursors, A, heads, S, i)
+
+    step()
+    torch.cuda.synchronize()
+    if args.no_graph:
+        fn = step
+    else:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        fn = graph.replay
+    ms, wall_ms = time_steps(torch, fn, args.steps, args.warmup)
+    assert torch.isfinite(buf.x.float()).all()
+    print(json.dumps({"metric": "RWKV-v7 7B-shape layers, every op (no embedding, no head), tokens/s", "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
+                      "config": {"workload": f"{args.layers} v7 layers ({C} x {hidden}, {heads} heads), {args.quant}, {A} token(s) of one request per step, "
+                                             "51 ops per layer (47 in the first), the three independent projections in one launch", "hip_graph": not args.no_graph}, "data": "synthetic"}))
+
+
 def ops_table(wrq, torch, args, C):
     """Time of every layer op alone at the 7B layer shape, A tokens (HIP graph of 20 calls)."""
     LayerOp = wrq.LayerOp
@@ -567,6 +601,8 @@ def main():
     ap.add_argument("--ops", action="store_true", help="time of every layer op alone at the 7B layer shape")
     ap.add_argument("--fused", action="store_true", help="with --full-layers / --full-model: the fused small ops (12 launches per layer instead of 35)")
     ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
+    ap.add_argument("--v7-layers", action="store_true",
+                    help="every op of RWKV-v7 layers at the 7B shape (4096 channels, 64 heads, FFN 16384): --layers of them, --tokens per step")
     ap.add_argument("--v5-model", action="store_true",
                     help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
     args = ap.parse_args()
@@ -594,6 +630,9 @@ def main():
         return
     if args.v5_model:
         v5_model(wrq, torch, args)
+        return
+    if args.v7_layers:
+        v7_layers(wrq, torch, args)
         return
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
     if args.schedule:

@@ -7,7 +7,7 @@ import importlib
 import numpy as np
 
 _pkg = importlib.import_module(__name__.rsplit(".", 1)[0])
-LayerOp, Matrix, turbo = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo
+LayerOp, Matrix, turbo, matmul_vec_group = _pkg.LayerOp, _pkg.Matrix, _pkg.turbo, _pkg.matmul_vec_group
 ACT_NONE, ACT_SQUARED_RELU, ACT_TANH, ACT_SIGMOID = _pkg.ACT_NONE, _pkg.ACT_SQUARED_RELU, _pkg.ACT_TANH, _pkg.ACT_SIGMOID
 
 L2_EPS = 1.0e-12  # Model::L2_EPS, src/runtime/v7.rs:46
@@ -82,9 +82,9 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, index, rescale_now=False
     LayerOp.layer_norm(t["att_ln_w"], t["att_ln_b"], buf.att_x, LN_EPS)
     for name, out in (("x_r", buf.att_rx), ("x_w", buf.att_wx), ("x_k", buf.att_kx), ("x_v", buf.att_vx), ("x_a", buf.att_ax), ("x_g", buf.att_gx)):
         LayerOp.token_shift(cursors, t[name], state, buf.att_x, out, True, state_view=att_state)
-    m["att_w_r"].matmul_op(buf.att_rx, buf.att_r, ACT_NONE, fast)
-    m["att_w_k"].matmul_op(buf.att_kx, buf.att_k, ACT_NONE, fast)
-    m["att_w_v"].matmul_op(buf.att_vx, buf.att_v, ACT_NONE, fast)
+    # the three independent projections in one call: the library's form of a `TensorOp::List` of them
+    matmul_vec_group([(m["att_w_r"], buf.att_rx, buf.att_r, ACT_NONE, False, {}), (m["att_w_k"], buf.att_kx, buf.att_k, ACT_NONE, False, {}),
+                      (m["att_w_v"], buf.att_vx, buf.att_v, ACT_NONE, False, {})])
     m["w1"].matmul_op(buf.att_wx, buf.aux_w, ACT_TANH, fast)
     m["w2"].matmul_op(buf.aux_w, buf.att_w, ACT_NONE, fast)
     LayerOp.add(t["w0"], buf.att_w)
