@@ -328,6 +328,31 @@ int wrq_channel_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_t
                        const wrq_tensor *v, const wrq_tensor *x, wrq_dtype dtype);
 
 /*
+ * The rest of the reference's op set: two row normalisations, and what its loader uses for states and
+ * for blending low-rank adapters into matrices at load time (src/runtime/loader.rs:568-686).
+ * TensorOp::recenter(x)                     src/tensor/ops.rs:511-564, src/shaders/normalize.wgsl:46-80
+ *   x [C, T, B, 1] <- x - mean over the row.
+ * TensorOp::rms_norm(w, b, x, eps)          src/tensor/ops.rs:566-640, src/shaders/normalize.wgsl:82-116
+ *   x <- x / sqrt(mean of squares over the row + eps) * w + b; w, b f16 [C, 1, 1, 1].
+ * TensorOp::broadcast(input, output)        src/tensor/ops.rs:2070-2119, src/shaders/reshape.wgsl:35-56
+ *   output [C, T, B, 1] <- input [C, t, b, 1] repeated along tokens and batches (index modulo t, b).
+ * TensorOp::blend(factor, input, output)    src/tensor/ops.rs:2171-2224, src/shaders/blend.wgsl
+ *   output <- factor[0] input + factor[1] output; factor f32 [4, 1, 1, 1] on the device, equal shapes.
+ * TensorOp::blend_lora(factor, xa, xb, output)
+ *                                           src/tensor/ops.rs:2226-2282, src/shaders/blend_lora.wgsl
+ *   output [M, N, B, 1] <- factor[0] xa^T xb + factor[1] output with xa [K, M, B, 1], xb [K', N, B, 1], f16,
+ *   summed in f32 over min(K, K').
+ */
+int wrq_recenter(wrq_stream stream, const wrq_tensor *x, wrq_dtype dtype);
+int wrq_rms_norm(wrq_stream stream, const wrq_tensor *w, const wrq_tensor *b, const wrq_tensor *x,
+                 wrq_dtype dtype, float eps);
+int wrq_broadcast(wrq_stream stream, const wrq_tensor_view *input, const wrq_tensor_view *output);
+int wrq_blend(wrq_stream stream, const wrq_tensor *factor, const wrq_tensor *input, wrq_dtype input_dtype,
+              const wrq_tensor *output, wrq_dtype output_dtype);
+int wrq_blend_lora(wrq_stream stream, const wrq_tensor *factor, const wrq_tensor_view *xa,
+                   const wrq_tensor_view *xb, const wrq_tensor_view *output);
+
+/*
  * Fused forms of consecutive small ops of an RWKV-v6 layer (src/runtime/v6.rs:758-955).  They have no
  * counterpart among the reference's constructors; they are for callers that run a layer without hooks
  * between its ops: at batch 1 every op costs its launch, and these bring a layer from 35 launches to 12.

@@ -473,6 +473,33 @@ class TensorOp {
         });
     }
 
+    // the rest of the op set: src/tensor/ops.rs:511-564, :566-640, :2070-2119, :2171-2224, :2226-2282
+    template <typename F>
+    static TensorOp recenter(const TensorGpu<F> &x) {
+        return checked([=](wrq_stream s) { const wrq_tensor tx = x.c(); return wrq_recenter(s, &tx, (wrq_dtype)dtype_of<F>::value); });
+    }
+    template <typename F>
+    static TensorOp rms_norm(const TensorGpu<f16> &w, const TensorGpu<f16> &b, const TensorGpu<F> &x, float eps) {
+        return checked([=](wrq_stream s) { const wrq_tensor tw = w.c(), tb = b.c(), tx = x.c(); return wrq_rms_norm(s, &tw, &tb, &tx, (wrq_dtype)dtype_of<F>::value, eps); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp broadcast(const TensorGpuView<F0> &input, const TensorGpuView<F1> &output) {
+        return checked([=](wrq_stream s) { const wrq_tensor_view i = input.c(), o = output.c(); return wrq_broadcast(s, &i, &o); });
+    }
+    template <typename F0, typename F1>
+    static TensorOp blend(const TensorGpu<float> &factor, const TensorGpu<F0> &input, const TensorGpu<F1> &output) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor f = factor.c(), i = input.c(), o = output.c();
+            return wrq_blend(s, &f, &i, (wrq_dtype)dtype_of<F0>::value, &o, (wrq_dtype)dtype_of<F1>::value);
+        });
+    }
+    static TensorOp blend_lora(const TensorGpu<float> &factor, const TensorGpuView<f16> &xa, const TensorGpuView<f16> &xb, const TensorGpuView<f16> &output) {
+        return checked([=](wrq_stream s) {
+            const wrq_tensor f = factor.c();
+            const wrq_tensor_view a = xa.c(), b = xb.c(), o = output.c();
+            return wrq_blend_lora(s, &f, &a, &b, &o);
+        });
+    }
     // the ops an RWKV-v7 layer adds: src/tensor/ops.rs:642-700, :1800-1858, :1679-1741, :1743-1798, :1917-1970
     template <typename F>
     static TensorOp l2_norm(const TensorGpu<F> &x, float eps) {

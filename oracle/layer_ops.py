@@ -371,3 +371,59 @@ def time_mix_v4(cursors, time_decay, time_first, state, k, v, r, x):
         e1, e2 = np.exp(ww - q, dtype=F), np.exp(k32[t] - q, dtype=F)
         state[slot, 1], state[slot, 2], state[slot, 3] = e1 * aa + e2 * v32[t], e1 * bb + e2, q
     return out.astype(x.dtype)
+
+
+def _row_sum_tree(row, block, square):
+    """the shaders' row sum: per-lane vectors strided over the row, the tree over the threads, the four lanes"""
+    vec, valid = _lanes(row, block)
+    acc = np.zeros((block, 4), dtype=F)
+    for it in range(vec.shape[0]):
+        acc = np.where(valid[it][:, None], acc + (vec[it] * vec[it] if square else vec[it]), acc)
+    step = block >> 1
+    while step:
+        acc[:step] = acc[:step] + acc[step:2 * step]
+        step >>= 1
+    return F(F(acc[0, 0] + acc[0, 1]) + acc[0, 2]) + acc[0, 3]
+
+
+def recenter(x, block=128):
+    """src/shaders/normalize.wgsl:46-80: x - mean over the last axis."""
+    rows, shape, dtype = _rows(x)
+    out = np.empty_like(rows)
+    for i, row in enumerate(rows):
+        out[i] = row - F(_row_sum_tree(row, block, False) / F(row.size))
+    return out.reshape(shape).astype(dtype)
+
+
+def rms_norm(w, b, x, eps, block=128):
+    """src/shaders/normalize.wgsl:82-116: fma(x / sqrt(mean(x^2) + eps), w, b)."""
+    rows, shape, dtype = _rows(x)
+    out = np.empty_like(rows)
+    w32, b32 = np.asarray(w).astype(F), np.asarray(b).astype(F)
+    for i, row in enumerate(rows):
+        norm = F(1) / np.sqrt(F(_row_sum_tree(row, block, True) / F(row.size) + F(eps)), dtype=F)
+        out[i] = _fma(row * norm, w32, b32)
+    return out.reshape(shape).astype(dtype)
+
+
+def broadcast(src, dst):
+    """src/shaders/reshape.wgsl:35-56: dst (B, T, C) <- src (b, t, C) repeated along batches and tokens."""
+    src = np.asarray(src)
+    B, T, _ = dst.shape
+    dst[...] = src[np.arange(B) % src.shape[0]][:, np.arange(T) % src.shape[1]].astype(F).astype(dst.dtype)
+
+
+def blend(factor, x, y):
+    """src/shaders/blend.wgsl:49-70: factor[0] x + factor[1] y in y's type."""
+    f = np.asarray(factor, dtype=F)
+    return (f[0] * np.asarray(x).astype(F) + f[1] * np.asarray(y).astype(F)).astype(np.asarray(y).dtype)
+
+
+def blend_lora(factor, xa, xb, out):
+    """src/shaders/blend_lora.wgsl:49-119: out (B, N, M) <- factor[0] xb xa^T + factor[1] out; xa (B, M, K), xb (B, N, K') f16,
+    f32 sums over min(K, K') (in float64 here, rounded once: the shader's order of the 4 x 4 block sums is not followed)."""
+    f = np.asarray(factor, dtype=F)
+    xa, xb, out = np.asarray(xa), np.asarray(xb), np.asarray(out)
+    K = min(xa.shape[-1], xb.shape[-1])
+    prod = np.einsum("bnk,bmk->bnm", xb[..., :K].astype(np.float64), xa[..., :K].astype(np.float64)).astype(F)
+    return (f[0] * prod + f[1] * out.astype(F)).astype(out.dtype)

@@ -659,6 +659,97 @@ def test_gpu_v7_small_ops(gpu, lop, dtype):
 
 
 # ---------------------------------------------------------------------------------------------
+# the rest of the op set (no test in the reference: float64 forms and invariants pin the restatements)
+def test_oracle_misc_ops(lop):
+    rng = np.random.default_rng(SEED + 11)
+    f = np.float64
+    rows = (3.0 + rng.standard_normal((2, 5, 1000))).astype(np.float32)
+    got = lop.recenter(rows)
+    assert_close(got, rows.astype(f) - rows.astype(f).mean(axis=-1, keepdims=True), 1e-5, "recenter vs float64")
+    assert np.abs(got.astype(f).mean(axis=-1)).max() < 1e-5
+    w, b = (1.0 + 0.1 * rng.standard_normal(1000)).astype(np.float16), (0.1 * rng.standard_normal(1000)).astype(np.float16)
+    got = lop.rms_norm(w, b, rows, 1e-5)
+    want = rows.astype(f) / np.sqrt((rows.astype(f) ** 2).mean(axis=-1, keepdims=True) + 1e-5) * w.astype(f) + b.astype(f)
+    assert_close(got, want, 1e-5, "rms_norm vs float64")
+    # a row of equal values c: recenter gives 0, rms_norm gives sign(c) w + b (eps aside)
+    const = np.full((1, 64), -2.5, dtype=np.float32)
+    assert np.array_equal(lop.recenter(const), np.zeros((1, 64), dtype=np.float32))
+    assert_close(lop.rms_norm(w[:64], b[:64], const, 0.0), -w[:64].astype(f) + b[:64].astype(f), 1e-6, "rms_norm of a constant row")
+    src = rng.standard_normal((2, 3, 8)).astype(np.float16)
+    dst = np.zeros((4, 6, 8), dtype=np.float32)
+    lop.broadcast(src, dst)
+    for bb in range(4):
+        for t in range(6):
+            assert np.array_equal(dst[bb, t], src[bb % 2, t % 3].astype(np.float32))
+    x, y = rng.standard_normal((3, 16)).astype(np.float16), rng.standard_normal((3, 16)).astype(np.float32)
+    assert_close(lop.blend([0.25, 1.5, 0, 0], x, y), 0.25 * x.astype(f) + 1.5 * y.astype(f), 1e-6, "blend vs float64")
+    assert np.array_equal(lop.blend([0, 1, 0, 0], x, y), y) and np.array_equal(lop.blend([1, 0, 0, 0], x, y), x.astype(np.float32))
+    xa, xb = rng.standard_normal((2, 12, 8)).astype(np.float16), rng.standard_normal((2, 20, 8)).astype(np.float16)
+    out = rng.standard_normal((2, 20, 12)).astype(np.float16)
+    got = lop.blend_lora([0.5, 1.0, 0, 0], xa, xb, out)
+    want = 0.5 * np.stack([xb[i].astype(f) @ xa[i].astype(f).T for i in range(2)]) + out.astype(f)
+    assert_close(got, want, 2e-3, "blend_lora vs float64")
+    eye = np.eye(8, dtype=np.float16)[None]
+    assert np.array_equal(lop.blend_lora([1, 0, 0, 0], eye, xb[:1], np.zeros((1, 20, 8), dtype=np.float16)), xb[:1])  # xa = I: the product is xb
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_gpu_misc_ops(gpu, lop, dtype):
+    import torch
+
+    print("recenter / rms_norm / broadcast / blend / blend_lora on the GPU", dtype.__name__, flush=True)
+    rng = np.random.default_rng(SEED + 96)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    eps = 2e-3 if dtype == np.float16 else 2e-6
+    f = np.float64
+    for shape in ((2, 5, 1000), (1, 3, 4096), (3, 1, 64)):
+        rows = (1.0 + rng.standard_normal(shape)).astype(dtype)
+        C = shape[-1]
+        w, b = (1.0 + 0.1 * rng.standard_normal(C)).astype(np.float16), (0.1 * rng.standard_normal(C)).astype(np.float16)
+        xd = dev(rows)
+        gpu.LayerOp.recenter(xd)
+        assert_close(xd.cpu().numpy(), lop.recenter(rows), eps, f"recenter vs oracle {shape}")
+        assert_close(xd.cpu().numpy(), rows.astype(f) - rows.astype(f).mean(axis=-1, keepdims=True), 2 * eps, f"recenter vs float64 {shape}")
+        xd = dev(rows)
+        gpu.LayerOp.rms_norm(dev(w), dev(b), xd, 1e-5)
+        assert_close(xd.cpu().numpy(), lop.rms_norm(w, b, rows, 1e-5), eps, f"rms_norm vs oracle {shape}")
+    src = rng.standard_normal((2, 3, 256)).astype(np.float16)
+    big = np.zeros((5, 7, 256), dtype=dtype)
+    bd = dev(big)
+    gpu.LayerOp.broadcast(dev(src), bd, output_view=((256, 6, 4), (256, 7, 5), (0, 1, 1)))
+    want = big.copy()
+    lop.broadcast(src, want[1:, 1:])
+    assert np.array_equal(bd.cpu().numpy(), want)
+    x, y = rng.standard_normal((3, 5, 64)).astype(np.float16), rng.standard_normal((3, 5, 64)).astype(dtype)
+    factor = np.array([0.25, 1.5, 0, 0], dtype=np.float32)
+    yd = dev(y)
+    gpu.LayerOp.blend(dev(factor), dev(x), yd)
+    assert_close(yd.cpu().numpy(), lop.blend(factor, x, y), eps, "blend vs oracle")
+    with pytest.raises(gpu.TensorError):
+        gpu.LayerOp.blend(dev(factor), dev(x[:2]), yd)
+    if dtype == np.float16:
+        # a rank-32 adapter blended into a 768 x 512 matrix, and into a slice of a stack of matrices
+        M, N, K = 512, 768, 32
+        xa, xb = (0.1 * rng.standard_normal((1, M, K))).astype(np.float16), (0.1 * rng.standard_normal((1, N, K))).astype(np.float16)
+        out = (0.02 * rng.standard_normal((1, N, M))).astype(np.float16)
+        factor = np.array([2.0 / K, 1.0, 0, 0], dtype=np.float32)
+        od = dev(out)
+        gpu.LayerOp.blend_lora(dev(factor), dev(xa), dev(xb), od)
+        assert_close(od.cpu().numpy(), lop.blend_lora(factor, xa, xb, out), 2e-3, "blend_lora vs oracle")
+        want = factor[0] * (xb[0].astype(f) @ xa[0].astype(f).T) + out[0].astype(f)
+        assert_close(od.cpu().numpy()[0], want, 2e-3, "blend_lora vs float64")
+        stack = (0.02 * rng.standard_normal((3, 20, 64))).astype(np.float16)
+        xa, xb = rng.standard_normal((1, 64, 8)).astype(np.float16), rng.standard_normal((1, 20, 8)).astype(np.float16)
+        sd = dev(stack)
+        gpu.LayerOp.blend_lora(dev(factor), dev(xa), dev(xb), sd, output_view=((64, 20, 1), (64, 20, 3), (0, 0, 2)))
+        want = stack.copy()
+        want[2:] = lop.blend_lora(factor, xa, xb, stack[2:])
+        assert_close(sd.cpu().numpy(), want, 2e-3, "blend_lora into a slice")
+        assert np.array_equal(sd.cpu().numpy()[:2], stack[:2])
+
+
+# ---------------------------------------------------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_data_movement_kats(gpu):
     import torch

@@ -45,6 +45,7 @@ EXPORTS = [
     "wrq_blit", "wrq_transpose", "wrq_activate", "wrq_affine", "wrq_lerp",
     "wrq_token_shift", "wrq_channel_mix", "wrq_time_mix_v4", "wrq_time_mix_v5", "wrq_time_mix_v6", "wrq_embed",
     "wrq_l2_norm", "wrq_control_k_v7", "wrq_time_mix_v7", "wrq_time_first_v7", "wrq_channel_mix_v7",
+    "wrq_recenter", "wrq_rms_norm", "wrq_broadcast", "wrq_blend", "wrq_blend_lora",
     "wrq_v6_pre", "wrq_v6_time_mix", "wrq_v6_decay", "wrq_v6_wkv_gate", "wrq_v6_post_ffn",
 ]
 MAX_GROUP = 8
@@ -206,6 +207,11 @@ def lib():
         L.wrq_time_mix_v7.argtypes = [vp, T, V, T, T, T, T, i]
         L.wrq_time_first_v7.argtypes = [vp, T, T, T, T, i]
         L.wrq_channel_mix_v7.argtypes = [vp, T, V, T, T, i]
+        L.wrq_recenter.argtypes = [vp, T, i]
+        L.wrq_rms_norm.argtypes = [vp, T, T, T, i, C.c_float]
+        L.wrq_broadcast.argtypes = [vp, V, V]
+        L.wrq_blend.argtypes = [vp, T, T, i, T, i]
+        L.wrq_blend_lora.argtypes = [vp, T, V, V, V]
         L.wrq_embed.argtypes = [vp, T, T, T, i]
         u = C.c_uint32
         L.wrq_v6_pre.argtypes = [vp, u, u, vp, vp, vp, vp, vp, vp, C.c_float, V, i, vp, vp, vp, vp, vp]
@@ -383,6 +389,27 @@ class LayerOp:
         _check(lib().wrq_time_mix_v6(_stream(), C.byref(as_tensor(cursors)), C.byref(as_tensor(time_decay)), C.byref(as_tensor(time_first)),
                                      C.byref(as_view(state, state_view)), C.byref(as_tensor(k)), C.byref(as_tensor(v)), C.byref(as_tensor(r)),
                                      C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def recenter(x):
+        _check(lib().wrq_recenter(_stream(), C.byref(as_tensor(x)), _dtype(x)))
+
+    @staticmethod
+    def rms_norm(w, b, x, eps):
+        _check(lib().wrq_rms_norm(_stream(), C.byref(as_tensor(w)), C.byref(as_tensor(b)), C.byref(as_tensor(x)), _dtype(x), eps))
+
+    @staticmethod
+    def broadcast(input, output, input_view=None, output_view=None):
+        _check(lib().wrq_broadcast(_stream(), C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view))))
+
+    @staticmethod
+    def blend(factor, input, output):
+        _check(lib().wrq_blend(_stream(), C.byref(as_tensor(factor)), C.byref(as_tensor(input)), _dtype(input), C.byref(as_tensor(output)), _dtype(output)))
+
+    @staticmethod
+    def blend_lora(factor, xa, xb, output, xa_view=None, xb_view=None, output_view=None):
+        _check(lib().wrq_blend_lora(_stream(), C.byref(as_tensor(factor)), C.byref(as_view(xa, xa_view)), C.byref(as_view(xb, xb_view)),
+                                    C.byref(as_view(output, output_view))))
 
     @staticmethod
     def l2_norm(x, eps):
