@@ -1,0 +1,13 @@
+"""bench.py's command line where no GPU is needed: more than one GPU is refused with a message."""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and "shard by weight rows" in r.stderr
+    assert r.stdout.strip() == ""  # no bench line
