@@ -156,3 +156,50 @@ def dispatch_layer_auto(layer, buf, state, cursors, A, H, S, rescale_now=False):
         dispatch_layer_fused(layer, buf, state, cursors, A, H, S, rescale_now)
     else:
         dispatch_layer(layer, buf, state, cursors, A, H, S, rescale_now)
+
+
+def random_model_weights(rng, num_layer, C, H, S, hidden, vocab):
+    """The tensors around the layers (src/runtime/v6.rs:110-135): embedding f16 [vocab, C] with its layer
+    norm, the head's layer norm and the f16 head [vocab, C]."""
+    h16 = lambda *s, std=0.02: (rng.standard_normal(s, dtype=np.float32) * np.float32(std)).astype(np.float16)
+    return {
+        "embed": h16(vocab, C, std=0.5), "embed_ln_w": (1.0 + 0.1 * rng.standard_normal(C)).astype(np.float16), "embed_ln_b": h16(C, std=0.1),
+        "head_ln_w": (1.0 + 0.1 * rng.standard_normal(C)).astype(np.float16), "head_ln_b": h16(C, std=0.1), "head": h16(vocab, C),
+        "layers": [random_layer_weights(rng, C, H, S, hidden, layer=i) for i in range(num_layer)],
+    }
+
+
+class Model:
+    """A whole model on the device and one run of it (`Bundle::dispatch`, src/runtime/v6.rs:596-700):
+    embedding rows of the run's tokens, their layer norm, the layers (halving the residual after every
+    `rescale`-th one), then layer norm and head on the last token of the run's one request.  `dispatch`
+    chooses how a layer runs: `dispatch_layer` (the op list), `dispatch_layer_fused` or `dispatch_layer_auto`."""
+
+    def __init__(self, torch, weights, quant, H, S, hidden, slots, rescale=6, dispatch=dispatch_layer_auto):
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+        self.torch, self.H, self.S, self.hidden, self.rescale, self.layer_fn = torch, H, S, hidden, rescale, dispatch
+        self.C = H * S
+        self.t = {k: dev(v) for k, v in weights.items() if k not in ("layers", "head")}
+        self.head = Matrix.fp16(dev(weights["head"]))
+        self.layers = [Layer(torch, w, quant) for w in weights["layers"]]
+        self.state = [torch.zeros((slots, S + 2, self.C), dtype=torch.float32, device="cuda") for _ in self.layers]
+        self.vocab = weights["head"].shape[0]
+
+    def run(self, tokens, slot):
+        """One run: `tokens` (up to 255) of the request in `slot`; returns the f32 logits after the last one."""
+        torch, C, A = self.torch, self.C, len(tokens)
+        buf = Runtime(torch, C, self.hidden, A)
+        ids = torch.tensor([list(tokens)], dtype=torch.int32, device="cuda")
+        cursors = torch.from_numpy(np.full(A, slot | (A << 24), dtype=np.uint32).view(np.int32)).cuda()
+        inp = torch.zeros((1, A, C), dtype=torch.float16, device="cuda")
+        head_x = torch.zeros((1, 1, C), dtype=torch.float16, device="cuda")
+        logits = torch.zeros((1, 1, self.vocab), dtype=torch.float32, device="cuda")
+        LayerOp.embed(ids, self.t["embed"], inp)
+        LayerOp.layer_norm(self.t["embed_ln_w"], self.t["embed_ln_b"], inp, LN_EPS)
+        LayerOp.blit(inp, buf.x)
+        for i, (layer, st) in enumerate(zip(self.layers, self.state)):
+            self.layer_fn(layer, buf, st, cursors, A, self.H, self.S, rescale_now=(i + 1) % self.rescale == 0)
+        LayerOp.blit(buf.x, head_x, input_view=((C, 1, 1), (C, A, 1), (0, A - 1, 0)))
+        LayerOp.layer_norm(self.t["head_ln_w"], self.t["head_ln_b"], head_x, LN_EPS)
+        self.head.matmul_op(head_x, logits, ACT_NONE, turbo(1))
+        return logits.view(-1)
