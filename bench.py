@@ -462,7 +462,7 @@ def v5_model(wrq, torch, args):
     v5 = importlib.import_module("web-rwkv_amd.v5")
     L, heads, S, hidden, V = 12, 12, 64, 2688, 65536
     rng = np.random.default_rng(SEED + 1)
-    model = v5.Model(torch, v5.random_model_weights(rng, L, heads * S, heads, S, hidden, V), args.quant, heads, S, hidden, 1)
+    model = v5.Model(torch, v5.random_model_weights(rng, L, heads * S, heads, S, hidden, V), args.quant, heads, S, hidden, 1, packed_shifts=args.packed_shifts)
     out = {}
     for A in (32, 1):
         model.run([int(t) for t in rng.integers(0, V, A)], 0)
@@ -482,7 +482,7 @@ def v5_model(wrq, torch, args):
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(out[1][1], 4), "gpu_ms_per_step": round(out[1][0], 4),
                       "prompt_32_tokens_ms": round(out[32][1], 4), "prompt_tok_s": round(32e3 / out[32][1], 1),
                       "config": {"workload": f"{L} v5 layers (768 x {hidden}, {heads} heads), {args.quant}, embedding, head 65536 x 768 f16 on the last token; "
-                                             "27 ops per layer", "hip_graph": not args.no_graph, "packed_bytes": packed}, "data": "synthetic"}))
+                                             + ("21 ops per layer (token shifts of a half in one launch)" if args.packed_shifts else "27 ops per layer"), "hip_graph": not args.no_graph, "packed_bytes": packed}, "data": "synthetic"}))
 
 
 def v7_layers(wrq, torch, args):
@@ -603,6 +603,7 @@ def main():
     ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
     ap.add_argument("--v7-layers", action="store_true",
                     help="every op of RWKV-v7 layers at the 7B shape (4096 channels, 64 heads, FFN 16384): --layers of them, --tokens per step")
+    ap.add_argument("--packed-shifts", action="store_true", help="with --v5-model: the token shifts of each half of a layer in one launch")
     ap.add_argument("--v5-model", action="store_true",
                     help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
     args = ap.parse_args()

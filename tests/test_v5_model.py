@@ -74,3 +74,22 @@ def test_v5_model_prompt_and_greedy_decode(gpu, oracle):
     for i in range(L):
         assert_close(model.state[i].cpu().numpy(), state[i], 2e-2, f"state of layer {i} after the runs")
         assert not model.state[i][0].any()  # the other slot was never touched
+
+
+@pytest.mark.gpu
+def test_v5_model_packed_token_shifts_equal_the_op_list(gpu):
+    # one token shift per half of a layer (factors stacked and repeated over the tokens with `broadcast`)
+    # against the reference's four and two: the same logits and states, bit for bit
+    import torch
+
+    v5 = importlib.import_module(gpu.__name__ + ".v5")
+    L, H, S, hidden, V, B = 3, 12, 64, 2688, 4096, 2
+    print("v5-shape model, packed token shifts", flush=True)
+    rng = np.random.default_rng(SEED + 1)
+    w = v5.random_model_weights(rng, L, H * S, H, S, hidden, V)
+    models = [v5.Model(torch, w, "int8", H, S, hidden, B, packed_shifts=p) for p in (False, True)]
+    for tokens in ([int(t) for t in rng.integers(0, V, 32)], [7], [9, 11, 13]):
+        a, b = (m.run(tokens, 1).cpu().numpy() for m in models)
+        assert np.array_equal(a, b), f"logits after a run of {len(tokens)}"
+    for sa, sb in zip(models[0].state, models[1].state):
+        assert torch.equal(sa, sb)
