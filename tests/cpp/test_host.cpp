@@ -442,6 +442,29 @@ static void test_matrix_blob() {
     EXPECT(alias[1] == 0x63 && alias[2] == 'F' && alias[3] == 'p' && alias[4] == '4');
     alias[2] = 'N', alias[3] = 'f';
     EXPECT(serde::from_slice(alias.data(), alias.size()) == f4);
+    // the same matrix spelled with open-ended maps and arrays, the fields of the variant in another order and an
+    // integer in a longer form than needed: read as the same value
+    {
+        serde::Writer w;
+        auto open_tensor = [&](const TensorBlob &t) {
+            w.out.push_back(0xbf);
+            w.text("data"), w.bytes(t.data.data(), t.data.size());
+            w.text("shape");
+            w.out.push_back(0x9f);
+            w.out.push_back(0x19), w.out.push_back(0x00), w.out.push_back((uint8_t)t.shape[0]); // 16-bit form of a small extent
+            for (int d = 1; d < 4; d++) w.uint(t.shape[d]);
+            w.out.push_back(0xff);
+            w.out.push_back(0xff);
+        };
+        w.out.push_back(0xbf);
+        w.text("Int8");
+        w.out.push_back(0xbf);
+        w.text("m"), open_tensor(i8.m);
+        w.text("w"), open_tensor(i8.w);
+        w.out.push_back(0xff);
+        w.out.push_back(0xff);
+        EXPECT(serde::from_slice(w.out.data(), w.out.size()) == i8);
+    }
     // what must be refused: a cut file, another variant, scales that do not fit the weights, trailing bytes
     auto refused = [](const std::vector<uint8_t> &b) {
         try {
