@@ -496,11 +496,12 @@ def v7_layers(wrq, torch, args):
     buf = v7.Runtime(torch, C, hidden, A)
     x0 = torch.randn((1, A, C), device="cuda").half()
     cursors = torch.from_numpy(np.full(A, (min(A, 255) << 24), dtype=np.uint32).view(np.int32)).cuda()
+    shifts = [v7.PackedShifts(torch, layer, A) for layer in layers] if args.packed_shifts else None
 
     def step():
         buf.x.copy_(x0)  # the embedding of the next token would land here
         for i, (layer, st) in enumerate(zip(layers, states)):
-            v7.dispatch_layer(layer, buf, st, cursors, A, heads, S, i)
+            v7.dispatch_layer(layer, buf, st, cursors, A, heads, S, i, shifts=shifts[i] if shifts else None)
 
     step()
     torch.cuda.synchronize()
@@ -516,7 +517,7 @@ def v7_layers(wrq, torch, args):
     print(json.dumps({"metric": "RWKV-v7 7B-shape layers, every op (no embedding, no head), tokens/s", "value": round(A * 1e3 / wall_ms, 2), "unit": "tok/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "gpu_ms_per_step": round(ms, 4),
                       "config": {"workload": f"{args.layers} v7 layers ({C} x {hidden}, {heads} heads), {args.quant}, {A} token(s) of one request per step, "
-                                             "51 ops per layer (47 in the first), the three independent projections in one launch", "hip_graph": not args.no_graph}, "data": "synthetic"}))
+                                             + ("46 ops per layer (the six token shifts in one launch)" if args.packed_shifts else "51 ops per layer (47 in the first)") + ", the three independent projections in one launch", "hip_graph": not args.no_graph}, "data": "synthetic"}))
 
 
 def ops_table(wrq, torch, args, C):
@@ -603,7 +604,7 @@ def main():
     ap.add_argument("--full-model", action="store_true", help="--full-layers plus embedding, head and softmax: a whole model step")
     ap.add_argument("--v7-layers", action="store_true",
                     help="every op of RWKV-v7 layers at the 7B shape (4096 channels, 64 heads, FFN 16384): --layers of them, --tokens per step")
-    ap.add_argument("--packed-shifts", action="store_true", help="with --v5-model: the token shifts of each half of a layer in one launch")
+    ap.add_argument("--packed-shifts", action="store_true", help="with --v5-model / --v7-layers: the token shifts of each half of a layer in one launch")
     ap.add_argument("--v5-model", action="store_true",
                     help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
     args = ap.parse_args()

@@ -99,3 +99,34 @@ def test_v7_layers_against_numpy(gpu, oracle, quant, runs):
         untouched = [b for b in range(B) if b not in [s for s, _ in runs]]
         assert np.array_equal(sd.cpu().numpy()[untouched], state[untouched])
         want = got  # the next layer starts from the device's x on both sides
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("runs", [[(2, 3), (0, 1), (5, 4)], [(1, 32)], [(4, 1)]], ids=["8 tokens", "32 tokens", "1 token"])
+def test_v7_layer_packed_token_shifts_equal_the_op_list(gpu, runs):
+    # the six token shifts in one launch (factors stacked and repeated over the tokens with `broadcast`): bit-equal
+    import torch
+
+    sys.path.insert(0, ROOT)
+    lop = importlib.import_module("oracle.layer_ops")
+    v7 = importlib.import_module(gpu.__name__ + ".v7")
+    print("v7 layer, packed token shifts", runs, flush=True)
+    H, S, hidden, B = 4, 64, 1024, 6
+    C = H * S
+    rng = np.random.default_rng(SEED + 50 + len(runs))
+    cursors = lop.pack_cursors(runs)
+    A = len(cursors)
+    curd = torch.from_numpy(cursors.view(np.int32)).cuda()
+    layer = v7.Layer(torch, v7.random_layer_weights(rng, C, H, S, hidden), "int8")
+    x = rng.standard_normal((A, C)).astype(np.float16)
+    state = (0.1 * rng.standard_normal((B, S + 2, C))).astype(np.float32)
+    outs = []
+    for packed in (False, True):
+        buf = v7.Runtime(torch, C, hidden, A)
+        buf.x.copy_(torch.from_numpy(x).cuda().reshape(1, A, C))
+        buf.att_v0.copy_(torch.from_numpy(x[::-1].copy()).cuda().reshape(1, A, C))
+        sd = torch.from_numpy(state.copy()).cuda()
+        v7.dispatch_layer(layer, buf, sd, curd, A, H, S, 1, shifts=v7.PackedShifts(torch, layer, A) if packed else None)
+        torch.cuda.synchronize()
+        outs.append((buf.x.cpu().numpy(), sd.cpu().numpy()))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])

@@ -66,7 +66,21 @@ class Runtime:
         self.ffn_k = z(1, A, hidden)
 
 
-def dispatch_layer(layer, buf, state, cursors, A, H, S, index, rescale_now=False):
+class PackedShifts:
+    """The six token-shift factors of a layer's attention half stacked and repeated over the tokens of a run
+    (`[C, A, 6]`, made once per layer and run length with `TensorOp::broadcast`), so that one `token_shift`
+    in the reference's per-token form (src/tensor/ops.rs:1409-1414) replaces six launches."""
+
+    NAMES = ("x_r", "x_w", "x_k", "x_v", "x_a", "x_g")
+
+    def __init__(self, torch, layer, A):
+        C = layer.t["x_r"].numel()
+        self.mix = torch.empty((6, A, C), dtype=torch.float16, device="cuda")
+        LayerOp.broadcast(torch.stack([layer.t[n] for n in self.NAMES]).view(6, 1, C), self.mix)
+        self.sx = torch.zeros_like(self.mix)
+
+
+def dispatch_layer(layer, buf, state, cursors, A, H, S, index, rescale_now=False, shifts=None):
     """src/runtime/v7.rs:704-1006.  `state`: this layer's f32 tensor (B, S + 2, C): rows 0..S the
     attention state, row S + 1 the feed-forward one; `index`: the layer's number (layer 0 keeps its
     values as `att_v0`, the later ones mix theirs with it)."""
@@ -80,18 +94,24 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, index, rescale_now=False
 
     LayerOp.blit(buf.x, buf.att_x)
     LayerOp.layer_norm(t["att_ln_w"], t["att_ln_b"], buf.att_x, LN_EPS)
-    for name, out in (("x_r", buf.att_rx), ("x_w", buf.att_wx), ("x_k", buf.att_kx), ("x_v", buf.att_vx), ("x_a", buf.att_ax), ("x_g", buf.att_gx)):
-        LayerOp.token_shift(cursors, t[name], state, buf.att_x, out, True, state_view=att_state)
+    if shifts is None:
+        for name, out in (("x_r", buf.att_rx), ("x_w", buf.att_wx), ("x_k", buf.att_kx), ("x_v", buf.att_vx), ("x_a", buf.att_ax), ("x_g", buf.att_gx)):
+            LayerOp.token_shift(cursors, t[name], state, buf.att_x, out, True, state_view=att_state)
+        rx, wx, kx, vx, ax, gx = ((b, {}) for b in (buf.att_rx, buf.att_wx, buf.att_kx, buf.att_vx, buf.att_ax, buf.att_gx))
+    else:
+        # one launch for the six shifts; the products read their slice of the stack through views
+        LayerOp.token_shift(cursors, shifts.mix, state, buf.att_x, shifts.sx, True, state_view=att_state)
+        rx, wx, kx, vx, ax, gx = ((shifts.sx, dict(input_view=((C, A, 1), (C, A, 6), (0, 0, i)))) for i in range(6))
     # the three independent projections in one call: the library's form of a `TensorOp::List` of them
-    matmul_vec_group([(m["att_w_r"], buf.att_rx, buf.att_r, ACT_NONE, False, {}), (m["att_w_k"], buf.att_kx, buf.att_k, ACT_NONE, False, {}),
-                      (m["att_w_v"], buf.att_vx, buf.att_v, ACT_NONE, False, {})])
-    m["w1"].matmul_op(buf.att_wx, buf.aux_w, ACT_TANH, fast)
+    matmul_vec_group([(m["att_w_r"], rx[0], buf.att_r, ACT_NONE, False, rx[1]), (m["att_w_k"], kx[0], buf.att_k, ACT_NONE, False, kx[1]),
+                      (m["att_w_v"], vx[0], buf.att_v, ACT_NONE, False, vx[1])])
+    m["w1"].matmul_op(wx[0], buf.aux_w, ACT_TANH, fast, **wx[1])
     m["w2"].matmul_op(buf.aux_w, buf.att_w, ACT_NONE, fast)
     LayerOp.add(t["w0"], buf.att_w)
-    m["a1"].matmul_op(buf.att_ax, buf.aux_a, ACT_NONE, fast)
+    m["a1"].matmul_op(ax[0], buf.aux_a, ACT_NONE, fast, **ax[1])
     m["a2"].matmul_op(buf.aux_a, buf.att_a, ACT_NONE, fast)
     LayerOp.add_activate(t["a0"], buf.att_a, ACT_NONE, ACT_NONE, ACT_SIGMOID)
-    m["g1"].matmul_op(buf.att_gx, buf.aux_g, ACT_SIGMOID, fast)
+    m["g1"].matmul_op(gx[0], buf.aux_g, ACT_SIGMOID, fast, **gx[1])
     m["g2"].matmul_op(buf.aux_g, buf.att_g, ACT_NONE, fast)
     LayerOp.blit(buf.att_k, buf.att_kk)
     LayerOp.mul(t["k_k"], buf.att_kk)
@@ -100,7 +120,7 @@ def dispatch_layer(layer, buf, state, cursors, A, H, S, index, rescale_now=False
     if index == 0:
         LayerOp.blit(buf.att_v, buf.att_v0)
     else:
-        m["v1"].matmul_op(buf.att_vx, buf.aux_v, ACT_NONE, fast)
+        m["v1"].matmul_op(vx[0], buf.aux_v, ACT_NONE, fast, **vx[1])
         m["v2"].matmul_op(buf.aux_v, buf.att_vv, ACT_NONE, fast)
         LayerOp.add_activate(t["v0"], buf.att_vv, ACT_NONE, ACT_NONE, ACT_SIGMOID)
         LayerOp.lerp(buf.att_v0, buf.att_v, buf.att_vv, True)
