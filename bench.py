@@ -485,6 +485,32 @@ def v5_model(wrq, torch, args):
                                              + ("21 ops per layer (token shifts of a half in one launch)" if args.packed_shifts else "27 ops per layer"), "hip_graph": not args.no_graph, "packed_bytes": packed}, "data": "synthetic"}))
 
 
+def loader_bench(args):
+    """Writes the eight matrices of `--layers` 7B-shape layers (f16, 450 MB per layer) as a safetensors file
+    under the temporary directory and times the C++ loader on it (tests/cpp/test_host --loader-bench)."""
+    import subprocess
+    import tempfile
+
+    from safetensors.numpy import save_file
+
+    binary = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "test_host")
+    assert os.path.exists(binary), "build first: python -c 'import __graft_entry__ as g; g.build()'"
+    C, H = 4096, 14336
+    rng = np.random.default_rng(SEED + 11)
+    layers = min(args.layers, 4)
+    tensors = {}
+    for i in range(layers):
+        for name, (R, K) in {"att.key": (C, C), "att.value": (C, C), "att.receptance": (C, C), "att.gate": (C, C), "att.output": (C, C),
+                             "ffn.key": (H, C), "ffn.value": (C, H), "ffn.receptance": (C, C)}.items():
+            tensors[f"blocks.{i}.{name}.weight"] = (rng.standard_normal((R, K), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "layers.st")
+        save_file(tensors, path)
+        r = subprocess.run([binary, "--loader-bench", path], capture_output=True, text=True, timeout=600)
+    sys.stdout.write(r.stdout)
+    assert r.returncode == 0, r.stdout + r.stderr
+
+
 def v7_layers(wrq, torch, args):
     """RWKV-v7 layers at the 7B shape, every op through the library (src/runtime/v7.rs:704-1006), one
     request, one HIP graph per step."""
@@ -605,11 +631,17 @@ def main():
     ap.add_argument("--v7-layers", action="store_true",
                     help="every op of RWKV-v7 layers at the 7B shape (4096 channels, 64 heads, FFN 16384): --layers of them, --tokens per step")
     ap.add_argument("--packed-shifts", action="store_true", help="with --v5-model / --v7-layers: the token shifts of each half of a layer in one launch")
+    ap.add_argument("--loader", action="store_true",
+                    help="the C++ loader: the f16 matrices of --layers 7B-shape layers from a safetensors file into Int8 matrices (file -> device -> pack)")
     ap.add_argument("--v5-model", action="store_true",
                     help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
+
+    if args.loader:
+        loader_bench(args)
+        return
 
     import torch
 

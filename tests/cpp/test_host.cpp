@@ -4,6 +4,7 @@
 // float64 product on host-dequantised weights.
 #include <cmath>
 #include <cstdio>
+#include <chrono>
 #include <cstdlib>
 #include <fstream>
 #include <random>
@@ -613,8 +614,42 @@ static void test_loader_gpu(const std::string &model_path, const std::string &di
     EXPECT(sf4.kind == Matrix::Kind::Fp4 && sf4.q.back() == float4_quant_student(5.0));
 }
 
+// Timing of the loader on a model file (bench.py --loader): every 2-axis F16 tensor into an Int8 matrix,
+// once as it is and once with a discount (the host-side f32 multiply and f16 rounding in between).
+static int loader_bench(const std::string &model_path) {
+    check(wrq_init());
+    SafeTensors model(model_path);
+    Queue queue;
+    Loader loader(model, queue);
+    std::vector<std::string> names;
+    uint64_t bytes = 0;
+    for (const auto &name : model.names())
+        if (model.entry(name).dtype == "F16" && model.shape(name).size() == 2) names.push_back(name), bytes += model.tensor(name).second;
+    for (int pass = 0; pass < 3; pass++) { // pass 0 warms the page cache and the library
+        const bool discount = pass == 2;
+        const auto t0 = std::chrono::steady_clock::now();
+        for (const auto &name : names) {
+            const Matrix mx = discount ? loader.load_matrix_discount(name, Quant::Int8, 0.5f) : loader.load_matrix(name, Quant::Int8);
+            (void)mx;
+        }
+        queue.sync();
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        if (pass) std::printf("{\"loader\": \"%s\", \"matrices\": %zu, \"f16_bytes\": %llu, \"ms\": %.2f, \"GBps\": %.2f}\n", discount ? "int8 with discount" : "int8",
+                              names.size(), (unsigned long long)bytes, ms, bytes / ms / 1e6);
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
+    if (argc > 2 && std::string(argv[1]) == "--loader-bench") {
+        try {
+            return loader_bench(argv[2]);
+        } catch (const std::exception &e) {
+            std::printf("FAIL: %s\n", e.what());
+            return 1;
+        }
+    }
     if (argc > 3 && (std::string(argv[1]) == "--loader" || std::string(argv[1]) == "--loader-gpu")) {
         // the loader against a model file and its expectations, both written by tests/test_loader.py
         try {
