@@ -10,8 +10,8 @@
 //   sa[i] = sum_j S[j][i] a[j];   S[j][i] <- S[j][i] w[j] + k[j] v[i] + sa[i] b[j];   y[i] = sum_j r[j] S[j][i]
 // The shader walks the state in memory twice per token; here four lanes share column i of S and hold a
 // quarter of its j range each in registers for all tokens of a request in the run (two quad reductions
-// per token, for sa and for y); the five vectors over j of a token are fetched one token ahead and
-// passed round through LDS (two buffers, one barrier per token).  One workgroup of 4 S lanes per head.
+// per token, for sa and for y); the vectors over j of 1024 / S tokens at a time are fetched a chunk ahead
+// and passed round through LDS (two buffers, one barrier per chunk).  One workgroup of 256 lanes per head.
 #include "layer_device.h"
 
 namespace wrq {
@@ -51,78 +51,102 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
-// thread = (column i of S, quarter q of the j range): 4 SZ threads per head, JQ = SZ / 4 values of S per lane
+// One workgroup of 256 threads per head: thread = (column i of S, quarter q of the j range), JQ = SZ / 4
+// values of S per lane; heads of more than 64 columns take several passes over the run.  The operands of the
+// head come in chunks of 1024 / SZ tokens: every thread fetches one 4-element vector of each of the six
+// while the previous chunk is worked on, the chunk is passed round through LDS (two buffers, one barrier per
+// chunk), and the lanes of a quarter read their j range as broadcasts.  Within a chunk a token needs no
+// barrier: both sums over j close inside a quad.
 template <typename XT, int SZ>
-__global__ __launch_bounds__(4 * SZ) void time_mix_v7_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *w, const XT *n, XT *x, ViewArgs vs,
-                                                             uint32_t H, uint32_t A) {
+__global__ __launch_bounds__(256) void time_mix_v7_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *w, const XT *n, XT *x, ViewArgs vs,
+                                                          uint32_t H, uint32_t A) {
     constexpr int JQ = SZ / 4;
-    // the vectors over j of a token and its v, two buffers: token t + 1 is written while token t may still be read
-    __shared__ __align__(16) float rs[2][SZ], ws[2][SZ], ks[2][SZ], as[2][SZ], bs[2][SZ], vsh[2][SZ];
-    const uint32_t head = blockIdx.x, tid = threadIdx.x, i = tid >> 2, q = tid & 3;
-    const uint32_t C = SZ * H, chan = head * SZ + i;
+    constexpr int TB = 1024 / SZ; // tokens per chunk
+    __shared__ __align__(16) float rs[2][1024], ws[2][1024], ks[2][1024], as[2][1024], bs[2][1024], vsh[2][1024];
+    __shared__ uint32_t csh[2][TB]; // the chunk's cursors
+    const uint32_t head = blockIdx.x, tid = threadIdx.x, q = tid & 3;
+    const uint32_t C = SZ * H;
     const uint64_t plane = (uint64_t)A * C; // n holds k, v, a, kk one after the other
-    const bool stager = tid < (uint32_t)SZ; // the first SZ threads fetch element `tid` of a token's operands, one token ahead
-    float s[JQ];
-    uint32_t held = 0xffffffffu; // request whose S is in registers
-    float fr = 0, fw = 0, fk = 0, fv = 0, fa = 0, fkk = 0;
-    uint32_t fc;
-    auto fetch = [&](uint32_t t) {
-        fc = cursors[t];
-        if (stager) {
-            const uint64_t ti = (uint64_t)t * C + head * SZ + tid;
-            fr = load_one(r + ti), fw = load_one(w + ti), fk = load_one(n + ti), fv = load_one(n + plane + ti);
-            fa = load_one(n + 2 * plane + ti), fkk = load_one(n + 3 * plane + ti);
-        }
+    const uint32_t nchunk = (A + TB - 1) / TB;
+    // this thread's vector of a chunk: token tid / (SZ / 4) of the chunk, elements 4 (tid % (SZ / 4)) ..
+    const uint32_t lt = tid / (SZ / 4), le = 4 * (tid % (SZ / 4));
+    float4 fr, fw, fk, fv, fa, fkk;
+    uint32_t fc = 0;
+    auto fetch = [&](uint32_t chunk) {
+        const uint32_t t = min(chunk * TB + lt, A - 1); // clamped: tokens past the run are never used
+        const uint64_t g = (uint64_t)t * C + head * SZ + le;
+        fr = load_vec4(r + g), fw = load_vec4(w + g), fk = load_vec4(n + g), fv = load_vec4(n + plane + g);
+        fa = load_vec4(n + 2 * plane + g), fkk = load_vec4(n + 3 * plane + g);
+        if (tid < (uint32_t)TB) fc = cursors[min(chunk * TB + tid, A - 1)];
     };
-    fetch(0);
-    for (uint32_t t = 0; t < A; t++) {
-        const int buf = t & 1;
-        Cursor cur = unpack_cursor(fc);
-        cur.batch = min(cur.batch, vs.shape[2] - 1); // as read_cursor
-        cur.token = min(cur.token, t);
-        if (stager) {
-            rs[buf][tid] = fr;
-            ws[buf][tid] = expf(-0.606531f / (1.0f + expf(-fw))); // exp(-exp(-0.5) sigmoid(w))
-            ks[buf][tid] = fk;
-            as[buf][tid] = -fkk;
-            bs[buf][tid] = fkk * fa;
-            vsh[buf][tid] = fv;
-        }
-        __syncthreads(); // token t is in LDS; the other buffer was last read before the previous barrier
-        if (t + 1 < A) fetch(t + 1);
-        if (cur.batch != held) {
-            if (held != 0xffffffffu) {
+    auto decay = [](float v) { return expf(-0.606531f / (1.0f + expf(-v))); }; // exp(-exp(-0.5) sigmoid(w))
+    auto stage = [&](int buf) {
+        *reinterpret_cast<float4 *>(&rs[buf][4 * tid]) = fr;
+        *reinterpret_cast<float4 *>(&ws[buf][4 * tid]) = make_float4(decay(fw.x), decay(fw.y), decay(fw.z), decay(fw.w));
+        *reinterpret_cast<float4 *>(&ks[buf][4 * tid]) = fk;
+        *reinterpret_cast<float4 *>(&as[buf][4 * tid]) = make_float4(-fkk.x, -fkk.y, -fkk.z, -fkk.w);
+        *reinterpret_cast<float4 *>(&bs[buf][4 * tid]) = make_float4(fkk.x * fa.x, fkk.y * fa.y, fkk.z * fa.z, fkk.w * fa.w);
+        *reinterpret_cast<float4 *>(&vsh[buf][4 * tid]) = fv;
+        if (tid < (uint32_t)TB) csh[buf][tid] = fc;
+    };
+    for (uint32_t i0 = 0; i0 < SZ; i0 += 64) {
+        const uint32_t i = i0 + (tid >> 2);
+        const bool live = i < SZ; // head sizes below 64 leave waves without a column
+        const uint32_t chan = head * SZ + min(i, (uint32_t)SZ - 1);
+        float s[JQ];
+        uint32_t held = 0xffffffffu; // request whose S is in registers
+        fetch(0);
+        __syncthreads(); // the buffers may still be read by the previous pass over i
+        stage(0);
+        for (uint32_t chunk = 0; chunk < nchunk; chunk++) {
+            const int buf = chunk & 1;
+            if (chunk + 1 < nchunk) fetch(chunk + 1);
+            __syncthreads(); // chunk `chunk` is in LDS; buffer buf ^ 1 is free
+            const uint32_t tend = min((uint32_t)TB, A - chunk * TB);
+            if (live) {
+                for (uint32_t tt = 0; tt < tend; tt++) {
+                    const uint32_t t = chunk * TB + tt;
+                    Cursor cur = unpack_cursor(csh[buf][tt]);
+                    cur.batch = min(cur.batch, vs.shape[2] - 1); // as read_cursor
+                    cur.token = min(cur.token, t);
+                    if (cur.batch != held) {
+                        if (held != 0xffffffffu) {
 #pragma unroll
-                for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
+                            for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
+                        }
+                        held = cur.batch;
+#pragma unroll
+                        for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
+                    }
+                    const uint64_t ti = (uint64_t)t * C + chan;
+                    // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
+                    if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti);
+                    const float vv = vsh[buf][tt * SZ + i];
+                    const float *ap = &as[buf][tt * SZ + q * JQ], *wp = &ws[buf][tt * SZ + q * JQ], *kp = &ks[buf][tt * SZ + q * JQ],
+                                *bp = &bs[buf][tt * SZ + q * JQ], *rp = &rs[buf][tt * SZ + q * JQ];
+                    float sa4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int jj = 0; jj < JQ; jj++) sa4[jj & 3] += s[jj] * ap[jj];
+                    const float sa = quad_sum((sa4[0] + sa4[1]) + (sa4[2] + sa4[3]));
+                    float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int jj = 0; jj < JQ; jj++) {
+                        s[jj] = s[jj] * wp[jj] + kp[jj] * vv + sa * bp[jj];
+                        y4[jj & 3] += rp[jj] * s[jj];
+                    }
+                    const float y = quad_sum((y4[0] + y4[1]) + (y4[2] + y4[3]));
+                    if (q == 0) {
+                        if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
+                        else x[ti] = y;
+                    }
+                }
             }
-            held = cur.batch;
-#pragma unroll
-            for (int jj = 0; jj < JQ; jj++) s[jj] = state[view_elem(vs, held, q * JQ + jj + 1, chan)];
+            if (chunk + 1 < nchunk) stage(buf ^ 1); // read two chunks ago, before the barrier above
         }
-        const uint64_t ti = (uint64_t)t * C + chan;
-        // row 0 of the request's state keeps the layer's input at its last token (read before x is overwritten)
-        if (q == 0 && t - cur.token + 1 == cur.len) state[view_elem(vs, cur.batch, 0, chan)] = load_one(x + ti);
-        const float vv = vsh[buf][i];
-        const float *ap = &as[buf][q * JQ], *wp = &ws[buf][q * JQ], *kp = &ks[buf][q * JQ], *bp = &bs[buf][q * JQ], *rp = &rs[buf][q * JQ];
-        float sa4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (live && held != 0xffffffffu) {
 #pragma unroll
-        for (int jj = 0; jj < JQ; jj++) sa4[jj & 3] += s[jj] * ap[jj];
-        const float sa = quad_sum((sa4[0] + sa4[1]) + (sa4[2] + sa4[3]));
-        float y4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int jj = 0; jj < JQ; jj++) {
-            s[jj] = s[jj] * wp[jj] + kp[jj] * vv + sa * bp[jj];
-            y4[jj & 3] += rp[jj] * s[jj];
+            for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
         }
-        const float y = quad_sum((y4[0] + y4[1]) + (y4[2] + y4[3]));
-        if (q == 0) {
-            if constexpr (sizeof(XT) == 2) x[ti] = f2h(y);
-            else x[ti] = y;
-        }
-    }
-    if (held != 0xffffffffu) {
-#pragma unroll
-        for (int jj = 0; jj < JQ; jj++) state[view_elem(vs, held, q * JQ + jj + 1, chan)] = s[jj];
     }
 }
 
@@ -230,10 +254,10 @@ int wrq_time_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
 #define WRQ_TM7(SZ)                                                                                                                                  \
     if (S == SZ) {                                                                                                                                   \
         if (dtype == WRQ_F16)                                                                                                                        \
-            hipLaunchKernelGGL((time_mix_v7_kernel<uint16_t, SZ>), dim3(H), dim3(4 * SZ), 0, hs, cur, sp, static_cast<const uint16_t *>(r->data),        \
+            hipLaunchKernelGGL((time_mix_v7_kernel<uint16_t, SZ>), dim3(H), dim3(256), 0, hs, cur, sp, static_cast<const uint16_t *>(r->data),        \
                                static_cast<const uint16_t *>(w->data), static_cast<const uint16_t *>(n->data), static_cast<uint16_t *>(x->data), vs, H, A); \
         else                                                                                                                                         \
-            hipLaunchKernelGGL((time_mix_v7_kernel<float, SZ>), dim3(H), dim3(4 * SZ), 0, hs, cur, sp, static_cast<const float *>(r->data),              \
+            hipLaunchKernelGGL((time_mix_v7_kernel<float, SZ>), dim3(H), dim3(256), 0, hs, cur, sp, static_cast<const float *>(r->data),              \
                                static_cast<const float *>(w->data), static_cast<const float *>(n->data), static_cast<float *>(x->data), vs, H, A);   \
         return check_launch("time_mix_v7");                                                                                                          \
     }
