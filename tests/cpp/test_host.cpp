@@ -340,6 +340,51 @@ static void test_gpu_layer_ops() {
 }
 
 
+// The ops of the v4 / v5 / v7 layers and of the loader: a mis-shaped operand is refused with the reference's
+// shape error when the op is submitted, before anything is launched (no device needed).
+static void test_layer_op_shape_errors() {
+    auto fake = reinterpret_cast<void *>(0x10000);
+    const uint32_t S = 64, H = 2, A = 3, B = 2, C = S * H;
+    auto cursors = TensorGpu<uint32_t>::wrap(fake, Shape(A, 1, 1, 1));
+    auto heads = TensorGpu<f16>::wrap(fake, Shape(S, H, A, 1));
+    auto heads32 = TensorGpu<float>::wrap(fake, Shape(S, H, A, 1));
+    auto n4 = TensorGpu<f16>::wrap(fake, Shape(S, H, A, 4)), n3 = TensorGpu<f16>::wrap(fake, Shape(S, H, A, 3));
+    auto u = TensorGpu<f16>::wrap(fake, Shape(S, H, 1, 1));
+    auto chan = TensorGpu<f16>::wrap(fake, Shape(C, 1, 1, 1));
+    auto decay = TensorGpu<float>::wrap(fake, Shape(S, H, 1, 1)), decay_t = TensorGpu<float>::wrap(fake, Shape(S, H, A, 1));
+    auto flat = TensorGpu<f16>::wrap(fake, Shape(C, A, 1, 1)), flat2 = TensorGpu<f16>::wrap(fake, Shape(C, A + 1, 1, 1));
+    auto vec32 = TensorGpu<float>::wrap(fake, Shape(C, 1, 1, 1));
+    auto state = TensorGpu<float>::wrap(fake, Shape(C, S + 2, B, 1));
+    const auto att = view_of(state, {{{0, C}, {0, S + 1}, {0, B}, {0, 1}}}), ffn = view_of(state, {{{0, C}, {S + 1, S + 2}, {0, B}, {0, 1}}});
+    auto factor = TensorGpu<float>::wrap(fake, Shape(4, 1, 1, 1));
+    Queue queue;
+    const std::pair<const char *, TensorOp> bad[] = {
+        {"time_mix_v4", TensorOp::time_mix_v4(cursors, vec32, vec32, att, flat, flat, flat, flat)},               // the v4 state has 4 rows
+        {"time_mix_v5", TensorOp::time_mix_v5(cursors, decay_t, decay, att, heads32, heads32, heads32, heads32)}, // a decay per token is v6's
+        {"time_mix_v6", TensorOp::time_mix_v6(cursors, decay, decay, att, heads32, heads32, heads32, heads32)},   // a decay per channel is v5's
+        {"time_mix_v7", TensorOp::time_mix_v7(cursors, att, heads, heads, n3, heads)},
+        {"time_first_v7", TensorOp::time_first_v7(chan, heads, n4, heads)},
+        {"control_k_v7", TensorOp::control_k_v7(u, TensorGpuView<f16>(flat), TensorGpuView<f16>(flat))},
+        {"channel_mix_v7", TensorOp::channel_mix_v7(cursors, att, flat, flat)},                                  // the feed-forward state is one row
+        {"l2_norm", TensorOp::l2_norm(n4, 1e-12f)},
+        {"rms_norm", TensorOp::rms_norm(u, u, flat, 1e-5f)},
+        {"broadcast", TensorOp::broadcast(TensorGpuView<f16>(u), TensorGpuView<f16>(flat))},
+        {"blend", TensorOp::blend(factor, flat, flat2)},
+        {"blend_lora", TensorOp::blend_lora(factor, TensorGpuView<f16>(flat), TensorGpuView<f16>(flat), TensorGpuView<f16>(flat))},
+    };
+    for (const auto &kv : bad) {
+        bool threw = false;
+        try {
+            queue.submit(kv.second);
+        } catch (const TensorError &e) {
+            threw = e.status == WRQ_ERR_SHAPE && std::string(e.what()).find(kv.first) == 0;
+        }
+        if (!threw) std::printf("not refused: %s\n", kv.first);
+        EXPECT(threw);
+    }
+    (void)ffn;
+}
+
 // ---------------------------------------------------------------- on-disk form of a Matrix
 
 static std::vector<uint8_t> hex(const char *s) {
@@ -668,6 +713,7 @@ int main(int argc, char **argv) {
     test_redirect();
     test_schedule_of_the_configs();
     test_build_time_errors();
+    test_layer_op_shape_errors();
     test_cbor_items();
     test_matrix_blob();
     if (!cpu_only) {
