@@ -109,3 +109,101 @@ def test_library_against_exact_fixtures(gpu, c):
         out = torch.empty((c["T"], c["R"]), dtype=torch.float32, device="cuda")
         (m.matmul_vec_op if entry == "vec" else m.matmul_mat_op)(xd, out)
         assert_close(out.cpu().numpy(), want, eps, f"{entry} vs exact product")
+
+
+# ---------------------------------------------------------------------------------------------
+# the recurrences of the four model versions against committed float64 vectors
+# (tests/golden/recurrent_float64.json, written by make_recurrent_golden.py beside it)
+with open(os.path.join(HERE, "golden", "recurrent_float64.json")) as f:
+    REC = json.load(f)
+
+
+def rec_arrays(version):
+    c, H, S, B = REC[version], REC["H"], REC["S"], REC["B"]
+    A = sum(n for _, n in REC["runs"])
+    f32 = lambda key, *shape: np.array(c[key], dtype=np.float32).reshape(shape)
+    f64 = lambda key, *shape: np.array(c[key], dtype=np.float64).reshape(shape)
+    return c, H, S, B, A, f32, f64
+
+
+def run_recurrence(version, ops, cursors, to_dev, to_host, dtype):
+    """`ops`: the oracle module or the library's LayerOp; returns (y, state after) as numpy arrays."""
+    c, H, S, B, A, f32, f64 = rec_arrays(version)
+    C = H * S
+    cast = lambda a: a.astype(dtype)
+    if version == "v4":
+        state = f32("state", B, 4, C)
+        k, v, r, x = (cast(f32(n, A, C)) for n in ("k", "v", "r", "x"))
+        w, u = f32("time_decay", C), f32("time_first", C)
+        return state, (k, v, r, x, w, u)
+    state = f32("state", B, S + 1, C)
+    if version == "v7":
+        return state, (cast(f32("r", A, H, S)), cast(f32("w", A, H, S)), cast(f32("n", 4, A, H, S)), cast(f32("x", A, H, S)))
+    wshape = (A, H, S) if version == "v6" else (H, S)
+    k, v, r, x = (cast(f32(n, A, H, S)) for n in ("k", "v", "r", "x"))
+    return state, (k, v, r, x, f32("time_decay", *wshape), f32("time_first", H, S))
+
+
+def check_recurrence(version, y, state_after, eps_y, eps_state):
+    c, H, S, B, A, f32, f64 = rec_arrays(version)
+    C = H * S
+    if version == "v4":
+        assert_close(y, f64("y", A, C), eps_y, "v4 y vs float64 fixture")
+        st = state_after.astype(np.float64)
+        assert_close(st[:, 1] * np.exp(st[:, 3]), f64("numerator_after", B, C), eps_state, "v4 numerator")
+        assert_close(st[:, 2] * np.exp(st[:, 3]), f64("denominator_after", B, C), eps_state, "v4 denominator")
+        assert_close(st[:, 0], f64("row0_after", B, C), 1e-7, "v4 row 0")
+        return
+    assert_close(y, f64("y", A, H, S), eps_y, f"{version} y vs float64 fixture")
+    assert_close(state_after, f64("state_after", B, S + 1, C), eps_state, f"{version} state vs float64 fixture")
+
+
+@pytest.mark.parametrize("version", ["v4", "v5", "v6", "v7"])
+def test_oracle_recurrences_against_float64_fixtures(version):
+    sys.path.insert(0, ROOT)
+    lop = importlib.import_module("oracle.layer_ops")
+    cursors = lop.pack_cursors([tuple(r) for r in REC["runs"]])
+    state, a = run_recurrence(version, lop, cursors, None, None, np.float32)
+    if version == "v4":
+        k, v, r, x, w, u = a
+        y = lop.time_mix_v4(cursors, w, u, state, k, v, r, x)
+    elif version == "v7":
+        r, w, n, x = a
+        y = lop.time_mix_v7(cursors, state, r, w, n, x)
+    else:
+        k, v, r, x, w, u = a
+        y = (lop.time_mix_v5 if version == "v5" else lop.time_mix_v6)(cursors, w, u, state, k, v, r, x)
+    check_recurrence(version, y, state, 2e-5, 2e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("version", ["v4", "v5", "v6", "v7"])
+def test_library_recurrences_against_float64_fixtures(gpu, version, dtype):
+    import torch
+
+    print("recurrence fixture on the GPU", version, dtype.__name__, flush=True)
+    sys.path.insert(0, ROOT)
+    lop = importlib.import_module("oracle.layer_ops")
+    cursors = lop.pack_cursors([tuple(r) for r in REC["runs"]])
+    state, a = run_recurrence(version, None, cursors, None, None, dtype)
+    dev = lambda t: torch.from_numpy(np.ascontiguousarray(t)).cuda()
+    cur, sd = dev(cursors.view(np.int32)), dev(state)
+    if version == "v4":
+        k, v, r, x, w, u = a
+        A, C = x.shape
+        xd = dev(x.reshape(1, A, C))
+        gpu.LayerOp.time_mix_v4(cur, dev(w), dev(u), sd, dev(k.reshape(1, A, C)), dev(v.reshape(1, A, C)), dev(r.reshape(1, A, C)), xd)
+        y = xd.cpu().numpy()[0]
+    elif version == "v7":
+        r, w, n, x = a
+        xd = dev(x)
+        gpu.LayerOp.time_mix_v7(cur, sd, dev(r), dev(w), dev(n), xd)
+        y = xd.cpu().numpy()
+    else:
+        k, v, r, x, w, u = a
+        xd = dev(x)
+        (gpu.LayerOp.time_mix_v5 if version == "v5" else gpu.LayerOp.time_mix_v6)(cur, dev(w), dev(u), sd, dev(k), dev(v), dev(r), xd)
+        y = xd.cpu().numpy()
+    # f16 operands are the fixture's values exactly (they were drawn as f16); an f16 result carries its rounding
+    check_recurrence(version, y, sd.cpu().numpy(), 2e-3 if dtype == np.float16 else 5e-5, 5e-5)
