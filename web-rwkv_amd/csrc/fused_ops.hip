@@ -31,8 +31,33 @@ __global__ __launch_bounds__(kPreThreads) void v6_pre_kernel(const uint32_t *cur
                                                              uint16_t *shift1, uint32_t C) {
     __shared__ float red[kPreThreads / 64];
     const uint32_t t = blockIdx.x, nv = C / 4;
+    // Everything that does not depend on the row statistics is requested first: a workgroup is a chain of
+    // dependent memory round trips otherwise (cursor, row, weights after the reductions, state, factors),
+    // and at one token per launch that chain is the kernel's whole time.
+    uint2 wq[kPreCache], bq[kPreCache], fq[NS][kPreCache];
+#pragma unroll
+    for (int c = 0; c < kPreCache; c++) {
+        const uint32_t i = threadIdx.x + c * kPreThreads;
+        if (i < nv) {
+            wq[c] = *reinterpret_cast<const uint2 *>(ln_w + 4 * i);
+            bq[c] = *reinterpret_cast<const uint2 *>(ln_b + 4 * i);
+#pragma unroll
+            for (int s = 0; s < NS; s++) fq[s][c] = *reinterpret_cast<const uint2 *>((s == 0 ? factor0 : factor1) + 4 * i);
+        }
+    }
+    auto unpack = [](uint2 v) {
+        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
+    };
     const Cursor cur = read_cursor(cursors, t, vs);
     const bool first = t == cur.token;
+    float4 pst[kPreCache]; // the request's state row, for its first token of the stack
+    if (first) {
+#pragma unroll
+        for (int c = 0; c < kPreCache; c++) {
+            const uint32_t i = threadIdx.x + c * kPreThreads;
+            if (i < nv) pst[c] = load_vec4(state + view_elem(vs, cur.batch, 0, 4 * i));
+        }
+    }
     // rows t (which = 0) and t - 1 (which = 1): normalised, rounded to f16 as the op list stores them
     float4 ln[2][kPreCache];
 #pragma unroll
@@ -68,7 +93,7 @@ __global__ __launch_bounds__(kPreThreads) void v6_pre_kernel(const uint32_t *cur
         for (int c = 0; c < kPreCache; c++) {
             const uint32_t i = threadIdx.x + c * kPreThreads;
             if (i < nv) {
-                const float4 v = row[c], w = load_vec4(ln_w + 4 * i), b = load_vec4(ln_b + 4 * i);
+                const float4 v = row[c], w = unpack(wq[c]), b = unpack(bq[c]);
                 ln[which][c] = make_float4(round_h(fmaf((v.x - mean) * dev, w.x, b.x)), round_h(fmaf((v.y - mean) * dev, w.y, b.y)),
                                            round_h(fmaf((v.z - mean) * dev, w.z, b.z)), round_h(fmaf((v.w - mean) * dev, w.w, b.w)));
                 if (which == 0) store_vec4(ln_out + base + 4 * i, ln[0][c]);
@@ -79,12 +104,12 @@ __global__ __launch_bounds__(kPreThreads) void v6_pre_kernel(const uint32_t *cur
     for (int c = 0; c < kPreCache; c++) {
         const uint32_t i = threadIdx.x + c * kPreThreads;
         if (i >= nv) continue;
-        const float4 p = first ? load_vec4(state + view_elem(vs, cur.batch, 0, 4 * i)) : ln[1][c];
+        const float4 p = first ? pst[c] : ln[1][c];
         const float4 a = ln[0][c];
         auto mix = [](float xx, float pp, float f) { return xx * (1.0f - f) + pp * f; }; // reversed token shift: mix(x, prev, f)
 #pragma unroll
         for (int s = 0; s < NS; s++) {
-            const float4 f = load_vec4((s == 0 ? factor0 : factor1) + 4 * i);
+            const float4 f = unpack(fq[s][c]);
             store_vec4((s == 0 ? shift0 : shift1) + (uint64_t)t * C + 4 * i, make_float4(mix(a.x, p.x, f.x), mix(a.y, p.y, f.y), mix(a.z, p.z, f.z), mix(a.w, p.w, f.w)));
         }
     }
