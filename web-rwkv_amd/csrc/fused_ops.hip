@@ -122,26 +122,38 @@ __global__ __launch_bounds__(256) void v6_time_mix_kernel(const uint32_t *cursor
                                                           const float *state, ViewArgs vs, const uint16_t *att_x, uint16_t *out, uint32_t C, uint32_t A) {
     __shared__ __align__(16) uint16_t ls[5 * KL];
     const uint32_t t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
-    for (uint32_t e = threadIdx.x; e < 5 * KL / 8; e += 256) *reinterpret_cast<uint4 *>(&ls[8 * e]) = load128(lora + (uint64_t)t * 5 * KL + 8 * e);
-    __syncthreads();
-    if (c >= C) return;
+    const uint32_t cc = min(c, C - 1); // threads past the row repeat its last channel and store nothing
+    // every operand is requested before the first wait: the rows of w2, the mix vectors, the token and the
+    // one before it (the state row needs the cursor: one more round trip, for a request's first token only)
+    uint4 wv[5][KL / 8];
+    float tm[5];
+#pragma unroll
+    for (int s = 0; s < 5; s++) {
+        const uint16_t *wrow = w2 + ((uint64_t)s * C + cc) * KL;
+#pragma unroll
+        for (int k8 = 0; k8 < KL / 8; k8++) wv[s][k8] = load128(wrow + 8 * k8);
+        tm[s] = h2f(time_mix[(uint64_t)s * C + cc]);
+    }
     const Cursor cur = read_cursor(cursors, t, vs);
-    const float a = h2f(att_x[(uint64_t)t * C + c]);
-    const float p = t == cur.token ? state[view_elem(vs, cur.batch, 0, c)] : h2f(att_x[(uint64_t)(t - 1) * C + c]);
+    const float a = h2f(att_x[(uint64_t)t * C + cc]);
+    const float before = h2f(att_x[(uint64_t)(t ? t - 1 : 0) * C + cc]);
+    for (uint32_t e = threadIdx.x; e < 5 * KL / 8; e += 256) *reinterpret_cast<uint4 *>(&ls[8 * e]) = load128(lora + (uint64_t)t * 5 * KL + 8 * e);
+    const float p = t == cur.token ? state[view_elem(vs, cur.batch, 0, cc)] : before;
+    lds_barrier();
+    if (c >= C) return;
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int s = 0; s < 5; s++) {
-        const uint16_t *wrow = w2 + ((uint64_t)s * C + c) * KL;
         float acc = 0.0f;
 #pragma unroll
         for (int k8 = 0; k8 < KL / 8; k8++) {
-            const uint4 wv = load128(wrow + 8 * k8), xv = *reinterpret_cast<const uint4 *>(&ls[s * KL + 8 * k8]);
-            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.x), __builtin_bit_cast(h2, xv.x), acc, false);
-            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.y), __builtin_bit_cast(h2, xv.y), acc, false);
-            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.z), __builtin_bit_cast(h2, xv.z), acc, false);
-            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.w), __builtin_bit_cast(h2, xv.w), acc, false);
+            const uint4 xv = *reinterpret_cast<const uint4 *>(&ls[s * KL + 8 * k8]);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[s][k8].x), __builtin_bit_cast(h2, xv.x), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[s][k8].y), __builtin_bit_cast(h2, xv.y), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[s][k8].z), __builtin_bit_cast(h2, xv.z), acc, false);
+            acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[s][k8].w), __builtin_bit_cast(h2, xv.w), acc, false);
         }
-        const float f = round_h(round_h(acc) + h2f(time_mix[(uint64_t)s * C + c]));
+        const float f = round_h(round_h(acc) + tm[s]);
         out[((uint64_t)s * A + t) * C + c] = f2h(a * (1.0f - f) + p * f);
     }
 }
@@ -151,21 +163,27 @@ template <int KL>
 __global__ __launch_bounds__(256) void v6_decay_kernel(const uint16_t *lora, const uint16_t *w2, const uint16_t *time_decay, float *out, uint32_t C) {
     __shared__ __align__(16) uint16_t ls[KL];
     const uint32_t t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t cc = min(c, C - 1); // threads past the row repeat its last channel and store nothing
+    // the row of w2 and the bias are requested together with the token's vector, before the first wait
+    const uint16_t *wrow = w2 + (uint64_t)cc * KL;
+    uint4 wv[KL / 8];
+#pragma unroll
+    for (int k8 = 0; k8 < KL / 8; k8++) wv[k8] = load128(wrow + 8 * k8);
+    const float bias = h2f(time_decay[cc]);
     for (uint32_t e = threadIdx.x; e < KL / 8; e += 256) *reinterpret_cast<uint4 *>(&ls[8 * e]) = load128(lora + (uint64_t)t * KL + 8 * e);
-    __syncthreads();
+    lds_barrier();
     if (c >= C) return;
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const uint16_t *wrow = w2 + (uint64_t)c * KL;
     float acc = 0.0f;
 #pragma unroll
     for (int k8 = 0; k8 < KL / 8; k8++) {
-        const uint4 wv = load128(wrow + 8 * k8), xv = *reinterpret_cast<const uint4 *>(&ls[8 * k8]);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.x), __builtin_bit_cast(h2, xv.x), acc, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.y), __builtin_bit_cast(h2, xv.y), acc, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.z), __builtin_bit_cast(h2, xv.z), acc, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv.w), __builtin_bit_cast(h2, xv.w), acc, false);
+        const uint4 xv = *reinterpret_cast<const uint4 *>(&ls[8 * k8]);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[k8].x), __builtin_bit_cast(h2, xv.x), acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[k8].y), __builtin_bit_cast(h2, xv.y), acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[k8].z), __builtin_bit_cast(h2, xv.z), acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, wv[k8].w), __builtin_bit_cast(h2, xv.w), acc, false);
     }
-    out[(uint64_t)t * C + c] = act_one<WRQ_ACT_STABLE_EXP>(h2f(time_decay[c]) + acc);
+    out[(uint64_t)t * C + c] = act_one<WRQ_ACT_STABLE_EXP>(bias + acc);
 }
 
 // One wave per head of 64: lane i keeps the whole column S[.][i] of the request's state in registers;
