@@ -27,6 +27,20 @@ __global__ __launch_bounds__(THREADS) void row_kernel(XT *x, const uint16_t *w, 
     const uint32_t nv = n / 4;
     float4 cache[kRowCache];
     const bool cached = nv <= (uint32_t)(THREADS * kRowCache);
+    // a cached row asks for its weights together with the row: they are needed only after both reductions, and
+    // fetched then they would add a memory round trip to a kernel that is little more than round trips
+    uint2 wq[MODE == 0 ? 1 : kRowCache], bq[MODE == 0 ? 1 : kRowCache];
+    const uint16_t *wr = MODE == 2 ? w + (uint64_t)(blockIdx.x % heads) * n : w;
+    const uint16_t *br = MODE == 2 ? b + (uint64_t)(blockIdx.x % heads) * n : b;
+    if constexpr (MODE != 0) {
+        if (cached) {
+#pragma unroll
+            for (int c = 0; c < kRowCache; c++) {
+                const uint32_t i = threadIdx.x + c * THREADS;
+                if (i < nv) wq[c] = *reinterpret_cast<const uint2 *>(wr + 4 * i), bq[c] = *reinterpret_cast<const uint2 *>(br + 4 * i);
+            }
+        }
+    }
     // pass 1: the row into registers (or a first reading), maximum / sum
     float part = MODE == 0 ? -1.0e30f : 0.0f;
     if (cached) {
@@ -63,14 +77,15 @@ __global__ __launch_bounds__(THREADS) void row_kernel(XT *x, const uint16_t *w, 
     }
     const float total = block_reduce<false, THREADS>(acc, red);
     const float scale = MODE == 0 ? 1.0f / total : rsqrtf(total / (float)n + eps);
-    const uint16_t *wr = MODE == 2 ? w + (uint64_t)(blockIdx.x % heads) * n : w;
-    const uint16_t *br = MODE == 2 ? b + (uint64_t)(blockIdx.x % heads) * n : b;
-    auto finish = [&](uint32_t i, float4 v) {
+    auto unpack = [](uint2 v) {
+        return make_float4(h2f((uint16_t)(v.x & 0xffffu)), h2f((uint16_t)(v.x >> 16)), h2f((uint16_t)(v.y & 0xffffu)), h2f((uint16_t)(v.y >> 16)));
+    };
+    auto finish = [&](uint32_t i, float4 v, int c) { // c: the vector's place in the cache, or -1
         float4 o;
         if (MODE == 0) {
             o = make_float4(expf(v.x - centre) * scale, expf(v.y - centre) * scale, expf(v.z - centre) * scale, expf(v.w - centre) * scale);
         } else {
-            const float4 wv = load_vec4(wr + 4 * i), bv = load_vec4(br + 4 * i);
+            const float4 wv = c >= 0 ? unpack(wq[MODE == 0 ? 0 : c]) : load_vec4(wr + 4 * i), bv = c >= 0 ? unpack(bq[MODE == 0 ? 0 : c]) : load_vec4(br + 4 * i);
             o = make_float4(fmaf((v.x - centre) * scale, wv.x, bv.x), fmaf((v.y - centre) * scale, wv.y, bv.y),
                             fmaf((v.z - centre) * scale, wv.z, bv.z), fmaf((v.w - centre) * scale, wv.w, bv.w));
         }
@@ -80,10 +95,10 @@ __global__ __launch_bounds__(THREADS) void row_kernel(XT *x, const uint16_t *w, 
 #pragma unroll
         for (int c = 0; c < kRowCache; c++) {
             const uint32_t i = threadIdx.x + c * THREADS;
-            if (i < nv) finish(i, cache[c]);
+            if (i < nv) finish(i, cache[c], c);
         }
     } else {
-        for (uint32_t i = threadIdx.x; i < nv; i += THREADS) finish(i, load_vec4(row + 4 * i));
+        for (uint32_t i = threadIdx.x; i < nv; i += THREADS) finish(i, load_vec4(row + 4 * i), -1);
     }
 }
 
