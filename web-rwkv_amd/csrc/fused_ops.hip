@@ -260,10 +260,12 @@ __global__ __launch_bounds__(256) void v6_post_ffn_kernel(const uint32_t *cursor
                                                           const uint16_t *ffn_x, const uint16_t *x_in, uint16_t *x_out, uint32_t C, int rescale) {
     const uint32_t index = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
     if (index >= C / 4) return;
-    const Cursor cur = read_cursor(cursors, t, vs);
     const uint64_t bti = (uint64_t)t * C + 4 * index;
-    if (t - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = load_vec4(ffn_x + bti);
-    const float4 rr = load_vec4(r + bti), vv = load_vec4(v + bti), xx = load_vec4(x_in + bti);
+    // all loads before the store into the state: the compiler cannot move them across it (the pointers may
+    // alias), and behind it they would wait for the cursor's round trip first
+    const float4 rr = load_vec4(r + bti), vv = load_vec4(v + bti), xx = load_vec4(x_in + bti), fx = load_vec4(ffn_x + bti);
+    const Cursor cur = read_cursor(cursors, t, vs);
+    if (t - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = fx;
     const float sc = rescale ? 0.5f : 1.0f;
     auto f = [&](float a, float b, float c) { return round_h(round_h(1.0f / (1.0f + expf(-a)) * b) + c) * sc; };
     store_vec4(x_out + bti, make_float4(f(rr.x, vv.x, xx.x), f(rr.y, vv.y, xx.y), f(rr.z, vv.z, xx.z), f(rr.w, vv.w, xx.w)));

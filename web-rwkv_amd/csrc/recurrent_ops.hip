@@ -43,10 +43,11 @@ template <typename XT>
 __global__ __launch_bounds__(256) void channel_mix_kernel(const uint32_t *cursors, float *state, const XT *r, const XT *v, XT *x, ViewArgs vs, uint32_t C) {
     const uint32_t index = blockIdx.x * 256 + threadIdx.x, stack = blockIdx.y;
     if (index >= C / 4) return;
-    const Cursor cur = read_cursor(cursors, stack, vs);
     const uint64_t bti = (uint64_t)stack * C + 4 * index;
-    if (stack - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = load_vec4(x + bti);
-    const float4 rr = load_vec4(r + bti), vv = load_vec4(v + bti);
+    // all loads before the store into the state (the compiler cannot move them across it: the pointers may alias)
+    const float4 rr = load_vec4(r + bti), vv = load_vec4(v + bti), xx = load_vec4(x + bti);
+    const Cursor cur = read_cursor(cursors, stack, vs);
+    if (stack - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = xx;
     auto g = [](float a, float b) { return 1.0f / (1.0f + expf(-a)) * b; };
     store_vec4(x + bti, make_float4(g(rr.x, vv.x), g(rr.y, vv.y), g(rr.z, vv.z), g(rr.w, vv.w)));
 }

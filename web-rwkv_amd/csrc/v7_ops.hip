@@ -171,10 +171,11 @@ template <typename XT>
 __global__ __launch_bounds__(256) void channel_mix_v7_kernel(const uint32_t *cursors, float *state, const XT *v, XT *x, ViewArgs vs, uint32_t C) {
     const uint32_t index = blockIdx.x * 256 + threadIdx.x, stack = blockIdx.y;
     if (index >= C / 4) return;
-    const Cursor cur = read_cursor(cursors, stack, vs);
     const uint64_t bti = (uint64_t)stack * C + 4 * index;
-    if (stack - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = load_vec4(x + bti);
-    store_vec4(x + bti, load_vec4(v + bti));
+    const float4 vv = load_vec4(v + bti), xx = load_vec4(x + bti); // both before the cursor's round trip and the store into the state
+    const Cursor cur = read_cursor(cursors, stack, vs);
+    if (stack - cur.token + 1 == cur.len) *reinterpret_cast<float4 *>(state + view_elem(vs, cur.batch, 0, 4 * index)) = xx;
+    store_vec4(x + bti, vv);
 }
 
 int check_float(wrq_dtype dtype, const char *name) {
