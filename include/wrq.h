@@ -96,6 +96,16 @@ typedef void *wrq_stream;
  * capturing entry points into a HIP graph: first use otherwise does the same lookups. */
 int wrq_init(void);
 
+/*
+ * Test and sweep hook; no counterpart in the reference.  The library chooses kernels and tiles by
+ * shape.  An override pins one choice so that a test can reach every instantiation: keys are
+ * "gemm_ntile", "gemm_mrt", "gemm_kg", "gemm_ksplit", "gemv_rows", "gemv_nt", "gemv_oneshot",
+ * "vec_chunk_min_t", ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
+ * library first looks (wrq_init, or the first product) presets the same table; nothing on the launch
+ * path reads the environment.  Overrides are process-wide: not for use while other threads launch.
+ */
+int wrq_debug_override(const char *key, int value);
+
 int wrq_abi_version(void);
 const char *wrq_status_string(int status);
 const char *wrq_last_error(void);

@@ -36,3 +36,18 @@ def gpu(wrq):
     status = wrq.lib().wrq_init()
     assert status == 0, wrq.lib().wrq_last_error().decode()
     return wrq
+
+
+@pytest.fixture
+def overrides(wrq):
+    """Pins kernel / tile choices through wrq_debug_override for one test; released afterwards."""
+    used = set()
+
+    def pin(**kv):
+        for key, value in kv.items():
+            wrq.debug_override(key, value)
+            used.add(key)
+
+    yield pin
+    for key in used:
+        wrq.debug_override(key, -1)

@@ -302,24 +302,22 @@ TILE_VARIANTS = [(1, 1, 1), (1, 2, 1), (1, 4, 1), (1, 8, 1), (2, 1, 1), (2, 2, 1
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
 @pytest.mark.parametrize("mrt,ntile,kg", TILE_VARIANTS, ids=str)
-def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, kg, monkeypatch):
+def test_chunk_tile_variants(gpu, oracle, kind, mrt, ntile, kg, overrides):
     # every tile instantiation of the chunk kernel, with and without split K, on a shape that
     # leaves ragged edges everywhere: 5 steps of K (a partial stage, fewer steps than some k
-    # groups get), rows and tokens that do not fill the tiles.  WRQ_GEMM_* are the library's
-    # tuning overrides, read at every launch.
+    # groups get), rows and tokens that do not fill the tiles.  The tile is pinned through the
+    # library's test hook (wrq_debug_override).
     announce("chunk tile variant", kind, mrt, ntile, kg)
     K, R, T = 640, 200, 40
     rng = np.random.default_rng(SEED + 11 + mrt * 16 + ntile + 64 * kg)
-    monkeypatch.setenv("WRQ_GEMM_KG", str(kg))
     w = gen_f16(rng, (R, K), 0.02)
     x = gen_f16(rng, (T, K), 1.0)
     wp, scale, wdeq = pack(oracle, kind, w)
     m = gpu_matrix(gpu, kind, wp, scale)
     truth = truth_matmul(wdeq, x)
-    monkeypatch.setenv("WRQ_GEMM_MRT", str(mrt))
-    monkeypatch.setenv("WRQ_GEMM_NTILE", str(ntile))
+    overrides(gemm_kg=kg, gemm_mrt=mrt, gemm_ntile=ntile)
     for ksplit in (1, 2, 5):
-        monkeypatch.setenv("WRQ_GEMM_KSPLIT", str(ksplit))
+        overrides(gemm_ksplit=ksplit)
         for out_dtype in (np.float16, np.float32):
             got = run(gpu, m, x, R, "mat", out_dtype, act=1)
             assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"{kind} tile ({mrt},{ntile},{kg}) ksplit {ksplit}")

@@ -37,6 +37,7 @@ NF4_QUANT = [
 
 EXPORTS = [
     "wrq_init", "wrq_abi_version", "wrq_status_string", "wrq_last_error",
+    "wrq_debug_override",
     "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
     "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
@@ -177,6 +178,7 @@ def lib():
         L.wrq_status_string.restype = C.c_char_p
         L.wrq_status_string.argtypes = [i]
         L.wrq_last_error.restype = C.c_char_p
+        L.wrq_debug_override.argtypes = [C.c_char_p, i]
         L.wrq_quantize_mat_int8.argtypes = [vp, T, T, T]
         L.wrq_quantize_mat_nf4.argtypes = [vp, T, T, T, T]
         L.wrq_matmul_vec_int8.argtypes = [vp, T, T, V, V, i, i]
@@ -223,6 +225,11 @@ def lib():
             getattr(L, name).restype = i
         _lib = L
     return _lib
+
+
+def debug_override(key, value=-1):
+    """``wrq_debug_override``: pin (value >= 0) or release (value < 0) one kernel / tile choice."""
+    _check(lib().wrq_debug_override(key.encode(), int(value)))
 
 
 def _check(status):

@@ -48,8 +48,6 @@
 #include "wrq_device.h"
 #include "wrq_host.h"
 
-#include <stdlib.h>
-
 namespace wrq {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -645,11 +643,6 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, co
 
 namespace {
 
-int env_int(const char *name, int fallback) {
-    const char *s = getenv(name);
-    return (s && *s) ? atoi(s) : fallback;
-}
-
 float *scratch_ptr() {
     // the array's name is a host-side handle: resolve the device address once per device
     static float *ptr[64] = {};
@@ -782,14 +775,14 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
             split_for();
         }
     }
-    ntile = env_int("WRQ_GEMM_NTILE", ntile);
-    mrt = env_int("WRQ_GEMM_MRT", mrt);
-    kg = env_int("WRQ_GEMM_KG", kg);
+    ntile = tune(kTuneGemmNtile, ntile);
+    mrt = tune(kTuneGemmMrt, mrt);
+    kg = tune(kTuneGemmKg, kg);
     if (kg != 1 && kg != 2 && kg != 4) kg = 1;
     if (kg == 4 && (mrt != 1 || ntile > 2)) kg = 2;
     if (kg == 2 && ntile > 4) kg = 1;
-    if (getenv("WRQ_GEMM_NTILE") || getenv("WRQ_GEMM_MRT") || getenv("WRQ_GEMM_KG")) split_for();
-    ksplit = (uint32_t)env_int("WRQ_GEMM_KSPLIT", (int)ksplit);
+    if (tune_is_set(kTuneGemmNtile) || tune_is_set(kTuneGemmMrt) || tune_is_set(kTuneGemmKg)) split_for();
+    ksplit = (uint32_t)tune(kTuneGemmKsplit, (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
 #define WRQ_CASE(M, N, G) \

@@ -5,9 +5,13 @@
 
 #include <stdlib.h>
 
+#include <ctype.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+
+#include <atomic>
+#include <mutex>
 
 namespace wrq {
 
@@ -21,6 +25,46 @@ int fail(int status, const char *fmt, ...) {
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
     return status;
+}
+
+// ---- tuning overrides: read from the environment once, then only from this table
+namespace {
+const char *const kTuneNames[kTuneCount] = {"gemv_oneshot", "gemv_rows", "gemv_sl", "gemv_nt", "gemv_grid", "gemm_ntile", "gemm_mrt",
+                                            "gemm_kg", "gemm_ksplit", "vec_chunk_min_t", "nf4_wide", "exp0", "exp1", "exp2", "exp3"};
+std::atomic<int> g_tune[kTuneCount];
+std::once_flag g_tune_once;
+
+void tune_load_env() {
+    for (int k = 0; k < kTuneCount; k++) {
+        char name[64] = "WRQ_";
+        size_t n = 4;
+        for (const char *c = kTuneNames[k]; *c && n + 1 < sizeof(name); c++) name[n++] = (char)toupper((unsigned char)*c);
+        name[n] = 0;
+        const char *e = getenv(name);
+        g_tune[k].store((e && *e) ? atoi(e) : -1, std::memory_order_relaxed);
+    }
+}
+} // namespace
+
+int tune(TuneKey key, int fallback) {
+    std::call_once(g_tune_once, tune_load_env);
+    const int v = g_tune[key].load(std::memory_order_relaxed);
+    return v >= 0 ? v : fallback;
+}
+
+bool tune_is_set(TuneKey key) {
+    std::call_once(g_tune_once, tune_load_env);
+    return g_tune[key].load(std::memory_order_relaxed) >= 0;
+}
+
+int tune_set(const char *name, int value) {
+    std::call_once(g_tune_once, tune_load_env);
+    for (int k = 0; k < kTuneCount; k++)
+        if (strcmp(name, kTuneNames[k]) == 0) {
+            g_tune[k].store(value < 0 ? -1 : value, std::memory_order_relaxed);
+            return WRQ_OK;
+        }
+    return fail(WRQ_ERR_UNSUPPORTED, "unknown tuning key %s", name);
 }
 
 int check_launch(const char *what) {
@@ -183,12 +227,7 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     // activations share one pass of the one-shot VALU kernels (7B int8 step: 1.8 - 2.1 ms at 2 - 4
     // tokens against 2.8 ms; f16 head: 97 us at 4 tokens against 120); longer runs go to the
     // matrix-core kernel.
-    // WRQ_VEC_CHUNK_MIN_T overrides the first token count that does
-    static const int64_t chunk_min_env = [] {
-        const char *e = getenv("WRQ_VEC_CHUNK_MIN_T");
-        return (int64_t)((e && *e) ? atoi(e) : -1);
-    }();
-    const uint64_t chunk_min_t = chunk_min_env >= 0 ? (uint64_t)chunk_min_env : quant == kNf4 ? 3u : 5u;
+    const uint64_t chunk_min_t = (uint64_t)tune(kTuneVecChunkMinT, quant == kNf4 ? 3 : 5);
     // f32 activations are rounded to f16 by the matrix-core kernel: keep them on the exact VALU
     // kernels below 16 tokens
     const bool chunk = entry == kMat ? true : n >= (in_f16 ? chunk_min_t : (uint64_t)16);
@@ -262,7 +301,13 @@ const char *wrq_status_string(int status) {
     }
 }
 
+int wrq_debug_override(const char *key, int value) {
+    if (!key) return fail(WRQ_ERR_NULL, "null pointer: key");
+    return tune_set(key, value);
+}
+
 int wrq_init(void) {
+    (void)tune(kTuneGemvOneshot, 0); // reads the environment overrides now rather than at the first product
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));

@@ -36,6 +36,34 @@ int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a
 // The same for `n` independent products of one quantisation and input type: those with one K
 // and token count share a launch (and then rarely need a split of K).
 int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
+// Overrides of the kernel and tile choice, for tests and sweeps that must reach one particular
+// instantiation.  Every key is unset (-1) unless the environment variable of the same name (WRQ_ +
+// upper-case key) was set when the library first looked, or wrq_debug_override() set it since; the
+// launch path reads an atomic, never the environment.
+enum TuneKey {
+    kTuneGemvOneshot, // gemv_oneshot: 0 sends one-token products to the resident kernel
+    kTuneGemvRows,    // gemv_rows: rows per task of the decode kernels
+    kTuneGemvSl,      // gemv_sl: chunks per lane and row of the resident kernel
+    kTuneGemvNt,      // gemv_nt: lanes per task of the decode kernels
+    kTuneGemvGrid,    // gemv_grid: workgroups of the resident kernel
+    kTuneGemmNtile,   // gemm_ntile, gemm_mrt, gemm_kg, gemm_ksplit: tile of the chunk kernel
+    kTuneGemmMrt,
+    kTuneGemmKg,
+    kTuneGemmKsplit,
+    kTuneVecChunkMinT, // vec_chunk_min_t: first token count the decode entry sends to the chunk kernel
+    kTuneNf4Wide,      // nf4_wide: 0 keeps nf4 decode on the per-task table kernel
+    kTuneExp0,         // exp0 .. exp3: free knobs of experimental kernels
+    kTuneExp1,
+    kTuneExp2,
+    kTuneExp3,
+    kTuneCount
+};
+// The override of `key`, or `fallback` when it is unset.
+int tune(TuneKey key, int fallback);
+bool tune_is_set(TuneKey key);
+// Sets (value >= 0) or clears (value < 0) the override called `name`; unknown names fail.
+int tune_set(const char *name, int value);
+
 // Resolves the split-K scratch array of the current device (also done lazily by the first
 // chunk product; calling it from wrq_init keeps the lookup out of stream capture).
 int prepare_gemm_scratch();
