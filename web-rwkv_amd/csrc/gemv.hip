@@ -1093,7 +1093,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // K per row group, 512 / nt row groups of 4 or 8 rows.  Two such workgroups fit a CU: 8 rows per
         // group once 4 would need more than 512 workgroups
         auto wide_nt_of = [](uint32_t K) { const uint32_t c = K / 32; return c > 256 ? 512 : c > 128 ? 256 : c > 64 ? 128 : 64; };
-        const bool wide = oneshot && quant == kNf4 && T == 1 && tune(kTuneNf4Wide, 1) != 0;
+        const bool wide = oneshot && quant == kNf4 && T == 1 && tune(kTuneNf4Wide, 0) != 0;
         const int wide_nt = wide_nt_of(args[i].K);
         int wide_rows = 4;
         if (wide) {
