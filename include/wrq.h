@@ -193,6 +193,20 @@ int wrq_matmul_vec_nf4_group(wrq_stream stream, const wrq_vec_nf4_op *ops, int c
 int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
                         const wrq_tensor_view *input, const wrq_tensor_view *output, int act);
 
+/*
+ * wrq_matmul_mat_int8 for callers that cannot allocate or must know that nothing they call does:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference.  Same operands, checks and results as wrq_matmul_mat_int8 (the same kernels).
+ * When the product splits K over workgroups, the partial sums go to a fixed 16 MiB array that the
+ * library's code object holds on every GPU it runs on, used by this entry point only; its address on
+ * a device is looked up once (wrq_init, else the first call on that device).  A product whose
+ * partial sums would not fit is refused with WRQ_ERR_SIZE before anything is launched (the plain
+ * entry point takes fewer splits instead).  The array keeps nothing between calls and every call
+ * writes the part it reads, but calls that overlap in time on one GPU share it: they race.
+ */
+int wrq_matmul_mat_int8_noalloc(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
+                                const wrq_tensor_view *input, const wrq_tensor_view *output, int act);
+
 /* TensorOp::matmul_mat_nf4(matrix, quant, absmax, input, output, act)
  *                                                          src/tensor/ops.rs:1150-1221
  *   matrix: view `[K/2, R, B, 1]` of u8, whole parent; K a multiple of 64. */

@@ -39,7 +39,7 @@ EXPORTS = [
     "wrq_init", "wrq_abi_version", "wrq_status_string", "wrq_last_error",
     "wrq_debug_override",
     "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
-    "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4",
+    "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4", "wrq_matmul_mat_int8_noalloc",
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
     "wrq_matmul_vec_fp16", "wrq_matmul_mat_fp16",
     "wrq_softmax", "wrq_layer_norm", "wrq_group_norm", "wrq_add_activate", "wrq_mul_activate",
@@ -184,6 +184,7 @@ def lib():
         L.wrq_matmul_vec_int8.argtypes = [vp, T, T, V, V, i, i]
         L.wrq_matmul_vec_nf4.argtypes = [vp, T, T, T, V, V, i, i]
         L.wrq_matmul_mat_int8.argtypes = [vp, V, T, V, V, i]
+        L.wrq_matmul_mat_int8_noalloc.argtypes = [vp, V, T, V, V, i]
         L.wrq_matmul_mat_nf4.argtypes = [vp, V, T, T, V, V, i]
         L.wrq_matmul_vec_fp16.argtypes = [vp, T, V, V, i, i]
         L.wrq_matmul_mat_fp16.argtypes = [vp, V, V, V, i]
@@ -305,6 +306,11 @@ class TensorOp:
     def matmul_mat_int8(matrix, minmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
         _check(lib().wrq_matmul_mat_int8(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(minmax)),
                                          C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
+
+    @staticmethod
+    def matmul_mat_int8_noalloc(matrix, minmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):
+        _check(lib().wrq_matmul_mat_int8_noalloc(_stream(), C.byref(as_view(matrix, matrix_view, dtype=F16)), C.byref(as_tensor(minmax)),
+                                                 C.byref(as_view(input, input_view)), C.byref(as_view(output, output_view)), act))
 
     @staticmethod
     def matmul_mat_nf4(matrix, quant, absmax, input, output, act=ACT_NONE, matrix_view=None, input_view=None, output_view=None):

@@ -48,6 +48,8 @@
 #include "wrq_device.h"
 #include "wrq_host.h"
 
+#include <atomic>
+
 namespace wrq {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -70,6 +72,13 @@ constexpr int kUnrollStages = WRQ_UNROLL_STAGES; // even
 // calls on one stream cannot.  Nothing in it outlives a call.
 constexpr size_t kScratchFloats = 8u << 20; // 32 MiB: splits * R * T up to 8 Mi partial outputs
 __device__ __align__(256) float g_splitk_scratch[kScratchFloats];
+
+// The same for wrq_matmul_mat_int8_noalloc: a file-scope array of its own (16 MiB), so that the entry
+// point for callers that cannot allocate never shares partial sums with the other entry points.  In
+// host code the name is only a handle: the device address comes from hipGetSymbolAddress, once per
+// device (static_scratch_ptr), and only that pointer is ever handed to a kernel.
+constexpr size_t kStaticScratchFloats = 4u << 20;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     return (uint32_t)f2h(a) | ((uint32_t)f2h(b) << 16);
@@ -643,21 +652,37 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, co
 
 namespace {
 
-float *scratch_ptr() {
-    // the array's name is a host-side handle: resolve the device address once per device
-    static float *ptr[64] = {};
+constexpr int kMaxDevices = 64;
+
+// Device address of a __device__ array on the current device, looked up once per device (every GPU
+// holds its own copy at its own address).  Threads may race to the first lookup: both get the same
+// answer and the slot is an atomic.
+template <typename Lookup>
+float *device_array(std::atomic<float *> (&slots)[kMaxDevices], Lookup lookup) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    if (!ptr[dev]) {
-        void *p = nullptr;
-        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_splitk_scratch)) != hipSuccess) return nullptr;
-        ptr[dev] = static_cast<float *>(p);
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    float *p = slots[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void *q = nullptr;
+        if (lookup(&q) != hipSuccess || !q) return nullptr;
+        p = static_cast<float *>(q);
+        slots[dev].store(p, std::memory_order_release);
     }
-    return ptr[dev];
+    return p;
+}
+
+float *scratch_ptr() {
+    static std::atomic<float *> slots[kMaxDevices];
+    return device_array(slots, [](void **q) { return hipGetSymbolAddress(q, HIP_SYMBOL(g_splitk_scratch)); });
+}
+
+float *static_scratch_ptr() {
+    static std::atomic<float *> slots[kMaxDevices];
+    return device_array(slots, [](void **q) { return hipGetSymbolAddress(q, HIP_SYMBOL(scratch)); });
 }
 
 template <int QUANT, typename XT, int MRT, int NTILE, int KG>
-int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t ksplit) {
+int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t ksplit, const ScratchPolicy *sp) {
     using G = Geometry<MRT, NTILE, KG>;
     constexpr size_t lds = G::lds_bytes(QUANT);
     auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE, KG>;
@@ -686,18 +711,23 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
         slices += slice[i];
     }
     const uint32_t steps = a0.K / kStep;
-    // the partial tiles of all splits must fit the scratch array, whoever chose `ksplit`
-    while (ksplit > 1 && slices * ksplit > kScratchFloats) ksplit /= 2;
     if (ksplit > steps) ksplit = steps;
     if (ksplit < 1) ksplit = 1;
+    // the partial tiles of all splits must fit the scratch array, whoever chose `ksplit`: the shared
+    // array takes fewer splits then, the fixed one of the no-allocation entry point refuses
+    const uint64_t cap = sp ? sp->floats : kScratchFloats;
+    if (sp && sp->strict && ksplit > 1 && slices * ksplit > cap)
+        return fail(WRQ_ERR_SIZE, "split-K partial sums of this product need %llu bytes of scratch, the fixed array holds %llu",
+                    (unsigned long long)(slices * ksplit * sizeof(float)), (unsigned long long)(cap * sizeof(float)));
+    while (ksplit > 1 && slices * ksplit > cap) ksplit /= 2;
     const uint32_t steps_per = (steps + ksplit - 1) / ksplit;
     ga.k_per_split = steps_per * kStep;
     const uint32_t splits = (steps + steps_per - 1) / steps_per;
     if (splits > 1) {
-        float *base = scratch_ptr();
+        float *base = sp ? sp->base : scratch_ptr();
         if (!base) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
-        if (slices * splits > kScratchFloats)
-            return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slices * splits), (unsigned long long)kScratchFloats);
+        if (slices * splits > cap)
+            return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slices * splits), (unsigned long long)cap);
         uint64_t off = 0;
         for (int i = 0; i < n; i++) {
             ga.scratch[i] = base + off;
@@ -722,7 +752,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
 
 // `n` products with one K, token count and batch count (the caller groups them so).
 template <int QUANT, typename XT>
-int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
+int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const ScratchPolicy *sp) {
     // Tile choice, from sweeps over the launch shapes of this path (rows 4096 .. 65536, K 2048 ..
     // 14336, 5 .. 256 tokens, single products and groups).  A group counts as one product with the
     // rows of all its members.  Token tile: as narrow as the run up to 32 tokens; beyond that 64
@@ -786,31 +816,38 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n) {
     if (ksplit < 1) ksplit = 1;
 
 #define WRQ_CASE(M, N, G) \
-    if (mrt == M && ntile == N && kg == G) return launch_one<QUANT, XT, M, N, G>(stream, args, n, ksplit);
+    if (mrt == M && ntile == N && kg == G) return launch_one<QUANT, XT, M, N, G>(stream, args, n, ksplit, sp);
     WRQ_CASE(1, 1, 1) WRQ_CASE(1, 2, 1) WRQ_CASE(1, 4, 1) WRQ_CASE(1, 8, 1)
     WRQ_CASE(2, 1, 1) WRQ_CASE(2, 2, 1) WRQ_CASE(2, 4, 1) WRQ_CASE(2, 8, 1)
     WRQ_CASE(1, 1, 2) WRQ_CASE(1, 2, 2) WRQ_CASE(1, 4, 2)
     WRQ_CASE(2, 1, 2) WRQ_CASE(2, 2, 2) WRQ_CASE(2, 4, 2)
     WRQ_CASE(1, 1, 4) WRQ_CASE(1, 2, 4)
 #undef WRQ_CASE
-    return launch_one<QUANT, XT, 1, 2, 1>(stream, args, n, ksplit);
+    return launch_one<QUANT, XT, 1, 2, 1>(stream, args, n, ksplit, sp);
 }
 
 } // namespace
 
 int prepare_gemm_scratch() {
-    return scratch_ptr() ? WRQ_OK : fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+    return scratch_ptr() && static_scratch_ptr() ? WRQ_OK : fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+}
+
+int launch_gemm_noalloc(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
+    float *base = static_scratch_ptr(); // looked up by wrq_init, or here on the first call on this device
+    if (!base) return fail(WRQ_ERR_DEVICE, "fixed scratch array not resolvable");
+    const ScratchPolicy sp{base, kStaticScratchFloats, true};
+    return launch_gemm_group(stream, quant, in_f16, &a, 1, &sp);
 }
 
 // Preconditions (checked by the caller): K % 128 == 0, R % 4 == 0, 16-byte aligned
 // activation rows and output rows of 4.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {
-    return launch_gemm_group(stream, quant, in_f16, &a, 1);
+    return launch_gemm_group(stream, quant, in_f16, &a, 1, nullptr);
 }
 
 // `n` <= kMaxGroup independent products of one quantisation and input type; those that share K,
 // T and B = 1 go into one launch, the others are launched one by one.
-int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n) {
+int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n, const ScratchPolicy *sp) {
     int i = 0;
     while (i < n) {
         if (args[i].R == 0 || args[i].T == 0 || args[i].B == 0) {
@@ -824,11 +861,11 @@ int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 m++;
         int s;
         if (quant == kInt8)
-            s = in_f16 ? launch_shape<kInt8, __half>(stream, args + i, m) : launch_shape<kInt8, float>(stream, args + i, m);
+            s = in_f16 ? launch_shape<kInt8, __half>(stream, args + i, m, sp) : launch_shape<kInt8, float>(stream, args + i, m, sp);
         else if (quant == kFp16)
-            s = in_f16 ? launch_shape<kFp16, __half>(stream, args + i, m) : launch_shape<kFp16, float>(stream, args + i, m);
+            s = in_f16 ? launch_shape<kFp16, __half>(stream, args + i, m, sp) : launch_shape<kFp16, float>(stream, args + i, m, sp);
         else
-            s = in_f16 ? launch_shape<kNf4, __half>(stream, args + i, m) : launch_shape<kNf4, float>(stream, args + i, m);
+            s = in_f16 ? launch_shape<kNf4, __half>(stream, args + i, m, sp) : launch_shape<kNf4, float>(stream, args + i, m, sp);
         if (s != WRQ_OK) return s;
         i += m;
     }

@@ -240,17 +240,17 @@ int launch_vec(hipStream_t stream, Quant quant, const Prepared &p) {
     return quant == kFp16 ? launch_gemv_fp16(stream, p.in_f16, p.a) : launch_gemv(stream, quant, p.in_f16, p.a);
 }
 
-int launch_chunk(hipStream_t stream, Quant quant, const Prepared &p) {
+int launch_chunk(hipStream_t stream, Quant quant, const Prepared &p, bool noalloc) {
     if (p.a.K == 0) return launch_vec(stream, quant, p); // nothing to stream: plain zeros through the generic kernel
-    return launch_gemm(stream, quant, p.in_f16, p.a);
+    return noalloc ? launch_gemm_noalloc(stream, quant, p.in_f16, p.a) : launch_gemm(stream, quant, p.in_f16, p.a);
 }
 
 int matmul(hipStream_t stream, Entry entry, Quant quant, const void *w, const Shape4 &mshape,
            const wrq_tensor *scale, const wrq_tensor *table, const wrq_tensor_view *input,
-           const wrq_tensor_view *output, int act) {
+           const wrq_tensor_view *output, int act, bool noalloc = false) {
     Prepared p;
     WRQ_TRY(prepare(entry, quant, w, mshape, scale, table, input, output, act, p));
-    if (p.mfma) return launch_chunk(stream, quant, p);
+    if (p.mfma) return launch_chunk(stream, quant, p, noalloc);
     return launch_vec(stream, quant, p);
 }
 
@@ -424,6 +424,17 @@ int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const 
     if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
     return matmul(static_cast<hipStream_t>(stream), kMat, kInt8, matrix->data, shape_of(matrix->view.shape), minmax,
                   nullptr, input, output, act);
+}
+
+int wrq_matmul_mat_int8_noalloc(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
+                                const wrq_tensor_view *input, const wrq_tensor_view *output, int act) {
+    WRQ_TRY(need_view(matrix, "matrix", false));
+    WRQ_TRY(need_tensor(minmax, "minmax"));
+    WRQ_TRY(need_view(input, "input", true));
+    WRQ_TRY(need_view(output, "output", true));
+    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    return matmul(static_cast<hipStream_t>(stream), kMat, kInt8, matrix->data, shape_of(matrix->view.shape), minmax,
+                  nullptr, input, output, act, true);
 }
 
 int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *quant,

@@ -31,11 +31,20 @@ int launch_gemv(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a
 int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
 // Decode-shaped products on plain f16 weights (matmul_vec_fp16).
 int launch_gemv_fp16(hipStream_t stream, int in_f16, const MatmulArgs &args);
+// Where split-K partial sums go: null means the library's shared array, which takes fewer splits when
+// a product would not fit; `strict` refuses instead.
+struct ScratchPolicy {
+    float *base;
+    uint64_t floats;
+    bool strict;
+};
 // Chunk-shaped products: f16 MFMA.
 int launch_gemm(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
+// The same with the partial sums in the fixed array of the no-allocation entry point.
+int launch_gemm_noalloc(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &args);
 // The same for `n` independent products of one quantisation and input type: those with one K
 // and token count share a launch (and then rarely need a split of K).
-int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n);
+int launch_gemm_group(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs *args, int n, const ScratchPolicy *sp = nullptr);
 // Overrides of the kernel and tile choice, for tests and sweeps that must reach one particular
 // instantiation.  Every key is unset (-1) unless the environment variable of the same name (WRQ_ +
 // upper-case key) was set when the library first looked, or wrq_debug_override() set it since; the
