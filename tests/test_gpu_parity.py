@@ -34,7 +34,9 @@ def announce(*what):
 # ---------------------------------------------------------------- packing
 
 
-PACK_SHAPES = [(64, 320), (2048, 2560), (2048, 2048), (2048, 7168), (7168, 2048), (768, 2688), (3, 8, 512)]
+# (R, K): the reference's test shapes, the 1.6B operator-sweep shapes (head 2048 -> 65536 included), the 7B FFN shapes
+PACK_SHAPES = [(64, 320), (2048, 2560), (2048, 2048), (2048, 7168), (7168, 2048), (768, 2688), (3, 8, 512),
+               (65536, 2048), (14336, 4096), (4096, 14336)]
 
 
 def special_blocks(rng):
@@ -270,7 +272,8 @@ def test_multi_token_vec_entry(gpu, oracle, kind, T):
 # reference's own test shapes (ops.rs:3058-3059), and T below one MFMA tile
 GEMM = [(2048, 2048, 32), (2048, 2048, 128), (2048, 2048, 256), (2048, 7168, 32), (7168, 2048, 128),
         (4096, 4096, 128), (2560, 2048, 64), (320, 64, 320), (768, 2688, 32), (2688, 768, 32), (2048, 512, 4),
-        (2048, 512, 20), (2048, 65536, 32)]
+        (2048, 512, 20), (2048, 65536, 32),
+        (4096, 14336, 128), (14336, 4096, 128), (4096, 4096, 256), (14336, 4096, 256), (2048, 65536, 256)]
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
@@ -292,6 +295,98 @@ def test_gemm_against_truth(gpu, oracle, kind, K, R, T):
     if R * T * K <= 2048 * 2048 * 32:
         ofn = oracle.matmul_mat_int8 if kind == "int8" else oracle.matmul_mat_nf4
         assert_close(got, ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("K,R", SWEEP[:4], ids=str)
+def test_eight_tokens_on_the_vec_entry(gpu, oracle, kind, K, R):
+    # the operator sweep's 8 activation rows at the 1.6B shapes: T = 8 is no multiple of 32, so the model
+    # builders send it to the decode entry point (src/runtime/v6.rs:568-570)
+    announce("vec entry, 8 tokens", kind, K, R)
+    rng = np.random.default_rng(SEED + 8 + K * 3 + R)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = gen_f16(rng, (8, K), 1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    for out_dtype in (np.float16, np.float32):
+        assert_close(run(gpu, m, x, R, "vec", out_dtype), truth, EPS, f"{kind} {K}x{R} T=8 vs float64")
+    if R <= 7168:
+        ofn = oracle.matmul_vec_int8 if kind == "int8" else oracle.matmul_vec_nf4
+        assert_close(run(gpu, m, x, R, "vec", np.float32), ofn(wp, scale, x, out_dtype=np.float32)[0], EPS, "vs oracle")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("entry,T", [("mat", 32), ("mat", 128), ("vec", 16), ("vec", 40)])
+def test_f32_activations_that_are_no_f16_values(gpu, oracle, kind, entry, T):
+    # the reference's Bundle<f32> feeds f32 activations to f32 arithmetic (src/shaders/matmul_mat_int8.wgsl:106-132):
+    # random f32 inputs, rows that cancel included, at the longest K of the path, against float64
+    announce("f32 activations", kind, entry, T)
+    K, R = 14336, 512
+    rng = np.random.default_rng(SEED + 77 + T)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = rng.standard_normal((T, K), dtype=np.float32) * np.float32(1.0009765625)
+    x[1] = x[0] * np.float32(-0.99993896484375)  # token 1 nearly cancels token 0 when summed by a caller
+    assert (x.astype(np.float16).astype(np.float32) != x).mean() > 0.9
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    got = run(gpu, m, x, R, entry, np.float32)
+    assert_close(got, truth, EPS, f"{kind} {entry} T={T} f32 activations vs float64")
+    # weights whose products cancel: w and -w interleaved along K, so every output is a small difference of large sums
+    w2 = w.copy()
+    w2[:, 1::2] = -w2[:, 0::2]
+    x2 = x.copy()
+    x2[:, 1::2] = x2[:, 0::2] * np.float32(1.0001220703125)
+    wp2, scale2, wdeq2 = pack(oracle, kind, w2)
+    got2 = run(gpu, gpu_matrix(gpu, kind, wp2, scale2), x2, R, entry, np.float32)
+    assert_close(got2, truth_matmul(wdeq2, x2), EPS, f"{kind} {entry} T={T} cancelling sums")
+
+
+@pytest.mark.parametrize("kind", ["nf4", "int8"])
+def test_serving_schedule_run_lengths(gpu, oracle, kind):
+    # every distinct run length of the 32-slot serving schedule (prompts 16 .. 1024, chunk 256, 128 decode
+    # tokens per slot, cut by the RnnIter restatement in bench.py) on the products of a 7B-shape layer, with
+    # the kernel choice of the model builders (chunk kernels iff T % 32 == 0); a sample of rows of every
+    # product against float64
+    import torch
+
+    import bench
+
+    announce("serving schedule", kind)
+    rng = np.random.default_rng(SEED + 5)
+    slots, chunk, gen_len = 32, 256, 128
+    prompts = rng.integers(16, 1025, size=slots)
+    state = [[False, int(p)] for p in prompts]
+    to_gen = [gen_len] * slots
+    lengths = set()
+    while any(read > 0 for _, read in state):
+        lens = bench.rnn_iter_next(state, chunk)
+        T = sum(lens)
+        if T == 0:
+            break
+        lengths.add(T)
+        for i in range(slots):
+            state[i][0] = False
+            if lens[i] > 0 and state[i][1] == 0 and to_gen[i] > 0:
+                to_gen[i] -= 1
+                state[i][1] = 1 if to_gen[i] > 0 else 0
+    assert 256 in lengths and 32 in lengths and min(lengths) < 32
+    C, H = 4096, 14336
+    mats = []
+    for K, R in ((C, C), (C, H), (H, C)):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        rows = np.sort(rng.choice(R, 96, replace=False))
+        mats.append((K, R, gpu_matrix(gpu, kind, wp, scale), wdeq[rows], rows))
+    for T in sorted(lengths):
+        for K, R, m, wsub, rows in mats:
+            x = gen_f16(rng, (T, K), 1.0)
+            out = torch.full((T, R), float("nan"), dtype=torch.float16, device="cuda")
+            m.matmul_op(dev(x), out, turbo=gpu.turbo(T))
+            got = host(out)
+            assert np.isfinite(got).all(), f"{kind} T={T} {K}x{R}"
+            assert_close(got[:, rows], truth_matmul(wsub, x), EPS, f"{kind} T={T} {K}x{R} vs float64")
 
 
 # (MRT, NTILE, KG) instantiations of the chunk kernel: 64 * MRT / KG rows x 16 * NTILE tokens per
@@ -704,8 +799,7 @@ def test_random_shapes_all_routes(gpu, oracle, seed):
         if acts[act] in ("stable_exp", "opposite_exp", "softplus") and not np.isfinite(truth).all():
             continue
         got = run(gpu, m, x, R, entry, out_dtype, act=act)
-        eps = EPS if x_dtype == np.float16 or entry == "vec" else 4e-3
-        assert_close(got, truth, eps, f"{kind} K={K} R={R} T={T} {entry} act={acts[act]}")
+        assert_close(got, truth, EPS, f"{kind} K={K} R={R} T={T} {entry} act={acts[act]}")
 
 
 def test_entry_points_from_several_threads(gpu, oracle):

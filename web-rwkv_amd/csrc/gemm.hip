@@ -191,6 +191,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     constexpr int TPITCH = G::tpitch(QUANT);
     uint8_t *tslots = smem + (size_t)2 * BN * PITCH * sizeof(uint16_t) + (size_t)2 * KSUB * BM * sizeof(float2) +
                       (size_t)2 * KSUB * BN * sizeof(float) + (QUANT == kNf4 ? 256 * sizeof(uint2) : 0);
+    // f32 activations are split into two f16 tiles, x = hi + lo * 2^-11 (exact to 2^-22 of x, like the nf4 table
+    // values): every product term is then taken twice, against hi and against lo.  The lo tile sits behind the rest.
+    constexpr bool XLO = sizeof(XT) == 4;
+    uint16_t(*xsl)[BN * PITCH] = reinterpret_cast<uint16_t(*)[BN * PITCH]>(smem + G::lds_bytes(QUANT));
 
     uint32_t row_tile, tblock;
     tile_of_block(tile_id, ga.tblocks, row_tile, tblock);
@@ -256,6 +260,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // token and step sit in 16 adjacent lanes, one DPP row
     struct Stage {
         uint4 x[NPIECE];
+        uint4 xl[XLO ? NPIECE : 1]; // lo halves of f32 activations
         uint32_t sc[KSUB];
     };
     const XT *xp[NPIECE]; // (token, k_begin + 8 * (piece & 15)) of each piece
@@ -276,10 +281,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                 st.x[p] = load128(src);
             } else {
                 const uint4 v0 = load128(src), v1 = load128(src + 4);
-                st.x[p] = make_uint4(pack_h2(__uint_as_float(v0.x), __uint_as_float(v0.y)),
-                                     pack_h2(__uint_as_float(v0.z), __uint_as_float(v0.w)),
-                                     pack_h2(__uint_as_float(v1.x), __uint_as_float(v1.y)),
-                                     pack_h2(__uint_as_float(v1.z), __uint_as_float(v1.w)));
+                const float f[8] = {__uint_as_float(v0.x), __uint_as_float(v0.y), __uint_as_float(v0.z), __uint_as_float(v0.w),
+                                    __uint_as_float(v1.x), __uint_as_float(v1.y), __uint_as_float(v1.z), __uint_as_float(v1.w)};
+                float l[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) l[e] = (f[e] - h2f(f2h(f[e]))) * 2048.0f;
+                st.x[p] = make_uint4(pack_h2(f[0], f[1]), pack_h2(f[2], f[3]), pack_h2(f[4], f[5]), pack_h2(f[6], f[7]));
+                st.xl[XLO ? p : 0] = make_uint4(pack_h2(l[0], l[1]), pack_h2(l[2], l[3]), pack_h2(l[4], l[5]), pack_h2(l[6], l[7]));
             }
         }
         if constexpr (QUANT == kFp16) {
@@ -307,11 +315,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
             const uint32_t piece = tid + THREADS * p;
             const uint32_t tok = piece / (16 * KSUB), c = piece % (16 * KSUB);
             *reinterpret_cast<uint4 *>(&xs[buf][tok * PITCH + (c << 3)]) = st.x[p];
+            if constexpr (XLO) *reinterpret_cast<uint4 *>(&xsl[buf][tok * PITCH + (c << 3)]) = st.xl[p];
             if (QUANT == kInt8) {
                 float s = dot2_ones(st.x[p].x, 0.0f);
                 s = dot2_ones(st.x[p].y, s);
                 s = dot2_ones(st.x[p].z, s);
                 s = dot2_ones(st.x[p].w, s);
+                if constexpr (XLO) {
+                    float sl = dot2_ones(st.xl[p].x, 0.0f);
+                    sl = dot2_ones(st.xl[p].y, sl);
+                    sl = dot2_ones(st.xl[p].z, sl);
+                    sl = dot2_ones(st.xl[p].w, sl);
+                    s = fmaf(sl, 1.0f / 2048.0f, s);
+                }
                 s = row16_sum(s);
                 if ((tid & 15) == 0) sxs[buf][c >> 4][tok] = s;
             }
@@ -363,6 +379,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
         for (int n = 0; n < NTILE; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
     const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
+    // plain f16 weights against the lo halves of f32 activations: a second set of accumulators, added at the end
+    float4v outl[(XLO && QUANT == kFp16) ? MRT : 1][(XLO && QUANT == kFp16) ? NTILE : 1];
+    if constexpr (XLO && QUANT == kFp16) {
+#pragma unroll
+        for (int i = 0; i < MRT; i++)
+#pragma unroll
+            for (int n = 0; n < NTILE; n++) outl[i][n] = zero4;
+    }
 
     // lane offsets into the staged tile, the row scales and the token sums; the k group of the wave is
     // part of them, so that the step of a stage stays an immediate offset
@@ -400,25 +424,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         if constexpr (QUANT == kFp16) {
             // plain f16 weights are the A operands as loaded; the accumulators stay in the matrix cores
             const uint16_t *xh = xs[buf] + sub * kStep + xlane8;
+            const uint16_t *xlo = xsl[buf] + sub * kStep + xlane8;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
 #pragma unroll
                 for (int n = 0; n < NTILE; n++) {
-                    HalfPack B;
+                    HalfPack B, Bl;
                     const uint4 v = *reinterpret_cast<const uint4 *>(xh + n * 16 * PITCH + 32 * j);
                     B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
+                    if constexpr (XLO) {
+                        const uint4 vl = *reinterpret_cast<const uint4 *>(xlo + n * 16 * PITCH + 32 * j);
+                        Bl.u[0] = vl.x; Bl.u[1] = vl.y; Bl.u[2] = vl.z; Bl.u[3] = vl.w;
+                    }
 #pragma unroll
                     for (int i = 0; i < MRT; i++) {
                         HalfPack A;
                         const uint4 &wv = wa[i][j < NW ? j : 0];
                         A.u[0] = wv.x; A.u[1] = wv.y; A.u[2] = wv.z; A.u[3] = wv.w;
                         out[i][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.h, B.h, out[i][n], 0, 0, 0);
+                        if constexpr (XLO) outl[i][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A.h, Bl.h, outl[i][n], 0, 0, 0);
                     }
                 }
             }
             return;
         }
         const uint16_t *xt = xs[buf] + sub * kStep + xlane16;
+        const uint16_t *xtl = xsl[buf] + sub * kStep + xlane16;
         // scales of the 4 D-side rows of this lane, per row tile: (s, c) x 4 or (absmax0, absmax1) x 4
         float4 sc0[MRT], sc1[MRT];
 #pragma unroll
@@ -442,7 +473,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
             }
 #pragma unroll
             for (int n = 0; n < NTILE; n++) {
-                float4v D[MRT];
+                float4v D[MRT], Dx[MRT];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     HalfPack B;
@@ -450,6 +481,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                     B.u[0] = v.x; B.u[1] = v.y; B.u[2] = v.z; B.u[3] = v.w;
 #pragma unroll
                     for (int i = 0; i < MRT; i++) D[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, B.h, j == 0 ? zero4 : D[i], 0, 0, 0);
+                    if constexpr (XLO) {
+                        HalfPack Bl;
+                        const uint4 vl = *reinterpret_cast<const uint4 *>(xtl + n * 16 * PITCH + 64 * (j >> 1) + 8 * (j & 1));
+                        Bl.u[0] = vl.x; Bl.u[1] = vl.y; Bl.u[2] = vl.z; Bl.u[3] = vl.w;
+#pragma unroll
+                        for (int i = 0; i < MRT; i++) Dx[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i][j].h, Bl.h, j == 0 ? zero4 : Dx[i], 0, 0, 0);
+                    }
+                }
+                if constexpr (XLO) {
+#pragma unroll
+                    for (int i = 0; i < MRT; i++)
+#pragma unroll
+                        for (int d = 0; d < 4; d++) D[i][d] = fmaf(Dx[i][d], 1.0f / 2048.0f, D[i][d]);
                 }
                 const float sx = (&sxs[buf][sub][0])[sxs_lane + n * 16];
 #pragma unroll
@@ -489,6 +533,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                         for (int i = 0; i < MRT; i++) {
                             Dh[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[i][2 * blk + j].h, B.h, j == 0 ? zero4 : Dh[i], 0, 0, 0);
                             Dl[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[i][2 * blk + j].h, B.h, j == 0 ? zero4 : Dl[i], 0, 0, 0);
+                        }
+                        if constexpr (XLO) { // hi table values against the lo halves of the activations join the 2^-11 sum
+                            HalfPack Bl;
+                            const uint4 vl = *reinterpret_cast<const uint4 *>(xtl + n * 16 * PITCH + 64 * blk + 8 * j);
+                            Bl.u[0] = vl.x; Bl.u[1] = vl.y; Bl.u[2] = vl.z; Bl.u[3] = vl.w;
+#pragma unroll
+                            for (int i = 0; i < MRT; i++) Dl[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah[i][2 * blk + j].h, Bl.h, Dl[i], 0, 0, 0);
                         }
                     }
 #pragma unroll
@@ -544,6 +595,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
     }
 
+    if constexpr (XLO && QUANT == kFp16) {
+#pragma unroll
+        for (int i = 0; i < MRT; i++)
+#pragma unroll
+            for (int n = 0; n < NTILE; n++)
+#pragma unroll
+                for (int d = 0; d < 4; d++) out[i][n][d] = fmaf(outl[i][n][d], 1.0f / 2048.0f, out[i][n][d]);
+    }
     // add the partial tiles of the k groups through LDS (the activation buffers are free now)
     if constexpr (KG > 1) {
         float4 *red = reinterpret_cast<float4 *>(smem);
@@ -684,7 +743,7 @@ float *static_scratch_ptr() {
 template <int QUANT, typename XT, int MRT, int NTILE, int KG>
 int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t ksplit, const ScratchPolicy *sp) {
     using G = Geometry<MRT, NTILE, KG>;
-    constexpr size_t lds = G::lds_bytes(QUANT);
+    constexpr size_t lds = G::lds_bytes(QUANT) + (sizeof(XT) == 4 ? (size_t)2 * G::BN * G::PITCH * sizeof(uint16_t) : 0);
     auto *kern = &gemm_kernel<QUANT, XT, MRT, NTILE, KG>;
     if (lds > 48 * 1024) {
         // one-time opt-in to more than the default dynamic LDS limit
@@ -815,6 +874,13 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     ksplit = (uint32_t)tune(kTuneGemmKsplit, (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
+    if (sizeof(XT) == 4 && (ntile == 8 || (mrt == 2 && ntile == 4 && kg == 2))) {
+        // f32 activations keep a second (lo) activation tile and a second set of products: the widest tiles
+        // would not fit the registers, and 128 rows x 64 tokens x 2 k groups not the LDS
+        if (ntile == 8) ntile = 4;
+        if (mrt == 2 && ntile == 4) kg = 1;
+        split_for();
+    }
 #define WRQ_CASE(M, N, G) \
     if (mrt == M && ntile == N && kg == G) return launch_one<QUANT, XT, M, N, G>(stream, args, n, ksplit, sp);
     WRQ_CASE(1, 1, 1) WRQ_CASE(1, 2, 1) WRQ_CASE(1, 4, 1) WRQ_CASE(1, 8, 1)
