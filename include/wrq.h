@@ -187,7 +187,11 @@ int wrq_matmul_vec_nf4_group(wrq_stream stream, const wrq_vec_nf4_op *ops, int c
 /*
  * TensorOp::matmul_mat_int8(matrix, minmax, input, output, act)
  *                                                          src/tensor/ops.rs:1072-1140
- *   matrix: view of a u8 tensor, `[K, R, B, 1]`; it must cover its whole parent.
+ *   matrix: view of a u8 tensor, `[K, R, B, 1]`: the whole parent, or its leading batches.  The
+ *   reference sizes `minmax` by the view (ops.rs:1088-1090) but indexes it by the position in the
+ *   parent and steps rows by the view's width (src/shaders/matmul_mat_int8.wgsl:66-68, :99-103), so
+ *   any other slice has no consistent meaning there; it is refused with WRQ_ERR_UNSUPPORTED.  No
+ *   call site of the reference slices a matrix (src/tensor/matrix.rs:136-160 pass full views).
  *   R and T multiples of 4 (ops.rs:1068-1069), K a multiple of 32.
  */
 int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,
@@ -209,7 +213,7 @@ int wrq_matmul_mat_int8_noalloc(wrq_stream stream, const wrq_tensor_view *matrix
 
 /* TensorOp::matmul_mat_nf4(matrix, quant, absmax, input, output, act)
  *                                                          src/tensor/ops.rs:1150-1221
- *   matrix: view `[K/2, R, B, 1]` of u8, whole parent; K a multiple of 64. */
+ *   matrix: view `[K/2, R, B, 1]` of u8 (whole parent or leading batches, as above); K a multiple of 64. */
 int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *quant,
                        const wrq_tensor *absmax, const wrq_tensor_view *input,
                        const wrq_tensor_view *output, int act);
@@ -222,7 +226,7 @@ int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const w
  *   matrix f16 [K, R, B, 1]; input view [K, T, B, 1]; output view [R, T, B, 1]; K % 4 == 0.
  *   Up to 4 tokens share a pass over the weights on the decode kernel, more on the matrix-core kernel.
  * TensorOp::matmul_mat_fp16(matrix, input, output, act)           src/tensor/ops.rs:999-1061
- *   matrix: view of an f16 tensor covering its whole parent; K, R and T multiples of 4.
+ *   matrix: view of an f16 tensor (whole parent or leading batches); K, R and T multiples of 4.
  */
 int wrq_matmul_vec_fp16(wrq_stream stream, const wrq_tensor *matrix, const wrq_tensor_view *input,
                         const wrq_tensor_view *output, int act, int sparse);
@@ -384,7 +388,7 @@ int wrq_blend_lora(wrq_stream stream, const wrq_tensor *factor, const wrq_tensor
  * Buffers are contiguous device arrays of `Runtime<f16>` (v6.rs:270-303): C channels x A tokens.
  *
  * wrq_v6_pre: [add(add, x) ->] blit + layer_norm + token_shift x `shifts` (reversed)   v6.rs:759-777, :906-933
- *   x_out (f16, only with `add`, must differ from x) <- add + x;  ln_out <- LN(row);  shift_s <- mix(ln, previous, factor_s).
+ *   x_out (f16, only with `add`; its A * C elements may overlap neither x nor add) <- add + x;  ln_out <- LN(row);  shift_s <- mix(ln, previous, factor_s).
  * wrq_v6_time_mix: transpose + time_mix_w2 + add(time_mix) + token_shift(5)           v6.rs:785-805
  *   lora f16 [lora_size, 5, A]; w2 f16 [lora_size, C, 5]; time_mix f16 [C, 1, 5]; att_sx f16 [C, A, 5].
  * wrq_v6_decay: time_decay_w2 + add(time_decay) + activate(StableExp)                 v6.rs:839-848

@@ -116,10 +116,12 @@ class SafeTensors {
             js.header(entries_, metadata_);
             for (const auto &kv : entries_) {
                 const Entry &e = kv.second;
-                uint64_t len = 1;
-                for (uint64_t d : e.shape) len *= d;
                 if (e.end < e.begin || e.end > data_size_) throw LoaderError(kv.first + ": data offsets run past the file");
-                if ((e.end - e.begin) != len * dtype_size(e.dtype)) throw LoaderError(kv.first + ": data size does not fit shape and type");
+                // the header is untrusted: extents whose product wraps must not pass as a small tensor
+                uint64_t bytes = dtype_size(e.dtype);
+                bool wraps = false;
+                for (uint64_t d : e.shape) wraps |= __builtin_mul_overflow(bytes, d, &bytes);
+                if (wraps || (e.end - e.begin) != bytes) throw LoaderError(kv.first + ": data size does not fit shape and type");
             }
         } catch (...) {
             munmap(const_cast<uint8_t *>(base_), size_);

@@ -210,8 +210,14 @@ inline TensorBlob read_tensor(Reader &rd, size_t elem_size) {
     });
     if (!has_shape || !has_data) throw Error("TensorBlob: missing field `" + std::string(has_shape ? "data" : "shape") + "`");
     // TensorGpu::from_data_u8: the bytes must fill the shape
-    if (t.data.size() != t.shape.len() * elem_size)
-        throw Error("TensorBlob: data size not match: " + std::to_string(t.data.size()) + " vs. " + std::to_string(t.shape.len() * elem_size));
+    {
+        // extents come from the file: a product that wraps must not pass as a small tensor
+        uint64_t bytes = elem_size;
+        bool wraps = false;
+        for (int i = 0; i < 4; i++) wraps |= __builtin_mul_overflow(bytes, (uint64_t)t.shape[i], &bytes);
+        if (wraps || t.data.size() != bytes)
+            throw Error("TensorBlob: data size not match: " + std::to_string(t.data.size()) + " vs. " + (wraps ? std::string("more than 2^64") : std::to_string(bytes)));
+    }
     return t;
 }
 

@@ -382,6 +382,29 @@ static void test_layer_op_shape_errors() {
         if (!threw) std::printf("not refused: %s\n", kv.first);
         EXPECT(threw);
     }
+    // a state view without slots (or, for token_shift, without rows) leaves the cursors nothing to be clamped into
+    const auto no_slots = view_of(state, {{{0, C}, {0, S + 1}, {0, 0}, {0, 1}}}), no_slots_ffn = view_of(state, {{{0, C}, {S + 1, S + 2}, {0, 0}, {0, 1}}});
+    const auto no_rows = view_of(state, {{{0, C}, {0, 0}, {0, B}, {0, 1}}});
+    const auto mix = TensorGpuView<f16>(chan);
+    const std::pair<const char *, TensorOp> empty_state[] = {
+        {"token_shift", TensorOp::token_shift(cursors, mix, no_slots_ffn, flat, flat, false)},
+        {"token_shift", TensorOp::token_shift(cursors, mix, no_rows, flat, flat, false)},
+        {"channel_mix", TensorOp::channel_mix(cursors, no_slots_ffn, flat, flat, flat)},
+        {"channel_mix_v7", TensorOp::channel_mix_v7(cursors, no_slots_ffn, flat, flat)},
+        {"time_mix_v5", TensorOp::time_mix_v5(cursors, decay, decay, no_slots, heads32, heads32, heads32, heads32)},
+        {"time_mix_v6", TensorOp::time_mix_v6(cursors, decay_t, decay, no_slots, heads32, heads32, heads32, heads32)},
+        {"time_mix_v7", TensorOp::time_mix_v7(cursors, no_slots, heads, heads, n4, heads)},
+    };
+    for (const auto &kv : empty_state) {
+        bool threw = false;
+        try {
+            queue.submit(kv.second);
+        } catch (const TensorError &e) {
+            threw = e.status == WRQ_ERR_SHAPE && std::string(e.what()).find(kv.first) == 0;
+        }
+        if (!threw) std::printf("empty state not refused: %s\n", kv.first);
+        EXPECT(threw);
+    }
     (void)ffn;
 }
 
@@ -625,6 +648,13 @@ static void test_loader_host(const std::string &model_path, const std::string &d
     threw = false;
     try {
         SafeTensors cut(dir + "/cut.st"); // the same file without its last bytes
+    } catch (const LoaderError &) {
+        threw = true;
+    }
+    EXPECT(threw);
+    threw = false;
+    try {
+        SafeTensors wraps(dir + "/wraps.st"); // extents 2^31 x 2^31 x 4 of F16: the byte size wraps to 0 and would match offsets [0, 0]
     } catch (const LoaderError &) {
         threw = true;
     }

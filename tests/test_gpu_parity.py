@@ -511,6 +511,17 @@ def test_offset_views_f32_and_batch(gpu, oracle, kind):
     truth = np.stack([truth_matmul(wdq[b], xb[b]) for b in range(B)])
     assert_close(run(gpu, mb, xb, R, "vec", np.float32), truth, EPS, "batched vec")
     assert_close(run(gpu, mb, xb, R, "mat", np.float32), truth, EPS, "batched mat")
+    # a matrix view of the leading batches: the one kind of slice for which the reference's scale check (sized by the
+    # view) and scale indexing (by the position in the parent) agree
+    blocks = 2 * R * K // (64 if kind == "nf4" else 128) * (1 if kind == "nf4" else 2)
+    lead = gpu.Matrix(mb.kind, mb.w, mb.m[:blocks].contiguous(), mb.q)
+    out2 = torch.full((2, T, R), float("nan"), dtype=torch.float32, device="cuda")
+    kx = K // 2 if kind == "nf4" else K
+    lead.matmul_mat_op(dev(xb[:2]), out2, matrix_view=((kx, R, 2), (kx, R, B), (0, 0, 0)))
+    assert_close(host(out2), truth[:2], EPS, "leading batches of a matrix view")
+    with pytest.raises(gpu.TensorError) as e:
+        lead.matmul_mat_op(dev(xb[:2]), out2, matrix_view=((kx, R, 2), (kx, R, B), (0, 0, 1)))
+    assert e.value.status == gpu.ERR_UNSUPPORTED
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])

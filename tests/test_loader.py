@@ -28,6 +28,13 @@ def write_model(tmp_path, oracle):
         whole = f.read()
     with open(tmp_path / "cut.st", "wb") as f:
         f.write(whole[:-100])
+    # a header whose extents multiply to 2^65 bytes: in 64-bit arithmetic that is 0, the size of its data range
+    import json
+    import struct
+
+    header = json.dumps({"huge": {"dtype": "F16", "shape": [2 ** 31, 2 ** 31, 4], "data_offsets": [0, 0]}}).encode()
+    with open(tmp_path / "wraps.st", "wb") as f:
+        f.write(struct.pack("<Q", len(header)) + header)
     for name in ("blocks.6.att.output.weight", "blocks.6.ffn.value.weight"):
         for tag, d in ((".half.f16", 0.5), (".x03.f16", 0.3)):
             # Loader::load_matrix_f16_discount: f16::from_f32(discount * x.to_f32()), src/runtime/loader.rs:660-661

@@ -278,7 +278,7 @@ int check_ptr(const void *p, const char *what) {
 }
 
 int check_state(const wrq_tensor_view *state, uint32_t C, uint32_t rows, const char *what) {
-    const int s = check_layer_view(state, what);
+    const int s = check_state_view(state, what);
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: the state is f32", what);
     if (state->view.shape[0] != C || state->view.shape[1] != rows || state->view.shape[2] == 0 || state->view.shape[3] != 1)
@@ -309,7 +309,15 @@ int wrq_v6_pre(wrq_stream stream, uint32_t C, uint32_t A, const void *cursors, c
     if (s == WRQ_OK && shifts == 2) s = check_ptr(shift1, what);
     if (s == WRQ_OK && add) s = check_ptr(x_out, what);
     if (s != WRQ_OK) return s;
-    if (add && x_out == x) return fail(WRQ_ERR_UNSUPPORTED, "%s: the sum must go to another buffer (a token's workgroup reads its neighbour's row)", what);
+    if (add) {
+        // workgroup t rebuilds row t - 1 from x and add while workgroup t - 1 stores x_out: the sum may overlap neither
+        const uintptr_t lo = (uintptr_t)x_out, hi = lo + (size_t)A * C * 2;
+        for (const void *src : {x, add}) {
+            const uintptr_t a0 = (uintptr_t)src, a1 = a0 + (size_t)A * C * 2;
+            if (lo < a1 && a0 < hi)
+                return fail(WRQ_ERR_UNSUPPORTED, "%s: the sum must go to a buffer that overlaps neither input (a token's workgroup reads its neighbour's row)", what);
+        }
+    }
     const ViewArgs vs = view_args(state->view);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     auto u16 = [](const void *p) { return static_cast<const uint16_t *>(p); };

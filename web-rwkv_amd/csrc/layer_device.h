@@ -98,6 +98,17 @@ inline int check_layer_view(const wrq_tensor_view *t, const char *what) {
     return WRQ_OK;
 }
 
+// A state view: cursors address its slots (axis 2) and token_shift its row 0, and the kernels clamp both into
+// the view, so a view without slots or rows has nothing to clamp to and is refused.
+inline int check_state_view(const wrq_tensor_view *t, const char *what) {
+    const int s = check_layer_view(t, what);
+    if (s != WRQ_OK) return s;
+    if (t->view.shape[1] == 0 || t->view.shape[2] == 0)
+        return fail(WRQ_ERR_SHAPE, "%s: state view [%u, %u, %u, %u] has no rows or no slots", what, t->view.shape[0], t->view.shape[1], t->view.shape[2],
+                    t->view.shape[3]);
+    return WRQ_OK;
+}
+
 inline int check_layer_tensor(const wrq_tensor *t, const char *what) {
     if (!t || !t->data) return fail(WRQ_ERR_NULL, "%s: null tensor", what);
     if ((uintptr_t)t->data % 16) return fail(WRQ_ERR_ALIGNMENT, "%s: device pointers must be 16-byte aligned", what);

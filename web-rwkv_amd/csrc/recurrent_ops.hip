@@ -245,7 +245,7 @@ int wrq_token_shift(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
     if (s == WRQ_OK) s = check_layer_tensor(input, "token_shift");
     if (s == WRQ_OK) s = check_layer_tensor(output, "token_shift");
     if (s == WRQ_OK) s = check_layer_view(time_mix, "token_shift");
-    if (s == WRQ_OK) s = check_layer_view(state, "token_shift");
+    if (s == WRQ_OK) s = check_state_view(state, "token_shift");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "token_shift: the state is f32");
     for (int d : {(int)input_dtype, (int)output_dtype})
@@ -273,7 +273,7 @@ int wrq_channel_mix(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
     int s = check_layer_tensor(cursors, "channel_mix");
     for (const wrq_tensor *t : {r, v, x})
         if (s == WRQ_OK) s = check_layer_tensor(t, "channel_mix");
-    if (s == WRQ_OK) s = check_layer_view(state, "channel_mix");
+    if (s == WRQ_OK) s = check_state_view(state, "channel_mix");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: the state is f32");
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix: unsupported element type %d", (int)dtype);
@@ -308,7 +308,7 @@ int time_mix(const char *name, bool token_decay, wrq_stream stream, const wrq_te
     int s = check_layer_tensor(cursors, name);
     for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
         if (s == WRQ_OK) s = check_layer_tensor(t, name);
-    if (s == WRQ_OK) s = check_layer_view(state, name);
+    if (s == WRQ_OK) s = check_state_view(state, name);
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: the state is f32", name);
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "%s: unsupported element type %d", name, (int)dtype);
@@ -355,7 +355,7 @@ int wrq_time_mix_v4(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
     int s = check_layer_tensor(cursors, "time_mix_v4");
     for (const wrq_tensor *t : {time_decay, time_first, k, v, r, x})
         if (s == WRQ_OK) s = check_layer_tensor(t, "time_mix_v4");
-    if (s == WRQ_OK) s = check_layer_view(state, "time_mix_v4");
+    if (s == WRQ_OK) s = check_state_view(state, "time_mix_v4");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v4: the state is f32");
     if (dtype != WRQ_F16 && dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v4: unsupported element type %d", (int)dtype);

@@ -236,7 +236,7 @@ int wrq_time_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_tens
     int s = check_layer_tensor(cursors, "time_mix_v7");
     for (const wrq_tensor *t : {r, w, n, x})
         if (s == WRQ_OK) s = check_layer_tensor(t, "time_mix_v7");
-    if (s == WRQ_OK) s = check_layer_view(state, "time_mix_v7");
+    if (s == WRQ_OK) s = check_state_view(state, "time_mix_v7");
     if (s == WRQ_OK) s = check_float(dtype, "time_mix_v7");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "time_mix_v7: the state is f32");
@@ -296,7 +296,7 @@ int wrq_channel_mix_v7(wrq_stream stream, const wrq_tensor *cursors, const wrq_t
     int s = check_layer_tensor(cursors, "channel_mix_v7");
     for (const wrq_tensor *t : {v, x})
         if (s == WRQ_OK) s = check_layer_tensor(t, "channel_mix_v7");
-    if (s == WRQ_OK) s = check_layer_view(state, "channel_mix_v7");
+    if (s == WRQ_OK) s = check_state_view(state, "channel_mix_v7");
     if (s == WRQ_OK) s = check_float(dtype, "channel_mix_v7");
     if (s != WRQ_OK) return s;
     if (state->dtype != WRQ_F32) return fail(WRQ_ERR_TYPE, "channel_mix_v7: the state is f32");

@@ -125,10 +125,19 @@ int need_view(const wrq_tensor_view *v, const char *name, bool typed) {
     return WRQ_OK;
 }
 
-bool covers_parent(const wrq_view &v) {
+// Matrix views of the chunk products.  The reference sizes the scale tensor by the *view's* length
+// (src/tensor/ops.rs:1088-1090, :1166-1169) while its shader indexes the scales by the flat index in the
+// *parent* and steps from row to row by the view's width (src/shaders/matmul_mat_int8.wgsl:66-68, :99-103):
+// the two agree only for a view that starts at the origin and keeps whole rows and row counts, that is the
+// whole tensor or its leading batches.  Those are taken; any other slice has no consistent meaning there and
+// is refused.  The model builders pass `w.view(.., .., .., ..)` (src/tensor/matrix.rs:136-160).
+int check_matrix_view(const wrq_view &v) {
     for (int i = 0; i < 4; i++)
-        if (v.offset[i] != 0 || v.shape[i] != v.stride[i]) return false;
-    return true;
+        if (v.offset[i] != 0) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported: offset %u along axis %d", v.offset[i], i);
+    if (v.shape[0] != v.stride[0] || v.shape[1] != v.stride[1] || v.shape[3] != v.stride[3])
+        return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported: (%u, %u, %u, %u) of (%u, %u, %u, %u)", v.shape[0],
+                    v.shape[1], v.shape[2], v.shape[3], v.stride[0], v.stride[1], v.stride[2], v.stride[3]);
+    return WRQ_OK;
 }
 
 // Resolves views into element strides and offset pointers (compute_index of the
@@ -421,7 +430,7 @@ int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const 
     WRQ_TRY(need_tensor(minmax, "minmax"));
     WRQ_TRY(need_view(input, "input", true));
     WRQ_TRY(need_view(output, "output", true));
-    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    WRQ_TRY(check_matrix_view(matrix->view));
     return matmul(static_cast<hipStream_t>(stream), kMat, kInt8, matrix->data, shape_of(matrix->view.shape), minmax,
                   nullptr, input, output, act);
 }
@@ -432,7 +441,7 @@ int wrq_matmul_mat_int8_noalloc(wrq_stream stream, const wrq_tensor_view *matrix
     WRQ_TRY(need_tensor(minmax, "minmax"));
     WRQ_TRY(need_view(input, "input", true));
     WRQ_TRY(need_view(output, "output", true));
-    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    WRQ_TRY(check_matrix_view(matrix->view));
     return matmul(static_cast<hipStream_t>(stream), kMat, kInt8, matrix->data, shape_of(matrix->view.shape), minmax,
                   nullptr, input, output, act, true);
 }
@@ -445,7 +454,7 @@ int wrq_matmul_mat_nf4(wrq_stream stream, const wrq_tensor_view *matrix, const w
     WRQ_TRY(need_tensor(absmax, "absmax"));
     WRQ_TRY(need_view(input, "input", true));
     WRQ_TRY(need_view(output, "output", true));
-    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    WRQ_TRY(check_matrix_view(matrix->view));
     return matmul(static_cast<hipStream_t>(stream), kMat, kNf4, matrix->data, shape_of(matrix->view.shape), absmax,
                   quant, input, output, act);
 }
@@ -467,7 +476,7 @@ int wrq_matmul_mat_fp16(wrq_stream stream, const wrq_tensor_view *matrix, const 
     WRQ_TRY(need_view(matrix, "matrix", false));
     WRQ_TRY(need_view(input, "input", true));
     WRQ_TRY(need_view(output, "output", true));
-    if (!covers_parent(matrix->view)) return fail(WRQ_ERR_UNSUPPORTED, "sliced matrix views are not supported");
+    WRQ_TRY(check_matrix_view(matrix->view));
     return matmul(static_cast<hipStream_t>(stream), kMat, kFp16, matrix->data, shape_of(matrix->view.shape), nullptr,
                   nullptr, input, output, act);
 }
