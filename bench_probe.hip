@@ -1,5 +1,5 @@
-// Measurement probes, built into their own small library (libwrq_probe.so) and used only
-// by the benchmark: a streaming read and a plain copy of a known number of bytes.  They
+// Measurement probes of bench.py, built into their own small library (bench_probe.so beside this
+// file, by bench.py::build_probe): a streaming read and a plain copy of a known number of bytes.  They
 // give the read ceiling of the box that the product kernels are compared with, and the
 // reference dispatch against which rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled.
 #include <hip/hip_runtime.h>
