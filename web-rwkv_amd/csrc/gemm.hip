@@ -1103,7 +1103,7 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     for (int i = 0; i < n; i++) rows += args[i].R;
     if constexpr (QUANT == kInt8 && sizeof(XT) == 2) {
         // prefill chunks against many rows: the wide-tile kernel
-        if (a.B == 1 && T >= (uint32_t)tune(kTuneExp0, 96) && rows >= 4096 && steps >= 4 && tune(kTuneExp1, 1))
+        if (a.B == 1 && T >= (uint32_t)tune(kTuneExp0, 96) && rows >= 4096 && steps >= 4 && tune(kTuneExp1, 0))
             return launch_wide_int8<XT>(stream, args, n, sp);
     }
     const uint64_t rt = rows * a.B * T;
