@@ -667,224 +667,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     });
 }
 
-// Chunk products of many tokens (prefill chunks of 128 and 256): the wide-tile kernel.
-//
-// At 128 tokens and more the kernel above is bound by what crosses from L2 into a CU: with 64- or 128-row
-// tiles every workgroup pulls the activations of all its tokens, 2 bytes each, against 1 byte (int8) or half a
-// byte (nf4) per weight.  Here a workgroup of 8 waves owns 256 rows x 128 tokens x one K range: per weight
-// byte a quarter of the activation bytes of a 64-row tile, and K is split over workgroups until the grid
-// fills the CUs (partial tiles through the scratch array, summed by gemm_wide_finish_kernel).
-//   * a stage is one 128-block of K.  All 512 threads fetch it line-wise (a row's 128 codes, or a token's 128
-//     activations, in adjacent lanes) into registers one stage ahead; behind a barrier they write it to LDS as
-//     MFMA operands: the codes as exact f16 integers 1024 + u (one v_perm_b32 per two), the activations as they
-//     are; per-row (s, min - 1024 s) and per-token sums of the block go beside them.  Every weight is converted
-//     once per workgroup, not once per wave;
-//   * wave (rw, cw) of the 4 x 2 waves owns rows 64 rw .. + 64 and tokens 64 cw .. + 64: per 32-k slab 4 A and
-//     4 B operands from LDS feed 16 MFMAs (16x16x32), a quarter of an LDS read per MFMA;
-//   * D of a block starts from zero and joins the output with the block's scale: out += s D + (min - 1024 s) sum x.
-template <typename XT>
-__global__ __launch_bounds__(512) void gemm_wide_int8_kernel(const GemmArgs ga) {
-    constexpr int BM = 256, BN = 128, PITCH = kStep + 8; // f16 per LDS row: + 16 B rotates the banks
-    extern __shared__ __align__(16) uint8_t smem[];
-    uint16_t *As = reinterpret_cast<uint16_t *>(smem);                                // [BM][PITCH]
-    uint16_t *Bs = As + BM * PITCH;                                                   // [BN][PITCH]
-    float2 *scl = reinterpret_cast<float2 *>(Bs + BN * PITCH);                        // [BM]
-    float *sxs = reinterpret_cast<float *>(scl + BM);                                 // [BN]
-    uint32_t pi = 0;
-#pragma unroll
-    for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-        if (blockIdx.x >= ga.tile_begin[i]) pi = i;
-    pi = __builtin_amdgcn_readfirstlane(pi);
-    const MatmulArgs a = ga.m[pi];
-    const uint32_t tile_id = blockIdx.x - ga.tile_begin[pi];
-    float *const my_scratch = ga.scratch[pi];
-    const uint32_t row_tile = tile_id / ga.tblocks, tblock = tile_id % ga.tblocks;
-    const uint32_t tid = threadIdx.x, lane = tid & 63;
-    const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t rw = wv & 3, cw = wv >> 2;
-    const uint32_t r16 = lane & 15, g = lane >> 4;
-    const uint32_t K = a.K, t0 = tblock * BN, row0 = row_tile * BM;
-    const uint32_t k_begin = blockIdx.y * ga.k_per_split;
-    const uint32_t k_end = min(K, k_begin + ga.k_per_split);
-    const uint32_t nsteps = (k_end - k_begin) / kStep;
-
-    // fetch roles: weight piece (row 64 i + tid / 8, bytes 16 (tid & 7) ..), activation piece (token 32 j + tid / 16,
-    // elements 8 (tid & 15) ..), scale word of row tid
-    const uint8_t *wp[4];
-    const XT *xp[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t row = min(row0 + 64 * i + (tid >> 3), a.R - 1);
-        wp[i] = a.w + (uint64_t)row * K + k_begin + 16 * (tid & 7);
-        const uint32_t tok = min(t0 + 32 * i + (tid >> 4), a.T - 1);
-        xp[i] = reinterpret_cast<const XT *>(a.x) + (uint64_t)tok * a.x_token_stride + k_begin + 8 * (tid & 15);
-    }
-    const uint32_t *sp = reinterpret_cast<const uint32_t *>(a.scale) + (((uint64_t)min(row0 + min(tid, (uint32_t)BM - 1), a.R - 1) * K + k_begin) >> 7);
-
-    struct Fetch {
-        uint4 w[4], x[4];
-        uint32_t sc;
-    };
-    auto fetch = [&](uint32_t step, Fetch &f) {
-        const uint32_t st = min(step, nsteps - 1); // steps past the range repeat the last one (not used)
-#pragma unroll
-        for (int i = 0; i < 4; i++) f.w[i] = load128_stream(wp[i] + st * kStep);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const XT *src = xp[i] + st * kStep;
-            if constexpr (sizeof(XT) == 2) {
-                f.x[i] = load128(src);
-            } else {
-                const uint4 v0 = load128(src), v1 = load128(src + 4);
-                f.x[i] = make_uint4(pack_h2(__uint_as_float(v0.x), __uint_as_float(v0.y)), pack_h2(__uint_as_float(v0.z), __uint_as_float(v0.w)),
-                                    pack_h2(__uint_as_float(v1.x), __uint_as_float(v1.y)), pack_h2(__uint_as_float(v1.z), __uint_as_float(v1.w)));
-            }
-        }
-        f.sc = sp[st];
-    };
-    auto stage = [&](const Fetch &f) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t w[4] = {f.w[i].x, f.w[i].y, f.w[i].z, f.w[i].w};
-            uint32_t c[8];
-#pragma unroll
-            for (int d = 0; d < 4; d++) {
-                c[2 * d] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04010400u);
-                c[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, w[d], 0x04030402u);
-            }
-            uint16_t *dst = As + (64 * i + (tid >> 3)) * PITCH + 16 * (tid & 7);
-            *reinterpret_cast<uint4 *>(dst) = make_uint4(c[0], c[1], c[2], c[3]);
-            *reinterpret_cast<uint4 *>(dst + 8) = make_uint4(c[4], c[5], c[6], c[7]);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t tok = 32 * i + (tid >> 4);
-            *reinterpret_cast<uint4 *>(Bs + tok * PITCH + 8 * (tid & 15)) = f.x[i];
-            float s = dot2_ones(f.x[i].x, 0.0f);
-            s = dot2_ones(f.x[i].y, s);
-            s = dot2_ones(f.x[i].z, s);
-            s = dot2_ones(f.x[i].w, s);
-            s = row16_sum(s);
-            if ((tid & 15) == 0) sxs[tok] = s;
-        }
-        if (tid < BM) {
-            const float lo = h2f((uint16_t)(f.sc & 0xffffu)), hi = h2f((uint16_t)(f.sc >> 16));
-            const float sc = (hi - lo) * (1.0f / 255.0f);
-            scl[tid] = make_float2(sc, fmaf(-1024.0f, sc, lo));
-        }
-    };
-
-    float4v out[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int n = 0; n < 4; n++) out[i][n] = float4v{0.f, 0.f, 0.f, 0.f};
-    const float4v zero4 = float4v{0.f, 0.f, 0.f, 0.f};
-    const uint16_t *arow = As + (64 * rw + r16) * PITCH + 8 * g;
-    const uint16_t *brow = Bs + (64 * cw + r16) * PITCH + 8 * g;
-
-    Fetch f;
-    fetch(0, f);
-    for (uint32_t s = 0; s < nsteps; s++) {
-        lds_barrier(); // the previous stage has been read by every wave
-        stage(f);
-        fetch(s + 1, f);
-        lds_barrier();
-        float4v D[4][4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            HalfPack A[4], B[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(arow + 16 * i * PITCH + 32 * q);
-                A[i].u[0] = v.x; A[i].u[1] = v.y; A[i].u[2] = v.z; A[i].u[3] = v.w;
-            }
-#pragma unroll
-            for (int n = 0; n < 4; n++) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(brow + 16 * n * PITCH + 32 * q);
-                B[n].u[0] = v.x; B[n].u[1] = v.y; B[n].u[2] = v.z; B[n].u[3] = v.w;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int n = 0; n < 4; n++) D[i][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i].h, B[n].h, q == 0 ? zero4 : D[i][n], 0, 0, 0);
-        }
-        float sx[4];
-#pragma unroll
-        for (int n = 0; n < 4; n++) sx[n] = sxs[64 * cw + 16 * n + r16];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float4 *q = reinterpret_cast<const float4 *>(scl + 64 * rw + 16 * i + 4 * g);
-            const float4 s01 = q[0], s23 = q[1]; // (s, c) of rows 4 g .. 4 g + 3 of the tile
-#pragma unroll
-            for (int n = 0; n < 4; n++) {
-                out[i][n][0] = fmaf(s01.x, D[i][n][0], fmaf(s01.y, sx[n], out[i][n][0]));
-                out[i][n][1] = fmaf(s01.z, D[i][n][1], fmaf(s01.w, sx[n], out[i][n][1]));
-                out[i][n][2] = fmaf(s23.x, D[i][n][2], fmaf(s23.y, sx[n], out[i][n][2]));
-                out[i][n][3] = fmaf(s23.z, D[i][n][3], fmaf(s23.w, sx[n], out[i][n][3]));
-            }
-        }
-    }
-
-    if (my_scratch) {
-        // partial tile of this split: [split][tile][wave][i][n][lane][4], 1 KiB per store instruction
-        float *dst = my_scratch + ((((uint64_t)blockIdx.y * ga.row_tiles[pi] * ga.tblocks + tile_id) * 8 + wv) * 16) * 256 + lane * 4;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int n = 0; n < 4; n++)
-                *reinterpret_cast<float4 *>(dst + (i * 4 + n) * 256) = make_float4(out[i][n][0], out[i][n][1], out[i][n][2], out[i][n][3]);
-        return;
-    }
-    act_dispatch(a.act, [&](auto act_tag) {
-        constexpr int ACT = decltype(act_tag)::value;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t orow = row0 + 64 * rw + 16 * i + 4 * g;
-#pragma unroll
-            for (int n = 0; n < 4; n++) {
-                const uint32_t t = t0 + 64 * cw + 16 * n + r16;
-                if (t < a.T && orow < a.R) {
-                    const uint64_t idx = (uint64_t)t * a.out_token_stride + orow;
-                    float v[4];
-#pragma unroll
-                    for (int d = 0; d < 4; d++) v[d] = act_one<ACT>(out[i][n][d]);
-                    if (a.out_f16)
-                        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
-                    else
-                        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
-                }
-            }
-        }
-    });
-}
-
-// Sum of the partial tiles of gemm_wide_int8_kernel over the splits, activation, output type: one thread per
-// lane slot of a tile, in the order the tiles were stored.
-__global__ __launch_bounds__(256) void gemm_wide_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits, uint32_t tiles, uint32_t tblocks) {
-    const uint64_t slots = (uint64_t)tiles * 8 * 16 * 64;
-    const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (q >= slots) return;
-    const uint32_t lane = (uint32_t)(q & 63), r16 = lane & 15, g = lane >> 4;
-    const uint32_t in = (uint32_t)((q >> 6) & 15), wv = (uint32_t)((q >> 10) & 7);
-    const uint32_t tile = (uint32_t)(q >> 13);
-    const uint32_t i = in >> 2, n = in & 3, rw = wv & 3, cw = wv >> 2;
-    const uint32_t row = (tile / tblocks) * 256 + 64 * rw + 16 * i + 4 * g;
-    const uint32_t t = (tile % tblocks) * 128 + 64 * cw + 16 * n + r16;
-    if (t >= a.T || row >= a.R) return;
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t k = 0; k < splits; k++) {
-        const float4 v = *reinterpret_cast<const float4 *>(scratch + (k * slots + q) * 4);
-        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
-    }
-    const float v[4] = {act_apply(a.act, s.x), act_apply(a.act, s.y), act_apply(a.act, s.z), act_apply(a.act, s.w)};
-    const uint64_t idx = (uint64_t)t * a.out_token_stride + row;
-    if (a.out_f16)
-        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + idx) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
-    else
-        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + idx) = make_float4(v[0], v[1], v[2], v[3]);
-}
-
 // Second half of a split-K product: sum of the partial tiles over the splits, activation,
 // output type.  One thread per lane slot of the first kernel's tiles (same decoding).
 __global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits, uint32_t nwg,
@@ -1028,66 +810,6 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     return s;
 }
 
-
-// Wide tiles: 256 rows x 128 tokens per workgroup, K split over the grid until it fills the CUs.
-template <typename XT>
-int launch_wide_int8(hipStream_t stream, const MatmulArgs *args, int n, const ScratchPolicy *sp) {
-    constexpr uint32_t BM = 256, BN = 128;
-    constexpr size_t lds = (size_t)(BM + BN) * (kStep + 8) * sizeof(uint16_t) + BM * sizeof(float2) + BN * sizeof(float);
-    auto *kern = &gemm_wide_int8_kernel<XT>;
-    static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    (void)once;
-    GemmArgs ga;
-    const MatmulArgs &a0 = args[0];
-    ga.tblocks = (a0.T + BN - 1) / BN;
-    uint32_t total = 0;
-    uint64_t slice[kMaxGroup], slices = 0; // partial-tile floats of one split, per product
-    for (int i = 0; i < kMaxGroup; i++) {
-        ga.tile_begin[i] = 0xffffffffu;
-        ga.row_tiles[i] = 0;
-        ga.scratch[i] = nullptr;
-        if (i >= n) continue;
-        ga.m[i] = args[i];
-        ga.row_tiles[i] = (args[i].R + BM - 1) / BM;
-        ga.tile_begin[i] = total;
-        total += ga.row_tiles[i] * ga.tblocks;
-        slice[i] = (uint64_t)ga.row_tiles[i] * ga.tblocks * BM * BN;
-        slices += slice[i];
-    }
-    const uint32_t steps = a0.K / kStep;
-    uint32_t ksplit = (uint32_t)tune(kTuneGemmKsplit, (int)std::max(1u, std::min(8u, 256u / std::max(total, 1u))));
-    ksplit = std::max(1u, std::min(ksplit, steps / 2 ? steps / 2 : 1u)); // at least two steps per split
-    const uint64_t cap = sp ? sp->floats : kScratchFloats;
-    if (sp && sp->strict && ksplit > 1 && slices * ksplit > cap)
-        return fail(WRQ_ERR_SIZE, "split-K partial sums of this product need %llu bytes of scratch, the fixed array holds %llu",
-                    (unsigned long long)(slices * ksplit * sizeof(float)), (unsigned long long)(cap * sizeof(float)));
-    while (ksplit > 1 && slices * ksplit > cap) ksplit--;
-    const uint32_t steps_per = (steps + ksplit - 1) / ksplit;
-    ga.k_per_split = steps_per * kStep;
-    const uint32_t splits = (steps + steps_per - 1) / steps_per;
-    if (splits > 1) {
-        float *base = sp ? sp->base : scratch_ptr();
-        if (!base) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
-        uint64_t off = 0;
-        for (int i = 0; i < n; i++) {
-            ga.scratch[i] = base + off;
-            off += slice[i] * splits;
-        }
-    }
-    hipLaunchKernelGGL(kern, dim3(total, splits), dim3(512), lds, stream, ga);
-    int s = check_launch("matmul_mat (wide)");
-    if (s != WRQ_OK) return s;
-    if (splits > 1) {
-        for (int i = 0; i < n; i++) {
-            const uint32_t tiles = ga.row_tiles[i] * ga.tblocks;
-            const uint64_t slots = (uint64_t)tiles * 8 * 16 * 64;
-            hipLaunchKernelGGL(gemm_wide_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, args[i], ga.scratch[i], splits, tiles, ga.tblocks);
-        }
-        s = check_launch("matmul_mat (wide, finish)");
-    }
-    return s;
-}
-
 // `n` products with one K, token count and batch count (the caller groups them so).
 template <int QUANT, typename XT>
 int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const ScratchPolicy *sp) {
@@ -1101,11 +823,6 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     const uint32_t steps = a.K / kStep;
     uint64_t rows = 0;
     for (int i = 0; i < n; i++) rows += args[i].R;
-    if constexpr (QUANT == kInt8 && sizeof(XT) == 2) {
-        // prefill chunks against many rows: the wide-tile kernel
-        if (a.B == 1 && T >= (uint32_t)tune(kTuneExp0, 96) && rows >= 4096 && steps >= 4 && tune(kTuneExp1, 0))
-            return launch_wide_int8<XT>(stream, args, n, sp);
-    }
     const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
     // long rows against 256 tokens and more also take the 128-token tile (measured on 4096 x 14336: 7 % faster)

@@ -608,152 +608,6 @@ __global__ __launch_bounds__(NT) void gemv_nf4_oneshot_kernel(const GemvGroup g)
     oneshot_reduce_store<ROWS, NT, TT>(acc, red, p, row0, g.T);
 }
 
-// nf4, one token, wide workgroups.  Counters of the kernel above show what bounds it: two thirds of
-// its LDS cycles are bank conflicts (64 lanes gather random entries of one 2 KiB table), and the LDS
-// is its busiest unit.  Here the byte table has one copy per lane & 31: entry v of copy c lives at
-// byte v * 256 + c * 8, so the 32 lanes that the LDS serves together always read 32 different banks
-// pairs, and one v_perm_b32 builds the address (table byte -> address byte 1, lane offset -> byte 0).
-// The table is 64 KiB; a workgroup of NT * RG threads (RG row groups of ROWS rows, NT lanes along K
-// each) shares it, so that building it (8192 entries) is a small part of the workgroup's life.
-// A workgroup never spans two products: each product brings its own table.
-template <typename XT, int ROWS, int NT, int RG, bool SINGLE>
-__global__ __launch_bounds__(NT *RG) void gemv_nf4_wide_kernel(const GemvGroup g) {
-    constexpr int NTHREADS = NT * RG;
-    constexpr int NROW16 = NT / 16; // DPP rows per row group
-    constexpr bool F16 = sizeof(XT) == 2;
-    extern __shared__ __align__(16) uint8_t smem[];
-    uint2 *tab = reinterpret_cast<uint2 *>(smem); // [256][32]
-    float(*red)[ROWS][NROW16] = reinterpret_cast<float(*)[ROWS][NROW16]>(smem + 256 * 32 * sizeof(uint2));
-    const uint32_t tid = threadIdx.x;
-    const uint32_t grp = RG == 1 ? 0u : __builtin_amdgcn_readfirstlane(tid / NT); // NT is a multiple of 64
-    const uint32_t gl = tid % NT;                                                 // lane inside the row group
-    const uint32_t wg = blockIdx.x;
-    uint32_t pi = 0;
-    if constexpr (!SINGLE) {
-#pragma unroll
-        for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-            if (wg >= g.task_begin[i]) pi = i;
-        pi = __builtin_amdgcn_readfirstlane(pi);
-    }
-    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
-    const uint32_t K = p.K, nchunk = K >> 5;
-    const uint32_t row0 = ((wg - p.task_begin) * RG + grp) * ROWS;
-    const bool have_rows = row0 < p.R;
-    const uint32_t rows_valid = have_rows ? min((uint32_t)ROWS, p.R - row0) : 1u;
-    const uint32_t rbase = have_rows ? row0 : 0u; // idle row groups repeat rows 0 .. and drop the result
-    const uint64_t e0 = p.e_base + (uint64_t)rbase * K;
-    const uint8_t *wbase = p.w + (((uint64_t)rbase * K) >> 1);
-    const XT *x = reinterpret_cast<const XT *>(p.x);
-
-    float acc[ROWS];
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) acc[r] = 0.0f;
-
-    // table values behind this thread's slots: slot e = v * 32 + copy for e = tid + 512 i, so v & 15 is
-    // (tid >> 5) & 15 for all 16 slots of a thread and v >> 4 is i: one value per thread and the 16
-    // values as uniform (scalar) loads, requested before anything else
-    static_assert(NTHREADS == 512, "the slot numbering of the table build assumes 512 threads");
-    const float q0 = p.quant[(tid >> 5) & 15u];
-    float q[16];
-#pragma unroll
-    for (int j = 0; j < 16; j++) q[j] = p.quant[j];
-
-    const uint32_t lane_off = (tid & 31u) * 8u;
-    bool table_ready = false;
-    for (uint32_t c = gl; c < nchunk || !table_ready; c += NT) {
-        const bool live = c < nchunk && have_rows;
-        const uint32_t cc = c < nchunk ? c : 0; // idle lanes of the first pass repeat chunk 0 and drop it
-        constexpr int NX = F16 ? 4 : 8;
-        uint4 xv[NX];
-#pragma unroll
-        for (int i = 0; i < NX; i++) xv[i] = load128(reinterpret_cast<const uint8_t *>(x + ((uint64_t)cc << 5)) + 16 * i);
-        uint4 wv[ROWS];
-        uint16_t sc[ROWS];
-#pragma unroll
-        for (int r = 0; r < ROWS; r++) {
-            const uint32_t rr = min((uint32_t)r, rows_valid - 1);
-            const uint64_t off = (uint64_t)rr * K + ((uint64_t)cc << 5);
-            wv[r] = load128_stream(wbase + (off >> 1));
-            sc[r] = p.scale[(e0 + off) >> 6];
-        }
-        if (!table_ready) {
-            // built once, behind the loads of the first pass, which stay in flight across the barrier
-            const float h0 = h2f(f2h(q0));
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float q1 = q[i];
-                if constexpr (F16) {
-                    const float h1 = h2f(f2h(q1));
-                    tab[tid + i * NTHREADS] = make_uint2((uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16),
-                                                         (uint32_t)f2h((q0 - h0) * 2048.0f) | ((uint32_t)f2h((q1 - h1) * 2048.0f) << 16));
-                } else {
-                    tab[tid + i * NTHREADS] = make_uint2(__float_as_uint(q0), __float_as_uint(q1));
-                }
-            }
-            lds_barrier();
-            table_ready = true;
-        }
-        if (!live) continue;
-        const uint8_t *tabb = reinterpret_cast<const uint8_t *>(tab);
-        if constexpr (F16) {
-#pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float ph = 0.0f, pl = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; j++) {
-                    const uint32_t addr = __builtin_amdgcn_perm(lane_off, w[j >> 2], 0x0c0c0004u | ((j & 3) << 8));
-                    const uint2 e = *reinterpret_cast<const uint2 *>(tabb + addr);
-                    const uint4 &xq = xv[j >> 2];
-                    const uint32_t xd = (j & 3) == 0 ? xq.x : (j & 3) == 1 ? xq.y : (j & 3) == 2 ? xq.z : xq.w;
-                    ph = dot2(e.x, xd, ph);
-                    pl = dot2(e.y, xd, pl);
-                }
-                acc[r] = fmaf(h2f(sc[r]), fmaf(pl, 1.0f / 2048.0f, ph), acc[r]);
-            }
-        } else {
-            float xf[32];
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                xf[4 * i] = __uint_as_float(xv[i].x);
-                xf[4 * i + 1] = __uint_as_float(xv[i].y);
-                xf[4 * i + 2] = __uint_as_float(xv[i].z);
-                xf[4 * i + 3] = __uint_as_float(xv[i].w);
-            }
-#pragma unroll
-            for (int r = 0; r < ROWS; r++) {
-                const uint32_t w[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
-                float pr = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; j++) {
-                    const uint32_t addr = __builtin_amdgcn_perm(lane_off, w[j >> 2], 0x0c0c0004u | ((j & 3) << 8));
-                    const uint2 e = *reinterpret_cast<const uint2 *>(tabb + addr);
-                    pr = fmaf(__uint_as_float(e.x), xf[2 * j], pr);
-                    pr = fmaf(__uint_as_float(e.y), xf[2 * j + 1], pr);
-                }
-                acc[r] = fmaf(h2f(sc[r]), pr, acc[r]);
-            }
-        }
-    }
-    // lanes reduce inside DPP rows; the NT / 16 row partials of every output row meet in LDS
-#pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-        const float s = row_sum(acc[r]);
-        if ((gl & 15) == 0) red[grp][r][gl >> 4] = s;
-    }
-    __syncthreads();
-    const uint32_t l = gl & 15;
-    for (uint32_t o = gl >> 4; o < (uint32_t)ROWS; o += NROW16) {
-        float s = 0.0f;
-#pragma unroll
-        for (int i = 0; i < NROW16 / 16; i++) s += red[grp][o][l + 16 * i];
-        if (NROW16 < 16) s = l < NROW16 ? red[grp][o][l] : 0.0f;
-        s = row_sum(s);
-        const uint32_t row = row0 + o;
-        if (l == 0 && row < p.R) store_out(p.out, p.out_f16, row, act_apply(p.act, s));
-    }
-}
-
 // f16 weights, one token (matmul_vec_fp16, src/shaders/matmul_vec_fp16.wgsl:57-120): the same
 // one-shot shape without any dequantisation.  A lane holds 8 weights (16 bytes) of each of its
 // ROWS rows and the 8 activations they meet; f16 activations go through v_dot2_f32_f16, f32
@@ -989,35 +843,6 @@ int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt
     return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
 
-template <typename XT, int ROWS, int NT, int RG>
-int launch_nf4_wide_cfg(hipStream_t stream, const GemvGroup &g) {
-    constexpr size_t lds = 256 * 32 * sizeof(uint2) + (size_t)RG * ROWS * (NT / 16) * sizeof(float);
-    const dim3 grid(g.total_tasks);
-    if (g.n == 1) {
-        auto *kern = &gemv_nf4_wide_kernel<XT, ROWS, NT, RG, true>;
-        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)once;
-        hipLaunchKernelGGL(kern, grid, dim3(NT * RG), lds, stream, g);
-    } else {
-        auto *kern = &gemv_nf4_wide_kernel<XT, ROWS, NT, RG, false>;
-        static const hipError_t once = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)once;
-        hipLaunchKernelGGL(kern, grid, dim3(NT * RG), lds, stream, g);
-    }
-    return check_launch("matmul_vec_nf4");
-}
-
-// nt lanes along K per row group, 512 / nt row groups of `rows` rows per workgroup
-template <typename XT, int ROWS>
-int launch_nf4_wide(hipStream_t stream, const GemvGroup &g, int nt) {
-    switch (nt) {
-    case 64: return launch_nf4_wide_cfg<XT, ROWS, 64, 8>(stream, g);
-    case 128: return launch_nf4_wide_cfg<XT, ROWS, 128, 4>(stream, g);
-    case 256: return launch_nf4_wide_cfg<XT, ROWS, 256, 2>(stream, g);
-    default: return launch_nf4_wide_cfg<XT, ROWS, 512, 1>(stream, g);
-    }
-}
-
 bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
     const uint32_t chunk = quant == kInt8 ? 16 : 32;
     const size_t xs = in_f16 ? 2 : 4;
@@ -1089,18 +914,6 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (oneshot && quant == kInt8 && ott == 2 && !tune_is_set(kTuneGemvRows)) rows = 4;
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
-        // nf4, one token: workgroups of 512 threads around one conflict-free 64 KiB table; nt lanes along
-        // K per row group, 512 / nt row groups of 4 or 8 rows.  Two such workgroups fit a CU: 8 rows per
-        // group once 4 would need more than 512 workgroups
-        auto wide_nt_of = [](uint32_t K) { const uint32_t c = K / 32; return c > 256 ? 512 : c > 128 ? 256 : c > 64 ? 128 : 64; };
-        const bool wide = oneshot && quant == kNf4 && T == 1 && tune(kTuneNf4Wide, 0) != 0;
-        const int wide_nt = wide_nt_of(args[i].K);
-        int wide_rows = 4;
-        if (wide) {
-            const uint64_t per4 = (uint64_t)(512 / wide_nt) * 4;
-            wide_rows = tune(kTuneGemvRows, (rows_total + per4 - 1) / per4 > 512 ? 8 : 4) == 8 ? 8 : 4;
-            rows = (512 / wide_nt) * wide_rows; // rows per task: a task is a workgroup
-        }
         while (i < n && g.n < (uint32_t)kMaxGroup) {
             const MatmulArgs &a = args[i];
             if (a.R == 0 || a.T == 0 || a.B == 0) {
@@ -1117,7 +930,6 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             }
             // the resident kernel builds one table per workgroup: its groups share the table tensor
             if (!oneshot && a.quant != g.quant && g.n) break;
-            if (wide && wide_nt_of(a.K) != wide_nt && g.n) break;
             if (a.B > 1 && g.n + a.B > (uint32_t)kMaxGroup && g.n) break;
             if (lds + need * a.B > kGemvLdsBudget && g.n) break;
             // the batch axis unrolls into products of its own
@@ -1163,15 +975,6 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         }
         if (!g.n) continue;
         g.total_tasks = tasks;
-        if (wide) {
-            int s1;
-            if (wide_rows == 8)
-                s1 = in_f16 ? launch_nf4_wide<__half, 8>(stream, g, wide_nt) : launch_nf4_wide<float, 8>(stream, g, wide_nt);
-            else
-                s1 = in_f16 ? launch_nf4_wide<__half, 4>(stream, g, wide_nt) : launch_nf4_wide<float, 4>(stream, g, wide_nt);
-            if (s1 != WRQ_OK) return s1;
-            continue;
-        }
         if (oneshot && quant == kNf4) {
             const uint32_t nchunk = g.p[0].K / 32;
             int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk >= 128 ? 128 : 64;

@@ -60,11 +60,6 @@ enum TuneKey {
     kTuneGemmKg,
     kTuneGemmKsplit,
     kTuneVecChunkMinT, // vec_chunk_min_t: first token count the decode entry sends to the chunk kernel
-    kTuneNf4Wide,      // nf4_wide: 0 keeps nf4 decode on the per-task table kernel
-    kTuneExp0,         // exp0 .. exp3: free knobs of experimental kernels
-    kTuneExp1,
-    kTuneExp2,
-    kTuneExp3,
     kTuneCount
 };
 // The override of `key`, or `fallback` when it is unset.
