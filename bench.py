@@ -32,6 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 matrix cores
 SEED = 0x57525100
 
 
@@ -268,7 +269,16 @@ def sweep_pack(wrq, torch, quant, w):
 
 def sweep(wrq, torch, args):
     """Per-operator figures of configs 2 and 3: cold (rotating weight copies) GB/s per shape."""
+    import ctypes as C
+
     rows = []
+    probe = None
+    if args.probe:
+        if not os.path.exists(PROBE_LIB):
+            build_probe()
+        probe = C.CDLL(PROBE_LIB)
+        probe.wrq_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int]
+        sink = torch.zeros(16, dtype=torch.int32, device="cuda")
     g = torch.Generator(device="cuda").manual_seed(SEED + 2)
     shapes = [(2048, 2048), (2048, 7168), (7168, 2048), (2048, 65536), (4096, 4096), (4096, 14336), (14336, 4096)]
     for quant in ("int8", "nf4", "fp16"):
@@ -309,6 +319,26 @@ def sweep(wrq, torch, args):
                 rows.append({"quant": quant, "K": K, "R": R, "T": T, "us": round(us, 2),
                              "GBps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
                              "TFLOPs": round(flops / us / 1e6, 1), "copies": ncopy})
+                if T == 1 and probe is not None:
+                    # what a launch of this size can reach at all: the probe's plain streaming read of the same
+                    # packed weights, in the same graph of back-to-back launches over the same rotating copies
+                    it[0] = 0
+
+                    def rd():
+                        wt = mats[it[0] % ncopy].w
+                        st = C.c_void_p(torch.cuda.current_stream().cuda_stream)  # the capture stream, inside a capture
+                        probe.wrq_probe_read(st, C.c_void_p(wt.data_ptr()), C.c_void_p(sink.data_ptr()), wt.numel() * wt.element_size(), 2, 1)
+                        it[0] += 1
+
+                    rd()
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        for _ in range(reps):
+                            rd()
+                    ms, _ = time_steps(torch, graph.replay, 5, 2)
+                    rows[-1]["plain_read_us"] = round(ms * 1e3 / reps, 2)
+                    rows[-1]["of_plain_read"] = round(ms * 1e3 / reps / us, 3)
                 print(json.dumps(rows[-1]), flush=True)
             del mats, m0
             torch.cuda.empty_cache()
@@ -751,7 +781,9 @@ def main():
     traffic = None
     if args.tokens == 1 and grouped and not args.with_head and args.layers == 32:
         traffic = read_traffic(args.quant)
-    kernel = {("int8", True): "gemv_int8_oneshot_kernel", ("nf4", True): "gemv_nf4_oneshot_kernel"}.get((args.quant, args.tokens == 1), "gemm_kernel")
+    # the vec entry point keeps runs of up to 4 (int8) or 2 (nf4) tokens on the decode kernels
+    on_decode_kernel = args.tokens <= (4 if args.quant == "int8" else 2)
+    kernel = f"gemv_{args.quant}_oneshot_kernel" if on_decode_kernel else "gemm_kernel"
     out = {
         "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
         "value": round(tok_s, 2),
@@ -780,6 +812,13 @@ def main():
             "avg_launch_us": round(launch_us, 3), "bytes_per_launch": nbytes // dec.launches,
         },
     }
+    # from some token count on the matrix cores bound a step, not HBM: 2 K R T flops per product against the
+    # dense f16 peak take longer than the packed bytes against the HBM peak
+    flops = 2.0 * args.tokens * len(layers) * (5 * C * C + 2 * C * H + C * C) + (2.0 * args.tokens * C * 65536 if args.with_head else 0.0)
+    if flops / (MFMA_F16_PEAK_TFLOPS * 1e12) > nbytes / (HBM_PEAK_GBPS * 1e9):
+        tflops = flops / dec.launches / launch_us / 1e6
+        out["roofline"].update({"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "flops_per_launch": int(flops // dec.launches)})
     if probe:
         out["probe"] = probe
     if not args.no_cpu_baseline:
