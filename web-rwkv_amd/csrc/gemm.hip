@@ -353,6 +353,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     };
     // k group `kg` owns the steps kg, kg + KG, ...: local step m is step m * KG + kg
     const uint32_t nlocal = (nsteps + KG - 1 - kg) / KG;
+    // Weight loads.  From 32-token tiles on they are plain cacheable loads: marked nontemporal, the compiler's
+    // load-counter bookkeeping falls back to a full wait at the head of the main loop and the ring of prefetched
+    // K steps drains once per iteration.  The 16-token tile keeps streaming loads: its launches are short, the
+    // drain costs little there and weights that bypass the caches leave them to the activations.
+    constexpr bool STREAM_W = NTILE == 1;
+    auto lw128 = [&](const uint8_t *p) { return STREAM_W ? load128_stream(p) : load128(p); };
+    auto lw64 = [&](const uint8_t *p) { return STREAM_W ? load64_stream(p) : *reinterpret_cast<const uint2 *>(p); };
     auto load_w = [&](uint32_t m, StepRegs &dst) {
         const uint32_t step = min(min(m, max(nlocal, 1u) - 1) * KG + kg, last); // clamped to the K range
 #pragma unroll
@@ -360,15 +367,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
             const uint8_t *p = wp[i] + step * WSTEP;
             if constexpr (TRW) {
 #pragma unroll
-                for (int j = 0; j < NW; j++) dst.w[i][j] = load128(wq[i][j] + step * WSTEP);
+                for (int j = 0; j < NW; j++) dst.w[i][j] = lw128(wq[i][j] + step * WSTEP);
             } else if (QUANT == kFp16) {
 #pragma unroll
-                for (int j = 0; j < NW; j++) dst.w[i][j] = load128(p + 64 * j); // operand j: k = 32 j + 8 g .. + 8
+                for (int j = 0; j < NW; j++) dst.w[i][j] = lw128(p + 64 * j); // operand j: k = 32 j + 8 g .. + 8
             } else if (QUANT == kInt8) {
-                dst.w[i][0] = load128(p);
-                dst.w[i][NW - 1] = load128(p + 64);
+                dst.w[i][0] = lw128(p);
+                dst.w[i][NW - 1] = lw128(p + 64);
             } else {
-                const uint2 v0 = *reinterpret_cast<const uint2 *>(p), v1 = *reinterpret_cast<const uint2 *>(p + 32);
+                const uint2 v0 = lw64(p), v1 = lw64(p + 32);
                 dst.w[i][0] = make_uint4(v0.x, v0.y, v1.x, v1.y);
             }
         }
