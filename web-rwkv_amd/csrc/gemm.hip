@@ -41,6 +41,8 @@
 //   nf4:  A holds table values split into two f16 halves (hi + lo * 2^-11, exact to
 //         2^-22), fetched per byte (two weights) from a 256-entry LDS table; after each
 //         64-block   out += absmax * (D_hi + 2^-11 D_lo).
+// f32 activations are split the same way while they are staged (hi + lo * 2^-11 as two f16 tiles, exact to 2^-22):
+// every product term is then taken against both tiles.
 // D is produced by MFMAs that start from a zero C operand, in ordinary vector registers,
 // so the only per-block work outside the matrix cores is one or two fmas per output.
 // Plain f16 weights (matmul_mat_fp16, src/shaders/matmul_mat_fp16.wgsl:57-140) take the same
