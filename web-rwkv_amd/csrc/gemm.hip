@@ -676,10 +676,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     });
 }
 
-// Second half of a split-K product: sum of the partial tiles over the splits, activation,
-// output type.  One thread per lane slot of the first kernel's tiles (same decoding).
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const MatmulArgs a, const float *scratch, uint32_t splits, uint32_t nwg,
-                                                          uint32_t tblocks, uint32_t row_tiles, uint32_t rw, uint32_t mrt, uint32_t ntile) {
+// Second half of a split-K launch: sum of the partial tiles over the splits, activation, output type, for every
+// product of the launch (blockIdx.y).  One thread per lane slot of the first kernel's tiles (same decoding).
+__global__ __launch_bounds__(256) void gemm_finish_kernel(const GemmArgs ga, uint32_t splits, uint32_t rw, uint32_t mrt, uint32_t ntile) {
+    const uint32_t pi = blockIdx.y;
+    const MatmulArgs a = ga.m[pi];
+    const float *scratch = ga.scratch[pi];
+    const uint32_t tblocks = ga.tblocks, row_tiles = ga.row_tiles[pi];
+    const uint32_t nwg = (row_tiles + 7) / 8 * 8 * tblocks;
     const uint32_t per_wg = rw * mrt * ntile * 64; // lane slots per workgroup tile
     const uint64_t slots = (uint64_t)a.B * nwg * per_wg;
     const uint64_t q = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -809,11 +813,10 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     int s = check_launch("matmul_mat");
     if (s != WRQ_OK) return s;
     if (splits > 1) {
-        for (int i = 0; i < n; i++) {
-            const uint64_t slots = slice[i] / 4;
-            hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256)), dim3(256), 0, stream, args[i], ga.scratch[i], splits,
-                               nwg[i], ga.tblocks, ga.row_tiles[i], (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
-        }
+        uint64_t slots = 0; // of the largest product: smaller ones leave the rest of their grid row idle
+        for (int i = 0; i < n; i++) slots = std::max(slots, slice[i] / 4);
+        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256), (uint32_t)n), dim3(256), 0, stream, ga, splits,
+                           (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
         s = check_launch("matmul_mat (finish)");
     }
     return s;
@@ -835,19 +838,22 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
     // long rows against 256 tokens and more also take the 128-token tile (measured on 4096 x 14336: 7 % faster)
-    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128) ? 2 : (T > 64 && (rt >= (1u << 23) || (T >= 256 && a.K >= 8192))) ? 8 : 4;
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128 && n == 1) ? 2 : (T > 64 && (rt >= (1u << 23) || (T >= 256 && a.K >= 8192))) ? 8 : 4;
     int mrt = 2, kg = 1;
     uint32_t ksplit = 1;
     uint64_t wgs = 0; // workgroups of one split
     auto tblocks_of = [&](int nt) { return (uint64_t)(T + 16 * nt - 1) / (16 * nt); };
     // K is split over the grid until there are one (narrow tiles) to four workgroups per CU, at most
-    // 8 ways; a group that fills most CUs unsplit stays unsplit (every split product costs a finish launch)
+    // 8 ways.  A split launch costs one finish launch for all its products: with 64-token tiles a group is
+    // split like a single product (two workgroups per CU beat one: the attention group at 128 tokens 42.4
+    // against 46.2 us, nf4 at 64 tokens 35.8 against 43.7 us), with narrower tiles a group that fills most
+    // CUs stays unsplit
     auto split_for = [&]() {
         wgs = (uint64_t)((rows * kg + 64 * mrt - 1) / (64 * mrt)) * tblocks_of(ntile) * a.B;
-        const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 512 : 1024;
+        const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 640 : 1024;
         ksplit = 1;
         while (kg == 1 && ksplit < 8 && wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
-        if (n >= 2 && wgs >= 200) ksplit = 1;
+        if (n >= 2 && wgs >= 200 && ntile != 4) ksplit = 1;
     };
     // 64-row tiles where they give about one workgroup per CU without a split of K (a 16-token tile:
     // also below that); otherwise 128-row tiles, fewer activation copies per weight byte, and more splits
