@@ -449,6 +449,42 @@ def test_chunk_k_groups_by_default(gpu, oracle, kind, T):
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("T,ksplit", [(128, 2), (256, 1), (252, 1)], ids=str)
+def test_chunk_grid_a_little_above_two_workgroups_per_cu(gpu, oracle, kind, T, ksplit, overrides):
+    # 576 workgroups (288 tiles of 128 rows x 64 tokens split in two, or 576 tiles) run as two launches:
+    # the first 512 as they are, the tiles of the rest with K split 8 ways further, one finish launch
+    # for both kinds.  The group {14336, 4096} rows and a single product of 18432 rows both have that
+    # grid; with the cut switched off (gemm_tail=0) the results must agree to the same bound.
+    import torch
+
+    announce("chunk grid tail", kind, T, ksplit)
+    rng = np.random.default_rng(SEED + 43 + T)
+    K = 2048
+    packed = {}
+    for R in (4096, 14336, 18432):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        packed[R] = (gpu_matrix(gpu, kind, wp, scale), wdeq)
+    overrides(gemm_kg=1, gemm_mrt=2, gemm_ntile=4, gemm_ksplit=ksplit)
+    for tail in (1, 0):
+        overrides(gemm_tail=tail)
+        for x_dtype in (np.float16, np.float32):
+            rows = [14336, 4096]
+            xs = [gen_f16(rng, (T, K), 1.0).astype(x_dtype) for _ in rows]
+            outs = [torch.full((T, R), float("nan"), dtype=torch.float16 if R == 4096 else torch.float32, device="cuda") for R in rows]
+            gpu.matmul_vec_group([(packed[R][0], dev(xv), o, gpu.ACT_SQUARED_RELU if R == 14336 else gpu.ACT_NONE, False, {})
+                                  for R, xv, o in zip(rows, xs, outs)])
+            for R, xv, o in zip(rows, xs, outs):
+                truth = truth_matmul(packed[R][1], xv)
+                if R == 14336:
+                    truth = np.square(np.maximum(truth, 0.0))
+                assert_close(host(o), truth, EPS, f"{kind} group {rows} T={T} tail={tail} {np.dtype(x_dtype).name}")
+        m, wdeq = packed[18432]
+        x = gen_f16(rng, (T, K), 1.0)
+        assert_close(run(gpu, m, x, 18432, "mat", np.float32), truth_matmul(wdeq, x), EPS, f"{kind} 18432 rows T={T} tail={tail}")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
 def test_reference_test_data_scale(gpu, oracle, kind):
     # the reference's unit tests draw weights/inputs of magnitude ~1..5, outputs ~100 (ops.rs:2929-2937, 3072-3093)
     announce("reference test scale", kind)

@@ -155,6 +155,9 @@ struct GemmArgs {
     float *scratch[kMaxGroup]; // partial tiles of every product; null: store directly
     uint32_t k_per_split;      // K range of one workgroup, a multiple of kStep
     uint32_t tblocks;          // ceil(T / BN)
+    uint32_t tile_offset;      // blockIdx.x + tile_offset numbers the tiles of the group: a launch may cover a range of them
+    uint32_t split_from;       // finish kernel: tiles from this number on have `splits` partial tiles, ...
+    uint32_t splits_low;       // ... those below have this many (0 or 1: stored directly, nothing to finish)
 };
 
 // blockIdx.x -> (row tile, token block).  Workgroups are dealt round-robin to the 8 XCDs, each
@@ -171,13 +174,14 @@ template <int QUANT, typename XT, int MRT, int NTILE, int KG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs ga) {
     using G = Geometry<MRT, NTILE, KG>;
     // the product of this workgroup: one scalar load of the tile starts, then its descriptor
+    const uint32_t gid = blockIdx.x + ga.tile_offset; // tile number inside the group
     uint32_t pi = 0;
 #pragma unroll
     for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-        if (blockIdx.x >= ga.tile_begin[i]) pi = i;
+        if (gid >= ga.tile_begin[i]) pi = i;
     pi = __builtin_amdgcn_readfirstlane(pi);
     const MatmulArgs a = ga.m[pi];
-    const uint32_t tile_id = blockIdx.x - ga.tile_begin[pi];
+    const uint32_t tile_id = gid - ga.tile_begin[pi];
     const uint32_t my_row_tiles = ga.row_tiles[pi];
     float *const my_scratch = ga.scratch[pi];
     constexpr int BN = G::BN, BM = G::BM, RW = G::RW, KSUB = G::KSUB, LSUB = G::LSUB, PITCH = G::PITCH, NPIECE = G::NPIECE, NBUF = G::nbuf(QUANT), THREADS = G::THREADS;
@@ -682,6 +686,7 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const GemmArgs ga, uin
     const uint32_t pi = blockIdx.y;
     const MatmulArgs a = ga.m[pi];
     const float *scratch = ga.scratch[pi];
+    if (!scratch) return; // no tile of this product was split
     const uint32_t tblocks = ga.tblocks, row_tiles = ga.row_tiles[pi];
     const uint32_t nwg = (row_tiles + 7) / 8 * 8 * tblocks;
     const uint32_t per_wg = rw * mrt * ntile * 64; // lane slots per workgroup tile
@@ -693,6 +698,8 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const GemmArgs ga, uin
     const uint64_t bw = q / per_wg;
     const uint32_t wg = (uint32_t)(bw % nwg), b = (uint32_t)(bw / nwg);
     const uint32_t n = tp % ntile, wi = tp / ntile; // wi = wave * mrt + i
+    if (ga.tile_begin[pi] + wg < ga.split_from) splits = ga.splits_low;
+    if (splits <= 1) return; // stored directly by a launch without a split
     uint32_t row_tile, tblock;
     tile_of_block(wg, tblocks, row_tile, tblock);
     if (row_tile >= row_tiles) return;
@@ -808,6 +815,55 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
         }
     }
     if (a0.B > 65535u || splits > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a0.B > splits ? a0.B : splits, 65535u);
+    ga.tile_offset = 0;
+    ga.split_from = 0;
+    ga.splits_low = 0;
+    // Grid quantisation: two workgroups of these kernels fit a CU, 512 run at a time.  A grid a little above that
+    // (the 576 workgroups of {ffn.key, ffn.receptance} at 128 and 256 tokens) leaves most CUs waiting for the few
+    // that got a third one.  Such a launch is cut in two: the tiles that fill the CUs evenly run as they are, the
+    // rest follows with K split over up to 8 times as many workgroups per tile, so that the second round is short
+    // and wide.  One finish launch sums both kinds of tiles.
+    const uint32_t wgs_all = total * splits;
+    if (a0.B == 1 && wgs_all > 512 && wgs_all <= 640 && steps % splits == 0 && tune(kTuneGemmTail, 1)) {
+        const uint32_t even = 512 / splits, rest = total - even; // tiles of the two launches
+        uint32_t ks = 8 * splits;
+        while (ks > splits && (rest * ks > 512 || steps / ks < 2 || steps % ks != 0)) ks /= 2;
+        // partial tiles of the rest lie like those of a product split `ks` times: room for every product with tiles in it
+        auto planes = [&](int i, uint32_t k) { return ga.tile_begin[i] + nwg[i] > even ? k : splits > 1 ? splits : 0u; };
+        auto need = [&](uint32_t k) {
+            uint64_t f = 0;
+            for (int i = 0; i < n; i++) f += slice[i] * planes(i, k);
+            return f;
+        };
+        while (ks > splits && need(ks) > cap) ks /= 2;
+        float *base = sp ? sp->base : scratch_ptr();
+        if (ks > splits && base) {
+            GemmArgs gb = ga;
+            uint64_t off = 0;
+            for (int i = 0; i < n; i++) {
+                gb.scratch[i] = planes(i, ks) ? base + off : nullptr;
+                off += slice[i] * planes(i, ks);
+            }
+            gb.tile_offset = even;
+            gb.split_from = even;
+            gb.splits_low = splits;
+            gb.k_per_split = steps / ks * kStep;
+            if (splits > 1)
+                for (int i = 0; i < n; i++) ga.scratch[i] = gb.scratch[i];
+            hipLaunchKernelGGL(kern, dim3(even, splits, 1), dim3(G::THREADS), lds, stream, ga);
+            int s = check_launch("matmul_mat");
+            if (s != WRQ_OK) return s;
+            hipLaunchKernelGGL(kern, dim3(rest, ks, 1), dim3(G::THREADS), lds, stream, gb);
+            s = check_launch("matmul_mat (rest)");
+            if (s != WRQ_OK) return s;
+            uint64_t slots = 0;
+            for (int i = 0; i < n; i++)
+                if (gb.scratch[i]) slots = std::max(slots, slice[i] / 4);
+            hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256), (uint32_t)n), dim3(256), 0, stream, gb, ks,
+                               (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
+            return check_launch("matmul_mat (finish)");
+        }
+    }
     dim3 grid(total, splits, a0.B);
     hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), lds, stream, ga);
     int s = check_launch("matmul_mat");

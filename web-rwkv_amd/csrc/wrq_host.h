@@ -60,6 +60,7 @@ enum TuneKey {
     kTuneGemmKg,
     kTuneGemmKsplit,
     kTuneVecChunkMinT, // vec_chunk_min_t: first token count the decode entry sends to the chunk kernel
+    kTuneGemmTail,     // gemm_tail: 0 keeps a grid a little above two workgroups per CU in one launch
     kTuneCount
 };
 // The override of `key`, or `fallback` when it is unset.
