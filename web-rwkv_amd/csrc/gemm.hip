@@ -818,13 +818,14 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     ga.tile_offset = 0;
     ga.split_from = 0;
     ga.splits_low = 0;
-    // Grid quantisation: two workgroups of these kernels fit a CU, 512 run at a time.  A grid a little above that
+    // Grid quantisation: two workgroups of the kernels with 64-token tiles or wider fit a CU, 512 run at a time (the
+    // narrower tiles leave room for more, and their grids need no cut).  A grid a little above that
     // (the 576 workgroups of {ffn.key, ffn.receptance} at 128 and 256 tokens) leaves most CUs waiting for the few
     // that got a third one.  Such a launch is cut in two: the tiles that fill the CUs evenly run as they are, the
     // rest follows with K split over up to 8 times as many workgroups per tile, so that the second round is short
     // and wide.  One finish launch sums both kinds of tiles.
     const uint32_t wgs_all = total * splits;
-    if (a0.B == 1 && wgs_all > 512 && wgs_all <= 640 && steps % splits == 0 && tune(kTuneGemmTail, 1)) {
+    if (NTILE >= 4 && a0.B == 1 && wgs_all > 512 && wgs_all <= 640 && steps % splits == 0 && tune(kTuneGemmTail, 1)) {
         const uint32_t even = 512 / splits, rest = total - even; // tiles of the two launches
         uint32_t ks = 8 * splits;
         while (ks > splits && (rest * ks > 512 || steps / ks < 2 || steps % ks != 0)) ks /= 2;
