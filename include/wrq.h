@@ -100,7 +100,8 @@ int wrq_init(void);
  * Test and sweep hook; no counterpart in the reference.  The library chooses kernels and tiles by
  * shape.  An override pins one choice so that a test can reach every instantiation: keys are
  * "gemm_ntile", "gemm_mrt", "gemm_kg", "gemm_ksplit", "gemv_rows", "gemv_nt", "gemv_oneshot",
- * "vec_chunk_min_t", ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
+ * "vec_chunk_min_t", "gemm_tail" (0: a chunk grid a little above two workgroups per CU stays one
+ * launch), ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
  * library first looks (wrq_init, or the first product) presets the same table; nothing on the launch
  * path reads the environment.  Overrides are process-wide: not for use while other threads launch.
  */
