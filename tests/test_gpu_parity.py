@@ -243,6 +243,83 @@ def test_gemv_against_oracle(gpu, oracle, kind, K, R):
         assert_close(got, truth_matmul(wdeq, x), 1e-4, f"{kind} {K}x{R} f32 vs float64")
 
 
+# every K / 1024 the wave-owns-rows decode kernel is built for
+WAVE_ROWS_K = [1024 * b for b in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16)]
+
+
+@pytest.mark.parametrize("K", WAVE_ROWS_K)
+def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
+    # one token, f16 activations, K a multiple of 1024: single products and groups, rows that do not fill the last
+    # task, all output types, an activation, a z-offset view, the batch axis -- against the oracle and float64; the
+    # kernel it replaces (gemv_waverows=0) is held to the same bar on the same inputs
+    import torch
+
+    announce("int8 wave-owns-rows", K)
+    rng = np.random.default_rng(SEED + 77 + K)
+    rows = [204, 64, 8, 4, 132]  # multiples of 4 (the entry point requires it): ragged last tasks, a single task
+    mats, xs, truths, wants = [], [], [], []
+    for R in rows:
+        w = gen_f16(rng, (R, K), 0.02)
+        x = gen_f16(rng, (1, K), 1.0)
+        wp, scale, wdeq = pack(oracle, "int8", w)
+        mats.append(gpu_matrix(gpu, "int8", wp, scale))
+        xs.append(x)
+        truths.append(truth_matmul(wdeq, x))
+        wants.append(oracle.matmul_vec_int8(wp, scale, x, out_dtype=np.float32)[0])
+    for waverows in (1, 0):
+        overrides(gemv_waverows=waverows)
+        for m, x, R, truth, want in zip(mats, xs, rows, truths, wants):
+            for out_dtype in (np.float16, np.float32):
+                got = run(gpu, m, x, R, "vec", out_dtype)
+                assert_close(got, want, EPS, f"K={K} R={R} waverows={waverows} vs oracle")
+                assert_close(got, truth, EPS, f"K={K} R={R} waverows={waverows} vs float64")
+            got = run(gpu, m, x, R, "vec", np.float32, act=1)
+            assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"K={K} R={R} squared relu")
+        # all five in one grouped launch, mixed output types and activations
+        outs = [torch.full((1, R), float("nan"), dtype=torch.float16 if i % 2 else torch.float32, device="cuda") for i, R in enumerate(rows)]
+        gpu.matmul_vec_group([(m, dev(x), o, gpu.ACT_SQUARED_RELU if i == 2 else gpu.ACT_NONE, False, {})
+                              for i, (m, x, o) in enumerate(zip(mats, xs, outs))])
+        for i, (o, truth) in enumerate(zip(outs, truths)):
+            assert_close(host(o).astype(np.float32), np.square(np.maximum(truth, 0.0)) if i == 2 else truth, EPS, f"K={K} group member {i}")
+    overrides(gemv_waverows=1)
+    # a z-offset input view and an offset output view (v6: att_sx.view(.., .., i, ..), src/runtime/v6.rs:806-829)
+    parent = gen_f16(rng, (5, 1, K), 1.0)
+    out = torch.full((3, 3, rows[0]), -7.0, dtype=torch.float32, device="cuda")
+    mats[0].matmul_vec_op(dev(parent), out, input_view=((K, 1, 1), (K, 1, 5), (0, 0, 3)), output_view=((rows[0], 1, 1), (rows[0], 3, 3), (0, 1, 2)))
+    got = host(out)
+    assert_close(got[2, 1:2], oracle.matmul_vec_int8(host(mats[0].w), host(mats[0].m), parent[3], out_dtype=np.float32)[0], EPS, "offset views")
+    got[2, 1:2] = -7.0
+    assert (got == -7.0).all(), "wrote outside the output view"
+    # batch axis: matrix [K, R, B]
+    B, R = 3, 36
+    wb = gen_f16(rng, (B, R, K), 0.02)
+    xb = gen_f16(rng, (B, 1, K), 1.0)
+    wpb, sb, wdq = pack(oracle, "int8", wb)
+    truth = np.stack([truth_matmul(wdq[b], xb[b]) for b in range(B)])
+    assert_close(run(gpu, gpu_matrix(gpu, "int8", wpb, sb), xb, R, "vec", np.float32), truth, EPS, "batched")
+
+
+def test_int8_wave_rows_groups_of_mixed_k(gpu, oracle):
+    # products of different K in one grouped call: the launch is cut where K changes, every product still gets its result
+    import torch
+
+    announce("int8 wave-owns-rows, mixed K in a group")
+    rng = np.random.default_rng(SEED + 78)
+    shapes = [(4096, 96), (4096, 40), (2048, 72), (1152, 24), (4096, 12), (14336, 20), (14336, 4)]  # R % 4 == 0
+    ops, truths, outs = [], [], []
+    for K, R in shapes:
+        w = gen_f16(rng, (R, K), 0.02)
+        x = gen_f16(rng, (1, K), 1.0)
+        wp, scale, wdeq = pack(oracle, "int8", w)
+        o = torch.full((1, R), float("nan"), dtype=torch.float32, device="cuda")
+        ops.append((gpu_matrix(gpu, "int8", wp, scale), dev(x), o, gpu.ACT_NONE, False, {}))
+        outs.append(o)
+        truths.append(truth_matmul(wdeq, x))
+    gpu.matmul_vec_group(ops)
+    for (K, R), o, truth in zip(shapes, outs, truths):
+        assert_close(host(o), truth, EPS, f"mixed group member {K}x{R}")
+
+
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
 @pytest.mark.parametrize("T", [2, 3, 4, 5, 8, 15, 16, 17, 31])
 def test_multi_token_vec_entry(gpu, oracle, kind, T):

@@ -468,6 +468,144 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     oneshot_reduce_store<ROWS, NT, TT>(acc, red, p, row0, g.T);
 }
 
+// int8, one token, f16 activations, K = BPL * 1024: a wave owns RW whole rows.
+//
+// Lane L = (g = L >> 3, sub = L & 7) holds, for j < BPL, the 16 bytes at 128-block g * BPL + j, offset sub * 16 of each of its
+// rows: a wave instruction covers 8 full 128-byte lines, and the BPL (min, max) words of a lane's blocks are contiguous -- one
+// wide load per row instead of one word load per 16 weight bytes.  The activations reach LDS once per workgroup (4 waves; an
+// LDS-only barrier, the weight loads stay in flight across it) and every wave reads the 32 bytes that meet each of its chunks.
+// Request order: activations, scale words, weights chunk by chunk; rows are consumed in arrival order.  A row's sum closes
+// inside its wave (DPP + readlane): no LDS exchange and no barrier behind the last bytes.
+// Workgroups are handed to the 8 XCDs round-robin: tasks are renumbered so that an XCD takes runs of 64 consecutive output
+// rows, i.e. whole 128-byte lines of an f16 output, and no output line is dirty in two L2s.
+// The scalar arguments come first so that they arrive preloaded in SGPRs (no dependent scalar load in front of the first
+// vector load); a single product needs no descriptor load at all.
+template <int BPL, int RW>
+__device__ __forceinline__ void rows_task_int8(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
+                                               const int out_f16, const int act, const uint32_t task, uint4 *xs) {
+    constexpr int K = BPL * 1024;
+    constexpr int XP = (K / 8 + 255) / 256; // 16-byte pieces of the activations per thread
+    const uint32_t tid = threadIdx.x, lane = tid & 63, g = lane >> 3, sub = lane & 7;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t row0 = task * (4 * RW) + wave * RW;
+    uint4 xp[XP];
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const uint32_t idx = tid + i * 256;
+        if (XP * 256 == K / 8 || idx < K / 8) xp[i] = load128(reinterpret_cast<const uint4 *>(x) + idx);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t sc[RW][BPL];
+    const uint8_t *wrow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        const uint32_t row = min(row0 + r, R - 1); // rows past the end repeat the last one and are not stored
+        wrow[r] = w + (uint64_t)row * K + (g * BPL) * 128 + sub * 16;
+        const uint32_t *sp = mm + (uint64_t)row * (K / 128) + g * BPL;
+        if constexpr (BPL % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < BPL / 4; q++) {
+                const uint4 v = load128(sp + 4 * q);
+                sc[r][4 * q] = v.x, sc[r][4 * q + 1] = v.y, sc[r][4 * q + 2] = v.z, sc[r][4 * q + 3] = v.w;
+            }
+        } else if constexpr (BPL % 2 == 0) {
+#pragma unroll
+            for (int q = 0; q < BPL / 2; q++) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(sp + 2 * q);
+                sc[r][2 * q] = v.x, sc[r][2 * q + 1] = v.y;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < BPL; j++) sc[r][j] = sp[j];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint4 wv[RW][BPL];
+#pragma unroll
+    for (int j = 0; j < BPL; j++)
+#pragma unroll
+        for (int r = 0; r < RW; r++) wv[r][j] = load128_stream(wrow[r] + j * 128);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const uint32_t idx = tid + i * 256;
+        if (XP * 256 == K / 8 || idx < K / 8) xs[idx] = xp[i];
+    }
+    lds_barrier();
+    float acc[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) acc[r] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < BPL; j++) {
+        const uint4 x0 = xs[((g * BPL + j) * 8 + sub) * 2], x1 = xs[((g * BPL + j) * 8 + sub) * 2 + 1];
+        const uint32_t xd[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        float sx = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 8; q++) sx = dot2(xd[q], 0x3c003c00u, sx); // (1.0, 1.0)
+#pragma unroll
+        for (int r = 0; r < RW; r++) {
+            const uint32_t wd[4] = {wv[r][j].x, wv[r][j].y, wv[r][j].z, wv[r][j].w};
+            uint32_t code[8]; // f16 pairs (1024 + u0, 1024 + u1)
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                code[2 * d] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04010400u);
+                code[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04030402u);
+            }
+            const float mn = h2f((uint16_t)(sc[r][j] & 0xffffu));
+            const float mx = h2f((uint16_t)(sc[r][j] >> 16));
+            const float s = (mx - mn) * (1.0f / 255.0f);
+            const float c0 = fmaf(-1024.0f, s, mn);
+            float pr = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 8; q++) pr = dot2(code[q], xd[q], pr);
+            acc[r] = fmaf(s, pr, fmaf(c0, sx, acc[r]));
+        }
+    }
+    float mine = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        const float s = wave_sum(acc[r]);
+        if (lane == (uint32_t)r) mine = s;
+    }
+    if (lane < (uint32_t)RW && row0 + lane < R) store_out(out, out_f16, row0 + lane, act_apply(act, mine));
+}
+
+// Runs of `run` consecutive tasks per XCD (workgroup b starts on XCD b % 8); the tail that does not fill 8 runs keeps its numbers.
+__device__ __forceinline__ uint32_t xcd_task(uint32_t b, uint32_t total, uint32_t run) {
+    const uint32_t full = total / (8 * run) * (8 * run);
+    if (b >= full) return b;
+    const uint32_t xcd = b & 7, idx = b >> 3;
+    return ((idx / run) * 8 + xcd) * run + idx % run;
+}
+
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_single_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
+                                                                    const uint32_t R, const uint32_t total_tasks, const uint32_t flags) {
+    __shared__ uint4 xs[BPL * 128];
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    rows_task_int8<BPL, RW>(w, mm, x, out, R, (int)(flags & 1u), (int)(flags >> 1), task, xs);
+}
+
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t tb4,
+                                                                   const uint32_t tb5, const uint32_t tb6, const uint32_t tb7,
+                                                                   const uint32_t total_tasks, const GemvGroup g) {
+    __shared__ uint4 xs[BPL * 128];
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    uint32_t pi = 0;
+    pi = task >= tb1 ? 1u : pi;
+    pi = task >= tb2 ? 2u : pi;
+    pi = task >= tb3 ? 3u : pi;
+    pi = task >= tb4 ? 4u : pi;
+    pi = task >= tb5 ? 5u : pi;
+    pi = task >= tb6 ? 6u : pi;
+    pi = task >= tb7 ? 7u : pi;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
+    rows_task_int8<BPL, RW>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R,
+                            p.out_f16, p.act, task - p.task_begin, xs);
+}
+
 // nf4, one token: the same one-shot shape (one workgroup per task of ROWS rows, NT lanes along
 // K, every load of the task requested up front).  A lane holds 32 weights (16 packed bytes) of
 // each row and the 32 activations they meet.  A packed byte is two weights: a 256-entry LDS
@@ -843,6 +981,43 @@ int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt
     return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
 
+template <int BPL, int RW>
+int launch_rows_int8(hipStream_t stream, const GemvGroup &g) {
+    const dim3 grid(g.total_tasks);
+    if (g.n == 1) {
+        const GemvProblem &p = g.p[0];
+        hipLaunchKernelGGL((gemv_int8_rows_single_kernel<BPL, RW>), grid, dim3(256), 0, stream, p.w,
+                           reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R,
+                           g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1));
+    } else {
+        hipLaunchKernelGGL((gemv_int8_rows_group_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2], g.task_begin[3],
+                           g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, g);
+    }
+    return check_launch("matmul_vec_int8");
+}
+
+// Rows per wave of the wave-owns-rows kernel: two for short rows (at least four 16-byte loads per lane in flight), else one.
+constexpr int rows_per_wave(int bpl) { return bpl <= 2 ? 2 : 1; }
+
+// K / 1024 values the wave-owns-rows kernel is built for.
+bool rows_kernel_has(uint32_t K) {
+    if (K % 1024 != 0) return false;
+    switch (K / 1024) {
+    case 1: case 2: case 3: case 4: case 5: case 6: case 7: case 8: case 10: case 12: case 14: case 16: return true;
+    default: return false;
+    }
+}
+
+int launch_rows_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
+    switch (K / 1024) {
+#define WRQ_ROWS_CASE(B) case B: return launch_rows_int8<B, rows_per_wave(B)>(stream, g);
+    WRQ_ROWS_CASE(1) WRQ_ROWS_CASE(2) WRQ_ROWS_CASE(3) WRQ_ROWS_CASE(4) WRQ_ROWS_CASE(5) WRQ_ROWS_CASE(6) WRQ_ROWS_CASE(7) WRQ_ROWS_CASE(8)
+    WRQ_ROWS_CASE(10) WRQ_ROWS_CASE(12) WRQ_ROWS_CASE(14) WRQ_ROWS_CASE(16)
+#undef WRQ_ROWS_CASE
+    default: return fail(WRQ_ERR_UNSUPPORTED, "no wave-owns-rows kernel for K = %u", K);
+    }
+}
+
 bool fast_ok(Quant quant, int in_f16, const MatmulArgs &a) {
     const uint32_t chunk = quant == kInt8 ? 16 : 32;
     const size_t xs = in_f16 ? 2 : 4;
@@ -899,6 +1074,9 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         const int ott = T == 1 ? 1 : T == 2 ? 2 : 4; // tokens per pass of the one-shot kernel
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
+        // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
+        const bool waverows = oneshot && quant == kInt8 && in_f16 && T == 1 && rows_kernel_has(args[i].K) &&
+                              ((uintptr_t)args[i].scale % 16 == 0) && tune(kTuneGemvWaveRows, 1);
         // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
         if (oneshot && quant == kInt8 && args[i].K / 16 > 512) rows = 8;
         // chunks per lane: cover a whole row at once when it is short enough
@@ -914,6 +1092,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (oneshot && quant == kInt8 && ott == 2 && !tune_is_set(kTuneGemvRows)) rows = 4;
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
+        if (waverows) rows = 4 * rows_per_wave((int)(args[i].K / 1024));
         while (i < n && g.n < (uint32_t)kMaxGroup) {
             const MatmulArgs &a = args[i];
             if (a.R == 0 || a.T == 0 || a.B == 0) {
@@ -930,6 +1109,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             }
             // the resident kernel builds one table per workgroup: its groups share the table tensor
             if (!oneshot && a.quant != g.quant && g.n) break;
+            if (waverows && g.n && (a.K != g.p[0].K || (uintptr_t)a.scale % 16 != 0)) break;
+            if (waverows && !g.n && (a.K != args[i].K || !rows_kernel_has(a.K) || (uintptr_t)a.scale % 16 != 0)) break;
             if (a.B > 1 && g.n + a.B > (uint32_t)kMaxGroup && g.n) break;
             if (lds + need * a.B > kGemvLdsBudget && g.n) break;
             // the batch axis unrolls into products of its own
@@ -986,6 +1167,11 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 8>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 8>(stream, g, nt, ott);
             else
                 s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 4>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 4>(stream, g, nt, ott);
+            if (s1 != WRQ_OK) return s1;
+            continue;
+        }
+        if (waverows && rows_kernel_has(g.p[0].K) && rows == 4 * rows_per_wave((int)(g.p[0].K / 1024))) {
+            const int s1 = launch_rows_int8_k(stream, g, g.p[0].K);
             if (s1 != WRQ_OK) return s1;
             continue;
         }
