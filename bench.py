@@ -178,10 +178,30 @@ def cpu_baseline(wrq, torch, layers, dec, quant, sample_layers, seconds=10.0):
     }
 
 
+def dominant_kernel(quant, tokens):
+    """The library kernel that takes most of a step of `tokens` tokens through the vec entry point."""
+    if quant == "int8":
+        if tokens == 1:
+            return "gemv_int8_rows_group_kernel"  # K = 4096 and 14336 are multiples of 1024: the wave-owns-rows kernel (single products: gemv_int8_rows_single_kernel)
+        return "gemv_int8_oneshot_kernel" if tokens <= 4 else "gemm_kernel"
+    return "gemv_nf4_oneshot_kernel" if tokens <= 2 else "gemm_kernel"
+
+
+# What a plain streaming read of the same bytes reaches in the same kind of graph on this machine (measured with the probe kernels):
+# a dependent dispatch costs about 1.45 us and the stream runs at about 7.2 TB/s.
+PLAIN_READ_DISPATCH_US, PLAIN_READ_GBPS = 1.45, 7200.0
+
+
+def plain_read_frac(nbytes, launches):
+    """Fraction of the HBM peak that `launches` plain reads of `nbytes` in total would reach: the ceiling of the launch structure."""
+    us = launches * PLAIN_READ_DISPATCH_US + nbytes / PLAIN_READ_GBPS / 1e3
+    return round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)
+
+
 def read_traffic(quant):
-    """HBM bytes per launch of the default decode step from profiles/gemv_<quant>_oneshot_decode_7b_hbm_traffic.txt
+    """HBM bytes per launch of the default decode step from profiles/gemv_<quant>_decode_7b_hbm_traffic.txt
     (the line `traffic_bytes_per_launch: N`), or None."""
-    path = os.path.join(ROOT, "profiles", f"gemv_{quant}_oneshot_decode_7b_hbm_traffic.txt")
+    path = os.path.join(ROOT, "profiles", f"gemv_{quant}_decode_7b_hbm_traffic.txt")
     try:
         with open(path) as f:
             for line in f:
@@ -200,7 +220,8 @@ def build_probe():
     """Compiles the measurement probes (bench_probe.hip: a plain copy and a streaming read) for gfx950."""
     import subprocess
 
-    cmd = ["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    hipcc, arch = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), os.environ.get("ARCH", "gfx950")  # the Makefile's variables
+    cmd = [hipcc, f"--offload-arch={arch}", "-O3", "-std=c++17", "-fPIC", "-shared",
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", PROBE_LIB, PROBE_SRC]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -679,7 +700,7 @@ def main():
     ap.add_argument("--no-group", action="store_true", help="one launch per product instead of grouped launches of independent products")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-layers", type=int, default=8)
-    ap.add_argument("--cpu-seconds", type=float, default=10.0,
+    ap.add_argument("--cpu-seconds", type=float, default=3.0,
                     help="seconds of CPU work for the cpu_baseline sample (whole passes over the sampled layers; at least one)")
     ap.add_argument("--probe", action="store_true",
                     help="also run the plain copy (256 MiB) and stream-read probes: the dispatches rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled against")
@@ -738,6 +759,15 @@ def main():
         return
     dec = Decode(wrq, torch, layers, C, H, args.tokens)
 
+    def graph_ms(step_fn):
+        """ms per step (device, wall) of `step_fn` captured once and replayed."""
+        step_fn()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            step_fn()
+        return time_steps(torch, gr.replay, args.steps, args.warmup)
+
     grouped = not args.no_group
     step = dec.step_grouped if grouped else dec.step
     if grouped:
@@ -781,9 +811,7 @@ def main():
     traffic = None
     if args.tokens == 1 and grouped and not args.with_head and args.layers == 32:
         traffic = read_traffic(args.quant)
-    # the vec entry point keeps runs of up to 4 (int8) or 2 (nf4) tokens on the decode kernels
-    on_decode_kernel = args.tokens <= (4 if args.quant == "int8" else 2)
-    kernel = f"gemv_{args.quant}_oneshot_kernel" if on_decode_kernel else "gemm_kernel"
+    kernel = dominant_kernel(args.quant, args.tokens)
     out = {
         "metric": "Int8/NF4 matmul HBM GB/s (% of peak); RWKV-7B-shape decode tok/s, batch 1",
         "value": round(tok_s, 2),
@@ -808,10 +836,35 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "traffic_source": None if traffic is None else f"tracked rocprofv3 --pmc summary profiles/gemv_{args.quant}_decode_7b_hbm_traffic.txt (not measured in this run)",
             "kernel": kernel, "launches_per_step": dec.launches,
             "avg_launch_us": round(launch_us, 3), "bytes_per_launch": nbytes // dec.launches,
+            "plain_read_model_frac": plain_read_frac(nbytes, dec.launches),
         },
     }
+    default_line = (args.quant == "int8" and args.tokens == 1 and grouped and not args.no_graph and not args.with_head)
+    if default_line:
+        # the literal call pattern of the reference's layer (src/runtime/v6.rs:806-938): eight separate products per layer
+        ms_u, wall_u = graph_ms(dec.step)
+        out["ungrouped"] = {"value": round(1e3 / wall_u, 2), "unit": "tok/s", "ms_per_step": round(wall_u, 4), "launches_per_step": 8 * len(layers),
+                            "frac": round(nbytes / (ms_u * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                            "plain_read_model_frac": plain_read_frac(nbytes, 8 * len(layers))}
+        # the other half of the metric: the same step with every layer NF4
+        del graph
+        layers4 = build_model(wrq, torch, "nf4", args.layers, C, H)
+        dec4 = Decode(wrq, torch, layers4, C, H, 1)
+        ms4, wall4 = graph_ms(dec4.step_grouped)
+        nbytes4 = dec4.bytes_per_step("nf4")
+        n4 = 4 * len(layers4)
+        out["nf4"] = {"value": round(1e3 / wall4, 2), "unit": "tok/s", "ms_per_step": round(wall4, 4), "dtype": "u4",
+                      "hbm_gbps": round(nbytes4 / (ms4 * 1e-3) / 1e9, 1), "bytes_per_step": nbytes4,
+                      "roofline": {"bound": "hbm", "achieved": round(nbytes4 / (ms4 * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                   "frac": round(nbytes4 / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                   "traffic": read_traffic("nf4") if args.layers == 32 else None,
+                                   "kernel": dominant_kernel("nf4", 1), "launches_per_step": n4,
+                                   "avg_launch_us": round(ms4 * 1e3 / n4, 3), "bytes_per_launch": nbytes4 // n4,
+                                   "plain_read_model_frac": plain_read_frac(nbytes4, n4)}}
+        del dec4, layers4
     # from some token count on the matrix cores bound a step, not HBM: 2 K R T flops per product against the
     # dense f16 peak take longer than the packed bytes against the HBM peak
     flops = 2.0 * args.tokens * len(layers) * (5 * C * C + 2 * C * H + C * C) + (2.0 * args.tokens * C * 65536 if args.with_head else 0.0)

@@ -11,11 +11,14 @@
  * buffer.  All pointers inside tensors are device pointers owned by the caller
  * and must stay valid until the stream has passed the call.  No entry point
  * allocates, frees or copies to the host.  All may be called from several threads at
- * once.  One limit on overlap in time: products on the matrix-core kernel (wrq_matmul_mat_*,
- * and wrq_matmul_vec_* from 5 tokens on, nf4: 3) may split K over workgroups and
- * then keep partial sums in one scratch array per device, so two such calls on different
- * streams of one device must not run at the same time; on one stream, and for shorter runs
- * on any streams, there is no such limit.
+ * once, and calls on different streams may overlap in time: products on the matrix-core kernel
+ * (wrq_matmul_mat_*, and wrq_matmul_vec_* from 5 tokens on, nf4: 3) may split K over workgroups
+ * and keep partial sums in library-owned scratch memory, of which every stream gets a slice of its
+ * own (4 per device, 32 MiB each, handed out in order of first use and kept until the process ends;
+ * products on further streams run unsplit: correct, slower).  A call recorded into a HIP graph keeps
+ * the slice of the stream it was captured on, so two graphs captured on ONE stream must not be
+ * replayed at the same time on different streams; wrq_matmul_mat_int8_noalloc has one fixed array
+ * per device and its calls must not overlap at all.
  *
  * Shapes use the reference's order, x fastest (src/tensor/shape.rs:97): a matrix
  * `[K, R, B, 1]` holds B * R rows of K contiguous elements.
@@ -101,9 +104,13 @@ int wrq_init(void);
  * shape.  An override pins one choice so that a test can reach every instantiation: keys are
  * "gemm_ntile", "gemm_mrt", "gemm_kg", "gemm_ksplit", "gemv_rows", "gemv_nt", "gemv_oneshot",
  * "vec_chunk_min_t", "gemm_tail" (0: a chunk grid a little above two workgroups per CU stays one
- * launch), ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
+ * launch), "gemv_waverows" (0: one-token int8 products stay off the wave-owns-rows kernel), ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
  * library first looks (wrq_init, or the first product) presets the same table; nothing on the launch
- * path reads the environment.  Overrides are process-wide: not for use while other threads launch.
+ * path reads the environment.  Overrides are process-wide and the launch path reads them without a lock,
+ * so a product library must not have them changed under it: once the process has launched any kernel of
+ * the library the call is refused with WRQ_ERR_UNSUPPORTED, unless WRQ_TEST_HOOKS=1 was in the environment
+ * when the library first looked (test and sweep processes set it; they change overrides only between
+ * launches of their own).
  */
 int wrq_debug_override(const char *key, int value);
 

@@ -6,6 +6,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+# a test process: wrq_debug_override stays usable after the first launch (read by the library when it first looks)
+os.environ.setdefault("WRQ_TEST_HOOKS", "1")
 
 
 def pytest_configure(config):

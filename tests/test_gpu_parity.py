@@ -3,6 +3,8 @@
 Bars: packed bytes and scale blocks bit-exact; products within
 |a - b| <= max(eps, eps * max(|a|, |b|)), eps = 2e-3 (f16 output, f32 accumulate).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,7 @@ from helpers import (ACTS, EPS, NF4_QUANT, assert_close, gen_f16, int8_dequant64
                      truth_matmul)
 
 pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 SEED = 0x57525100
 
@@ -350,7 +353,9 @@ def test_multi_token_vec_entry(gpu, oracle, kind, T):
 GEMM = [(2048, 2048, 32), (2048, 2048, 128), (2048, 2048, 256), (2048, 7168, 32), (7168, 2048, 128),
         (4096, 4096, 128), (2560, 2048, 64), (320, 64, 320), (768, 2688, 32), (2688, 768, 32), (2048, 512, 4),
         (2048, 512, 20), (2048, 65536, 32),
-        (4096, 14336, 128), (14336, 4096, 128), (4096, 4096, 256), (14336, 4096, 256), (2048, 65536, 256)]
+        (4096, 14336, 128), (14336, 4096, 128), (4096, 4096, 256), (14336, 4096, 256), (2048, 65536, 256),
+        # the remaining cells of config 3 (every shape at every token count)
+        (7168, 2048, 32), (2048, 7168, 128), (2048, 65536, 128), (2048, 7168, 256), (7168, 2048, 256)]
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
@@ -418,6 +423,36 @@ def test_f32_activations_that_are_no_f16_values(gpu, oracle, kind, entry, T):
     wp2, scale2, wdeq2 = pack(oracle, kind, w2)
     got2 = run(gpu, gpu_matrix(gpu, kind, wp2, scale2), x2, R, entry, np.float32)
     assert_close(got2, truth_matmul(wdeq2, x2), EPS, f"{kind} {entry} T={T} cancelling sums")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("T", [1, 16, 40])
+def test_f32_activations_beyond_the_f16_range(gpu, oracle, kind, T):
+    # f32 activations up to 65535 in magnitude: the matrix-core kernel splits them into two f16 halves and must keep both finite
+    # (f16 ends at 65504); the decode kernels take f32 as it is.  The same inputs through both entry points, against float64.
+    announce("f32 activations beyond the f16 range", kind, T)
+    K, R = 1024, 128
+    rng = np.random.default_rng(SEED + 79 + T)
+    w = gen_f16(rng, (R, K), 0.02)
+    x = rng.standard_normal((T, K), dtype=np.float32)
+    big = np.float32([65505.0, -65519.5, 65520.0, -65535.0, 65504.0, 60000.25, -65534.99, 32768.5])
+    for t in range(T):
+        cols = rng.choice(K, size=len(big), replace=False)
+        x[t, cols] = big * np.float32(1.0 if t % 2 == 0 else -1.0)
+    wp, scale, wdeq = pack(oracle, kind, w)
+    m = gpu_matrix(gpu, kind, wp, scale)
+    truth = truth_matmul(wdeq, x)
+    # terms of magnitude 65535 * |w| cancel in these sums.  f32 accumulation (the reference's too) is good to a few 1e-7 of the
+    # sum of the terms' magnitudes; the kernels factor the block's scale and offset out of the sum of codes
+    # (s * sum((1024 + u) x) + (min - 1024 s) * sum(x)), whose two parts are about 30 times a term, so the bar is the usual
+    # one widened by 1e-5 of that sum -- invisible at any activation a model produces, visible at 65535
+    terms = np.abs(x.astype(np.float64)) @ np.abs(wdeq.astype(np.float64)).T
+    for entry in (("vec", "mat") if T % 4 == 0 else ("vec",)):  # the mat entry takes multiples of 4 tokens
+        got = run(gpu, m, x, R, entry, np.float32)
+        assert np.isfinite(got).all(), f"{kind} {entry} T={T}: non-finite outputs"
+        bound = np.maximum(np.maximum(EPS, EPS * np.abs(truth)), 1e-5 * terms)
+        bad = np.abs(got - truth) > bound
+        assert not bad.any(), f"{kind} {entry} T={T}: {bad.sum()} outputs off, worst {np.abs(got - truth)[bad].max()} at bound {bound[bad].min()}"
 
 
 @pytest.mark.parametrize("kind", ["nf4", "int8"])
@@ -979,3 +1014,62 @@ def test_entry_points_from_several_threads(gpu, oracle):
     for j in range(4):
         for o in results[j]:
             assert_close(o, cases[j][2], EPS, f"thread {j}")
+
+
+def test_split_products_on_several_streams(gpu, oracle, overrides):
+    # split-K products keep partial sums in library scratch memory: every stream has a slice of its own, so products of
+    # different streams may overlap in time; a stream beyond the slices runs unsplit.  Six streams (more than the slices),
+    # each with its own weights and inputs and a pinned 8-way split, launched interleaved; every result against float64.
+    import torch
+
+    announce("split-K on several streams")
+    K, R, T = 4096, 1024, 32
+    rng = np.random.default_rng(SEED + 91)
+    overrides(gemm_ksplit=8)
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    cases = []
+    for j, _ in enumerate(streams):
+        kind = "int8" if j % 2 == 0 else "nf4"
+        w = gen_f16(rng, (R, K), 0.02)
+        x = gen_f16(rng, (T, K), 1.0)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        cases.append((gpu_matrix(gpu, kind, wp, scale), dev(x), truth_matmul(wdeq, x), []))
+    torch.cuda.synchronize()
+    for rep in range(12):
+        for st, (m, xd, _, outs) in zip(streams, cases):
+            with torch.cuda.stream(st):
+                out = torch.full((T, R), float("nan"), dtype=torch.float32, device="cuda")
+                m.matmul_mat_op(xd, out)
+                outs.append(out)
+    torch.cuda.synchronize()
+    for j, (_, _, truth, outs) in enumerate(cases):
+        for rep, out in enumerate(outs):
+            assert_close(host(out), truth, EPS, f"stream {j} repetition {rep}")
+
+
+def test_overrides_are_refused_after_the_first_launch_outside_tests():
+    # wrq_debug_override is a process-wide table that launches read without a lock: a process that has not declared itself
+    # a test (WRQ_TEST_HOOKS) may set overrides before its first launch and is refused afterwards
+    import subprocess
+    import sys
+
+    announce("override gate")
+    code = r'''
+import importlib, os, sys
+os.environ.pop("WRQ_TEST_HOOKS", None)
+import torch
+wrq = importlib.import_module("web-rwkv_amd")
+assert wrq.lib().wrq_init() == 0
+assert wrq.lib().wrq_debug_override(b"gemm_ksplit", 2) == 0          # before any launch: allowed
+assert wrq.lib().wrq_debug_override(b"gemm_ksplit", -1) == 0
+w = (torch.randn((64, 256), device="cuda") * 0.02).half()
+m = wrq.Matrix.quant_u8(w)                                           # launches the packer
+torch.cuda.synchronize()
+s = wrq.lib().wrq_debug_override(b"gemm_ksplit", 2)
+assert s == wrq.ERR_UNSUPPORTED, s
+assert b"WRQ_TEST_HOOKS" in wrq.lib().wrq_last_error()
+print("gate ok")
+'''
+    env = {k: v for k, v in os.environ.items() if k != "WRQ_TEST_HOOKS"}
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "gate ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]

@@ -70,11 +70,14 @@ constexpr int kStep = 128; // K elements per step
 #endif
 constexpr int kUnrollStages = WRQ_UNROLL_STAGES; // even
 
-// Partial tiles of split-K launches, in the tile order of the kernel.  One array per process and
-// GPU: split-K calls that overlap in time on one GPU (different streams) would race on it,
-// calls on one stream cannot.  Nothing in it outlives a call.
+// Partial tiles of split-K launches, in the tile order of the kernel.  Calls on one stream run one after the
+// other and share a slice; calls on different streams may overlap in time, so every stream that launches a split
+// product gets a slice of its own, kScratchSlices per device, handed out in order of first use and kept for the
+// life of the process.  A stream beyond those gets none: its products run unsplit (correct, slower).  Nothing in
+// a slice outlives a call.
 constexpr size_t kScratchFloats = 8u << 20; // 32 MiB: splits * R * T up to 8 Mi partial outputs
-__device__ __align__(256) float g_splitk_scratch[kScratchFloats];
+constexpr int kScratchSlices = 4;
+__device__ __align__(256) float g_splitk_scratch[kScratchSlices * kScratchFloats];
 
 // The same for wrq_matmul_mat_int8_noalloc: a file-scope array of its own (16 MiB), so that the entry
 // point for callers that cannot allocate never shares partial sums with the other entry points.  In
@@ -288,11 +291,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
                 st.x[p] = load128(src);
             } else {
                 const uint4 v0 = load128(src), v1 = load128(src + 4);
-                const float f[8] = {__uint_as_float(v0.x), __uint_as_float(v0.y), __uint_as_float(v0.z), __uint_as_float(v0.w),
-                                    __uint_as_float(v1.x), __uint_as_float(v1.y), __uint_as_float(v1.z), __uint_as_float(v1.w)};
-                float l[8];
+                const float raw[8] = {__uint_as_float(v0.x), __uint_as_float(v0.y), __uint_as_float(v0.z), __uint_as_float(v0.w),
+                                      __uint_as_float(v1.x), __uint_as_float(v1.y), __uint_as_float(v1.z), __uint_as_float(v1.w)};
+                // both halves stay finite f16 values: hi is clamped to the largest f16 magnitude before lo is formed, and lo
+                // saturates too.  Exact to 2^-22 for |x| <= 65535 (65504 + 31.98); beyond that the activation acts as +-65536
+                // instead of turning the sum into inf - inf.
+                float f[8], l[8];
 #pragma unroll
-                for (int e = 0; e < 8; e++) l[e] = (f[e] - h2f(f2h(f[e]))) * 2048.0f;
+                for (int e = 0; e < 8; e++) {
+                    f[e] = fminf(fmaxf(raw[e], -65504.0f), 65504.0f);
+                    l[e] = fminf(fmaxf((raw[e] - h2f(f2h(f[e]))) * 2048.0f, -65504.0f), 65504.0f);
+                }
                 st.x[p] = make_uint4(pack_h2(f[0], f[1]), pack_h2(f[2], f[3]), pack_h2(f[4], f[5]), pack_h2(f[6], f[7]));
                 st.xl[XLO ? p : 0] = make_uint4(pack_h2(l[0], l[1]), pack_h2(l[2], l[3]), pack_h2(l[4], l[5]), pack_h2(l[6], l[7]));
             }
@@ -751,9 +760,38 @@ float *device_array(std::atomic<float *> (&slots)[kMaxDevices], Lookup lookup) {
     return p;
 }
 
-float *scratch_ptr() {
+// Compute units of the current device (256 on MI355X); 0 if the query fails.
+uint32_t cu_count() {
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return (uint32_t)n;
+}
+
+float *scratch_base() {
     static std::atomic<float *> slots[kMaxDevices];
     return device_array(slots, [](void **q) { return hipGetSymbolAddress(q, HIP_SYMBOL(g_splitk_scratch)); });
+}
+
+// The slice of `stream` on the current device: the one it already owns, else the first free one (claimed with a
+// compare-and-swap, so two threads that meet here with different streams never share one); null when all are taken.
+float *scratch_ptr(hipStream_t stream) {
+    static std::atomic<uintptr_t> owner[kMaxDevices][kScratchSlices]; // stream handle + 1; 0 = free
+    float *base = scratch_base();
+    int dev = 0;
+    if (!base || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    const uintptr_t key = reinterpret_cast<uintptr_t>(stream) + 1;
+    for (int i = 0; i < kScratchSlices; i++) {
+        uintptr_t cur = owner[dev][i].load(std::memory_order_acquire);
+        if (cur == 0 && owner[dev][i].compare_exchange_strong(cur, key, std::memory_order_acq_rel)) cur = key;
+        if (cur == key) return base + (size_t)i * kScratchFloats;
+    }
+    return nullptr;
 }
 
 float *static_scratch_ptr() {
@@ -796,6 +834,16 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     // the partial tiles of all splits must fit the scratch array, whoever chose `ksplit`: the shared
     // array takes fewer splits then, the fixed one of the no-allocation entry point refuses
     const uint64_t cap = sp ? sp->floats : kScratchFloats;
+    // the slice of this stream, claimed when a launch first needs one; a stream that came after all slices were
+    // handed out runs its products unsplit
+    float *slice_cached = nullptr;
+    bool slice_asked = false;
+    auto slice_base = [&]() -> float * {
+        if (sp) return sp->base;
+        if (!slice_asked) slice_cached = scratch_ptr(stream), slice_asked = true;
+        return slice_cached;
+    };
+    if (ksplit > 1 && !slice_base()) ksplit = 1;
     if (sp && sp->strict && ksplit > 1 && slices * ksplit > cap)
         return fail(WRQ_ERR_SIZE, "split-K partial sums of this product need %llu bytes of scratch, the fixed array holds %llu",
                     (unsigned long long)(slices * ksplit * sizeof(float)), (unsigned long long)(cap * sizeof(float)));
@@ -804,7 +852,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     ga.k_per_split = steps_per * kStep;
     const uint32_t splits = (steps + steps_per - 1) / steps_per;
     if (splits > 1) {
-        float *base = sp ? sp->base : scratch_ptr();
+        float *base = slice_base();
         if (!base) return fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
         if (slices * splits > cap)
             return fail(WRQ_ERR_SIZE, "data size not match: %llu vs. %llu", (unsigned long long)(slices * splits), (unsigned long long)cap);
@@ -825,10 +873,13 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     // rest follows with K split over up to 8 times as many workgroups per tile, so that the second round is short
     // and wide.  One finish launch sums both kinds of tiles.
     const uint32_t wgs_all = total * splits;
-    if (NTILE >= 4 && a0.B == 1 && wgs_all > 512 && wgs_all <= 640 && steps % splits == 0 && tune(kTuneGemmTail, 1)) {
-        const uint32_t even = 512 / splits, rest = total - even; // tiles of the two launches
+    const uint32_t resident = 2 * cu_count(); // workgroups that run at a time at two per CU
+    // (f32 activations carry a second LDS tile: one workgroup per CU, the premise of the cut does not hold for them)
+    if (NTILE >= 4 && sizeof(XT) == 2 && a0.B == 1 && resident >= 64 && wgs_all > resident && wgs_all <= resident + resident / 4 && steps % splits == 0 &&
+        tune(kTuneGemmTail, 1)) {
+        const uint32_t even = resident / splits, rest = total - even; // tiles of the two launches
         uint32_t ks = 8 * splits;
-        while (ks > splits && (rest * ks > 512 || steps / ks < 2 || steps % ks != 0)) ks /= 2;
+        while (ks > splits && (rest * ks > resident || steps / ks < 2 || steps % ks != 0)) ks /= 2;
         // partial tiles of the rest lie like those of a product split `ks` times: room for every product with tiles in it
         auto planes = [&](int i, uint32_t k) { return ga.tile_begin[i] + nwg[i] > even ? k : splits > 1 ? splits : 0u; };
         auto need = [&](uint32_t k) {
@@ -837,7 +888,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
             return f;
         };
         while (ks > splits && need(ks) > cap) ks /= 2;
-        float *base = sp ? sp->base : scratch_ptr();
+        float *base = ks > splits ? slice_base() : nullptr;
         if (ks > splits && base) {
             GemmArgs gb = ga;
             uint64_t off = 0;
@@ -960,6 +1011,8 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
         if (ntile == 8) ntile = 4;
         if (mrt == 2 && ntile == 4) kg = 1;
         split_for();
+        ksplit = (uint32_t)tune(kTuneGemmKsplit, (int)ksplit); // a pinned split survives the adjustment
+        if (ksplit < 1) ksplit = 1;
     }
 #define WRQ_CASE(M, N, G) \
     if (mrt == M && ntile == N && kg == G) return launch_one<QUANT, XT, M, N, G>(stream, args, n, ksplit, sp);
@@ -975,7 +1028,7 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
 } // namespace
 
 int prepare_gemm_scratch() {
-    return scratch_ptr() && static_scratch_ptr() ? WRQ_OK : fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
+    return scratch_base() && static_scratch_ptr() ? WRQ_OK : fail(WRQ_ERR_DEVICE, "split-K scratch not resolvable");
 }
 
 int launch_gemm_noalloc(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs &a) {

@@ -33,6 +33,8 @@ const char *const kTuneNames[kTuneCount] = {"gemv_oneshot", "gemv_rows", "gemv_s
                                             "gemm_kg", "gemm_ksplit", "vec_chunk_min_t", "gemm_tail", "gemv_waverows"};
 std::atomic<int> g_tune[kTuneCount];
 std::once_flag g_tune_once;
+std::atomic<bool> g_test_hooks{false}; // WRQ_TEST_HOOKS was set when the library first looked: overrides stay allowed
+std::atomic<bool> g_launched{false};   // some kernel of the library has been launched by this process
 
 void tune_load_env() {
     for (int k = 0; k < kTuneCount; k++) {
@@ -43,6 +45,8 @@ void tune_load_env() {
         const char *e = getenv(name);
         g_tune[k].store((e && *e) ? atoi(e) : -1, std::memory_order_relaxed);
     }
+    const char *hooks = getenv("WRQ_TEST_HOOKS");
+    g_test_hooks.store(hooks && *hooks && atoi(hooks) != 0, std::memory_order_relaxed);
 }
 } // namespace
 
@@ -59,6 +63,10 @@ bool tune_is_set(TuneKey key) {
 
 int tune_set(const char *name, int value) {
     std::call_once(g_tune_once, tune_load_env);
+    // the table is process-wide and the launch path reads it without a lock: once launches have begun, only a
+    // process that declared itself a test (WRQ_TEST_HOOKS=1 in its environment at load time) may still change it
+    if (g_launched.load(std::memory_order_relaxed) && !g_test_hooks.load(std::memory_order_relaxed))
+        return fail(WRQ_ERR_UNSUPPORTED, "overrides are refused once a kernel has been launched (WRQ_TEST_HOOKS=1 in the environment keeps them)");
     for (int k = 0; k < kTuneCount; k++)
         if (strcmp(name, kTuneNames[k]) == 0) {
             g_tune[k].store(value < 0 ? -1 : value, std::memory_order_relaxed);
@@ -68,6 +76,7 @@ int tune_set(const char *name, int value) {
 }
 
 int check_launch(const char *what) {
+    g_launched.store(true, std::memory_order_relaxed);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(WRQ_ERR_DEVICE, "%s: %s", what, hipGetErrorString(e));
     return WRQ_OK;
@@ -237,8 +246,9 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
     // tokens against 2.8 ms; f16 head: 97 us at 4 tokens against 120); longer runs go to the
     // matrix-core kernel.
     const uint64_t chunk_min_t = (uint64_t)tune(kTuneVecChunkMinT, quant == kNf4 ? 3 : 5);
-    // f32 activations are rounded to f16 by the matrix-core kernel: keep them on the exact VALU
-    // kernels below 16 tokens
+    // f32 activations cost the matrix-core kernel a second LDS tile and a second product chain (they are split
+    // into two f16 halves there, exact to 2^-22 for |x| <= 65535): below 16 tokens the VALU kernels, which take
+    // f32 as it is, are the faster choice and have no range limit
     const bool chunk = entry == kMat ? true : n >= (in_f16 ? chunk_min_t : (uint64_t)16);
     out.in_f16 = in_f16;
     out.mfma = chunk && mfma_ok;
