@@ -699,6 +699,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-group", action="store_true", help="one launch per product instead of grouped launches of independent products")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--main-only", action="store_true", help="leave the ungrouped and NF4 figures out of the default line (for profiler runs of one workload)")
     ap.add_argument("--cpu-sample-layers", type=int, default=8)
     ap.add_argument("--cpu-seconds", type=float, default=3.0,
                     help="seconds of CPU work for the cpu_baseline sample (whole passes over the sampled layers; at least one)")
@@ -842,7 +843,7 @@ def main():
             "plain_read_model_frac": plain_read_frac(nbytes, dec.launches),
         },
     }
-    default_line = (args.quant == "int8" and args.tokens == 1 and grouped and not args.no_graph and not args.with_head)
+    default_line = (args.quant == "int8" and args.tokens == 1 and grouped and not args.no_graph and not args.with_head and not args.main_only)
     if default_line:
         # the literal call pattern of the reference's layer (src/runtime/v6.rs:806-938): eight separate products per layer
         ms_u, wall_u = graph_ms(dec.step)

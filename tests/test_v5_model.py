@@ -93,3 +93,32 @@ def test_v5_model_packed_token_shifts_equal_the_op_list(gpu):
         assert np.array_equal(a, b), f"logits after a run of {len(tokens)}"
     for sa, sb in zip(models[0].state, models[1].state):
         assert torch.equal(sa, sb)
+
+
+@pytest.mark.gpu
+def test_sparse_input_statistics_of_ffn_value(gpu):
+    # `matmul_vec_*` with SPARSE_INPUT (src/shaders/matmul_vec_int8.wgsl:80-84, matmul_vec_nf4.wgsl:110-120) skips a group of
+    # 4 (int8) or 8 (nf4) weights per row when all their activations are zero; the one call site is ffn.value, whose input
+    # is the squared ReLU of ffn.key (src/runtime/v5.rs:854-859).  The library accepts the flag and skips nothing: its
+    # kernels are bound by the weight bytes crossing HBM, which only aligned runs of zeros as long as a memory sector of
+    # a weight row (64 activations for int8) could save.  This measures, on the activations of this model's decode steps,
+    # how often such runs occur.
+    import torch
+
+    v5 = importlib.import_module(gpu.__name__ + ".v5")
+    L, H, S, hidden, V = 12, 12, 64, 2688, 65536
+    rng = np.random.default_rng(SEED)
+    model = v5.Model(torch, v5.random_model_weights(rng, L, H * S, H, S, hidden, V), "int8", H, S, hidden, 2)
+    seen = []
+    model.hook = lambda i, buf: seen.append(buf.ffn_k.detach().clone())
+    run = [int(t) for t in rng.integers(0, V, 32)]
+    for step in range(17):
+        logits = model.run(run, 1)
+        run = [int(logits.argmax())]
+    decode = [k.cpu().numpy().reshape(-1, hidden) for k in seen[L:]]  # the 16 one-token runs
+    k = np.concatenate(decode)  # [16 * 12, hidden]
+    zero = k == 0
+    stats = {g: float(zero.reshape(k.shape[0], hidden // g, g).all(axis=2).mean()) for g in (4, 8, 16, 64)}
+    print("ffn.value input: zero elements", float(zero.mean()), "all-zero aligned groups of 4 / 8 / 16 / 64:", stats, flush=True)
+    assert 0.3 < zero.mean() < 0.7  # a squared ReLU of a roughly symmetric pre-activation
+    assert stats[4] < 0.2 and stats[64] == 0.0  # zeros do not cluster: no sector of a weight row could be skipped

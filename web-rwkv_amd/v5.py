@@ -181,6 +181,7 @@ class Model:
         self.state = [torch.zeros((slots, S + 2, self.C), dtype=torch.float32, device="cuda") for _ in self.layers]
         self.vocab = weights["head"].shape[0]
         self._buffers, self._shifts = {}, {}
+        self.hook = None  # called as hook(layer index, run buffers) behind every layer, like a `Hook::PostFfn` of the reference (src/runtime/v5.rs:880-885)
 
     def buffers(self, A):
         """The buffers of runs of `A` tokens, made once per run length (`checkout_buffer`, src/runtime/v5.rs:497-510)."""
@@ -206,6 +207,8 @@ class Model:
                 dispatch_layer_packed(layer, self._shifts[A][i], buf, st, cursors, A, self.H, self.S, rescale_now=(i + 1) % self.rescale == 0)
             else:
                 dispatch_layer(layer, buf, st, cursors, A, self.H, self.S, rescale_now=(i + 1) % self.rescale == 0)
+            if self.hook is not None:
+                self.hook(i, buf)
         LayerOp.blit(buf.x, head_x, input_view=((C, 1, 1), (C, A, 1), (0, A - 1, 0)))
         LayerOp.layer_norm(self.t["head_ln_w"], self.t["head_ln_b"], head_x, LN_EPS)
         self.head.matmul_op(head_x, logits, ACT_NONE, turbo(1))
