@@ -269,7 +269,9 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
         xs.append(x)
         truths.append(truth_matmul(wdeq, x))
         wants.append(oracle.matmul_vec_int8(wp, scale, x, out_dtype=np.float32)[0])
-    for waverows in (1, 0):
+    # 2: the wave-owns-rows kernel at every K it is built for; 1: the default choice (beyond K = 8192 the K-split kernel);
+    # 0: the one-shot kernel they replace
+    for waverows in (2, 1, 0):
         overrides(gemv_waverows=waverows)
         for m, x, R, truth, want in zip(mats, xs, rows, truths, wants):
             for out_dtype in (np.float16, np.float32):
@@ -284,7 +286,7 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
                               for i, (m, x, o) in enumerate(zip(mats, xs, outs))])
         for i, (o, truth) in enumerate(zip(outs, truths)):
             assert_close(host(o).astype(np.float32), np.square(np.maximum(truth, 0.0)) if i == 2 else truth, EPS, f"K={K} group member {i}")
-    overrides(gemv_waverows=1)
+    overrides(gemv_waverows=2)
     # a z-offset input view and an offset output view (v6: att_sx.view(.., .., i, ..), src/runtime/v6.rs:806-829)
     parent = gen_f16(rng, (5, 1, K), 1.0)
     out = torch.full((3, 3, rows[0]), -7.0, dtype=torch.float32, device="cuda")

@@ -606,6 +606,71 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_
                             p.out_f16, p.act, task - p.task_begin, xs);
 }
 
+// int8, one token, f16 activations, long rows (K = WK * 1024, 8192 < K <= 16384): the WK waves of a workgroup split K, every wave
+// takes all RWG rows of the task over its 1024 elements -- one 16-byte chunk per lane and row, the lane's 16 activations in
+// registers for all rows (each activation crosses into the workgroup once, no LDS staging), one (min, max) word per chunk.
+// Request order: activations, scale words, weights; rows are consumed in arrival order; the partial sums of the waves meet in
+// LDS behind one barrier.  Same task numbering and argument passing as the wave-owns-rows kernel.
+template <int RWG, int WK>
+__global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
+                                                                  const uint32_t total_tasks, const uint32_t flags) {
+    constexpr int K = WK * 1024;
+    __shared__ float red[WK][RWG];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 64 / RWG);
+    const uint32_t row0 = task * RWG;
+    const uint32_t k0 = wave * 1024 + lane * 16; // first element of this lane's chunk
+    const uint4 *xp = reinterpret_cast<const uint4 *>(x + k0);
+    const uint4 x0 = load128(xp), x1 = load128(xp + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t sc[RWG];
+    const uint8_t *wrow[RWG];
+#pragma unroll
+    for (int r = 0; r < RWG; r++) {
+        const uint32_t row = min(row0 + r, R - 1); // rows past the end repeat the last one and are not stored
+        wrow[r] = w + (uint64_t)row * K + k0;
+        sc[r] = mm[(uint64_t)row * (K / 128) + (k0 >> 7)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint4 wv[RWG];
+#pragma unroll
+    for (int r = 0; r < RWG; r++) wv[r] = load128_stream(wrow[r]);
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t xd[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+    float sx = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) sx = dot2(xd[q], 0x3c003c00u, sx); // (1.0, 1.0)
+    float mine = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RWG; r++) {
+        const uint32_t wd[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+        uint32_t code[8]; // f16 pairs (1024 + u0, 1024 + u1)
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            code[2 * d] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04010400u);
+            code[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04030402u);
+        }
+        const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
+        const float mx = h2f((uint16_t)(sc[r] >> 16));
+        const float s = (mx - mn) * (1.0f / 255.0f);
+        const float c0 = fmaf(-1024.0f, s, mn);
+        float pr = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 8; q++) pr = dot2(code[q], xd[q], pr);
+        const float sum = wave_sum(fmaf(s, pr, c0 * sx));
+        if (lane == (uint32_t)r) mine = sum;
+    }
+    if (lane < (uint32_t)RWG) red[wave][lane] = mine;
+    __syncthreads();
+    if (tid < (uint32_t)RWG) {
+        float s = 0.0f;
+#pragma unroll
+        for (int q = 0; q < WK; q++) s += red[q][tid];
+        if (row0 + tid < R) store_out(out, (int)(flags & 1u), row0 + tid, act_apply((int)(flags >> 1), s));
+    }
+}
+
 // nf4, one token: the same one-shot shape (one workgroup per task of ROWS rows, NT lanes along
 // K, every load of the task requested up front).  A lane holds 32 weights (16 packed bytes) of
 // each row and the 32 activations they meet.  A packed byte is two weights: a 256-entry LDS
@@ -1000,11 +1065,40 @@ int launch_rows_int8(hipStream_t stream, const GemvGroup &g) {
 constexpr int rows_per_wave(int bpl) { return bpl <= 2 ? 2 : 1; }
 
 // K / 1024 values the wave-owns-rows kernel is built for.
-bool rows_kernel_has(uint32_t K) {
+bool rows_kernel_built(uint32_t K) {
     if (K % 1024 != 0) return false;
     switch (K / 1024) {
     case 1: case 2: case 3: case 4: case 5: case 6: case 7: case 8: case 10: case 12: case 14: case 16: return true;
     default: return false;
+    }
+}
+
+// ... and those it is used for unless an override says otherwise (gemv_waverows = 2 takes every built one).  Measured against
+// the one-shot kernel, cold, one product: 2048 x 2048 2.72 against 3.22 us, 2048 -> 7168 4.40 / 5.07, 7168 -> 2048 4.68 / 5.19,
+// 4096 x 4096 4.74 / 5.34, 4096 -> 14336 10.87 / 11.53, 2048 -> 65536 21.4 / 22.4; 14336 -> 4096 12.9 against 12.15: with rows
+// that long every wave pulls 28 KiB of activations through LDS for one row, and the one-shot kernel, whose lanes keep
+// their slice of the activations in registers for 8 rows, stays ahead.
+bool rows_kernel_has(uint32_t K) { return rows_kernel_built(K) && (K <= 8192 || tune(kTuneGemvWaveRows, 1) == 2); }
+
+// Long rows of a single product: the K-split kernel (8 rows per task).
+bool ksplit_kernel_has(uint32_t K) { return K % 1024 == 0 && (K == 10240 || K == 12288 || K == 14336 || K == 16384); }
+
+template <int WK>
+int launch_ksplit_int8(hipStream_t stream, const GemvGroup &g) {
+    const GemvProblem &p = g.p[0];
+    hipLaunchKernelGGL((gemv_int8_ksplit_kernel<8, WK>), dim3(g.total_tasks), dim3(WK * 64), 0, stream, p.w,
+                       reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R, g.total_tasks,
+                       (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1));
+    return check_launch("matmul_vec_int8");
+}
+
+int launch_ksplit_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
+    switch (K / 1024) {
+    case 10: return launch_ksplit_int8<10>(stream, g);
+    case 12: return launch_ksplit_int8<12>(stream, g);
+    case 14: return launch_ksplit_int8<14>(stream, g);
+    case 16: return launch_ksplit_int8<16>(stream, g);
+    default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u", K);
     }
 }
 
@@ -1077,6 +1171,9 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
         const bool waverows = oneshot && quant == kInt8 && in_f16 && T == 1 && rows_kernel_has(args[i].K) &&
                               ((uintptr_t)args[i].scale % 16 == 0) && tune(kTuneGemvWaveRows, 1);
+        // ... and long rows (8192 < K <= 16384, a multiple of 2048): the K-split kernel, one product per launch
+        const bool ksplit = oneshot && !waverows && quant == kInt8 && in_f16 && T == 1 && ksplit_kernel_has(args[i].K) && args[i].B == 1 &&
+                            tune(kTuneGemvWaveRows, 1);
         // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
         if (oneshot && quant == kInt8 && args[i].K / 16 > 512) rows = 8;
         // chunks per lane: cover a whole row at once when it is short enough
@@ -1093,6 +1190,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
         if (waverows) rows = 4 * rows_per_wave((int)(args[i].K / 1024));
+        if (ksplit) rows = 8;
         while (i < n && g.n < (uint32_t)kMaxGroup) {
             const MatmulArgs &a = args[i];
             if (a.R == 0 || a.T == 0 || a.B == 0) {
@@ -1109,6 +1207,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             }
             // the resident kernel builds one table per workgroup: its groups share the table tensor
             if (!oneshot && a.quant != g.quant && g.n) break;
+            if (ksplit && g.n) break; // one product per launch
             if (waverows && g.n && (a.K != g.p[0].K || (uintptr_t)a.scale % 16 != 0)) break;
             if (waverows && !g.n && (a.K != args[i].K || !rows_kernel_has(a.K) || (uintptr_t)a.scale % 16 != 0)) break;
             if (a.B > 1 && g.n + a.B > (uint32_t)kMaxGroup && g.n) break;
@@ -1167,6 +1266,11 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                 s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 8>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 8>(stream, g, nt, ott);
             else
                 s1 = in_f16 ? launch_oneshot_nf4_nt<__half, 4>(stream, g, nt, ott) : launch_oneshot_nf4_nt<float, 4>(stream, g, nt, ott);
+            if (s1 != WRQ_OK) return s1;
+            continue;
+        }
+        if (ksplit && g.n == 1 && ksplit_kernel_has(g.p[0].K) && rows == 8) {
+            const int s1 = launch_ksplit_int8_k(stream, g, g.p[0].K);
             if (s1 != WRQ_OK) return s1;
             continue;
         }

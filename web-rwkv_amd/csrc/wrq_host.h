@@ -61,7 +61,7 @@ enum TuneKey {
     kTuneGemmKsplit,
     kTuneVecChunkMinT, // vec_chunk_min_t: first token count the decode entry sends to the chunk kernel
     kTuneGemmTail,     // gemm_tail: 0 keeps a grid a little above two workgroups per CU in one launch
-    kTuneGemvWaveRows, // gemv_waverows: 0 keeps one-token int8 products off the wave-owns-rows kernel
+    kTuneGemvWaveRows, // gemv_waverows: 0 keeps one-token int8 products off the wave-owns-rows kernel, 2 sends every K it is built for there
     kTuneGemmPrio,     // gemm_prio: 0 leaves the wave priority alone around the matrix work of a chunk step (default: raised)
     kTuneCount
 };
