@@ -10,7 +10,8 @@
 // The discount (2^-(layer / rescale) on att.output and ffn.value) multiplies in f32 and rounds to
 // f16 (nearest even, subnormals kept: `half::f16::from_f32`) before the matrix is packed; the loader does
 // it on the device, `Loader::discounted` is the same expression on the host.
-// Low-rank adapters blended in at load time (`lora_matrices`, `lora_vectors`) are not built.
+//   Lora, LoraBlend, lora_matrices, lora_vectors      src/runtime/loader.rs:76-167, :328-386 (adapters blended in at load time:
+//                                                     `blend_lora` with alpha / rank for the low-rank halves, `blend` for whole tensors)
 //
 // The file format (safetensors): 8 bytes little-endian header length N, N bytes of JSON
 // `{ name: { "dtype", "shape", "data_offsets": [begin, end] }, "__metadata__": {..} }`, then the
@@ -24,6 +25,8 @@
 #include <unistd.h>
 
 #include <map>
+#include <regex>
+#include <sstream>
 
 #include "wrq.hpp"
 
@@ -290,37 +293,113 @@ class SafeTensors {
 
 enum class Quant { None, Int8, NF4, SF4 }; // src/runtime/model.rs:122-135
 
+// Low-rank adapters blended into the weights while they are loaded (src/runtime/loader.rs:76-167).
+// A blend pattern is a regular expression over tensor names and a factor; of the patterns of one adapter that match a name,
+// the LAST one counts (`rfind`, loader.rs:336-343).
+struct LoraBlendPattern {
+    std::regex pattern;
+    float alpha;
+    LoraBlendPattern(const std::string &p, float a) : pattern(p, std::regex::ECMAScript), alpha(a) {}
+};
+
+struct LoraBlend : std::vector<LoraBlendPattern> {
+    // replaces all vectors, adds to all matrices with `alpha` (loader.rs:120-124)
+    static LoraBlend full(float alpha) { return LoraBlend().add_nominal(1.0f).add_matrices(alpha); }
+    LoraBlend &add_nominal(float alpha) { // every tensor, interpolated with `alpha` (loader.rs:126-132)
+        emplace_back(".+", alpha);
+        return *this;
+    }
+    LoraBlend &add_matrices(float alpha) { // the matrices of the layers (loader.rs:134-145)
+        emplace_back("blocks\\.([0-9]+)\\.(att|ffn)\\.(key|value|receptance|gate|output)\\.weight", alpha);
+        return *this;
+    }
+    LoraBlend &add_layer(size_t layer, float alpha) { // ... of one layer (loader.rs:147-160)
+        emplace_back("blocks\\." + std::to_string(layer) + "\\.(att|ffn)\\.(key|value|receptance|gate|output)\\.weight", alpha);
+        return *this;
+    }
+    // the factor that applies to `name`, if any pattern matches
+    bool factor_of(const std::string &name, float &alpha) const {
+        for (auto it = rbegin(); it != rend(); ++it)
+            if (std::regex_search(name, it->pattern)) {
+                alpha = it->alpha;
+                return true;
+            }
+        return false;
+    }
+};
+
+struct Lora {
+    const SafeTensors *data; // the adapter file; outlives the loader
+    LoraBlend blend;
+};
+
 class Loader {
   public:
-    Loader(const SafeTensors &model, Queue &queue) : model_(model), queue_(queue) {}
+    Loader(const SafeTensors &model, Queue &queue, std::vector<Lora> lora = {}) : model_(model), queue_(queue), lora_(std::move(lora)) {}
 
-    // src/runtime/loader.rs:389-392 and `Shape::from_slice_rev`: [out, in] in the file is [in, out, 1, 1] here
-    Shape tensor_shape(const std::string &name) const {
-        const auto s = model_.shape(name);
-        if (s.empty() || s.size() > 4) throw LoaderError("`" + name + "`: " + std::to_string(s.size()) + " axes (1 to 4 are tensors)");
-        uint32_t d[4] = {1, 1, 1, 1};
-        for (size_t i = 0; i < s.size(); i++) {
-            if (s[s.size() - 1 - i] > 0xffffffffull) throw LoaderError("`" + name + "`: extent beyond 32 bits");
-            d[i] = (uint32_t)s[s.size() - 1 - i];
+    // What `lora_matrices` finds for a matrix name (loader.rs:355-386): per adapter whose last matching pattern gives a
+    // factor and whose file holds `<name without .weight>.lora.0` ([?, rank] in the file) and `.lora.1`.
+    struct LoraMatrixRef {
+        std::string x, y; // tensor names in the adapter file
+        const SafeTensors *data;
+        uint32_t rank;
+        float alpha;
+    };
+    static std::string lora_stem(const std::string &name) {
+        // `name.split('.').filter(|x| !x.contains("weight")).join(".")` (loader.rs:368)
+        std::string out, part;
+        std::istringstream in(name);
+        while (std::getline(in, part, '.'))
+            if (part.find("weight") == std::string::npos) out += (out.empty() ? "" : ".") + part;
+        return out;
+    }
+    std::vector<LoraMatrixRef> lora_matrices(const std::string &name) const {
+        std::vector<LoraMatrixRef> out;
+        for (const Lora &l : lora_) {
+            float alpha;
+            if (!l.blend.factor_of(name, alpha)) continue;
+            const std::string stem = lora_stem(name);
+            const std::string x = stem + ".lora.0", y = stem + ".lora.1";
+            if (!l.data->contains(x) || !l.data->contains(y)) continue;
+            const auto shape = l.data->shape(x);
+            if (shape.size() < 2 || shape[1] == 0 || shape[1] > 0xffffffffull) throw LoaderError("`" + x + "`: an adapter half has two axes");
+            out.push_back(LoraMatrixRef{x, y, l.data, (uint32_t)shape[1], alpha});
         }
-        return Shape(d[0], d[1], d[2], d[3]);
+        return out;
+    }
+    // ... and `lora_vectors` (loader.rs:330-353): a tensor of the same name in the adapter file
+    struct LoraVectorRef {
+        const SafeTensors *data;
+        float alpha;
+    };
+    std::vector<LoraVectorRef> lora_vectors(const std::string &name) const {
+        std::vector<LoraVectorRef> out;
+        for (const Lora &l : lora_) {
+            float alpha;
+            if (l.blend.factor_of(name, alpha) && l.data->contains(name)) out.push_back(LoraVectorRef{l.data, alpha});
+        }
+        return out;
     }
 
-    // src/runtime/loader.rs:568-592 (no adapters blended in)
+    // src/runtime/loader.rs:389-392 and `Shape::from_slice_rev`: [out, in] in the file is [in, out, 1, 1] here
+    Shape tensor_shape(const std::string &name) const { return shape_of(model_, name); }
+
+    // src/runtime/loader.rs:568-592: the file's matrix, then every adapter blended in on the device
+    // (`blend_lora` with factor alpha / rank for the low-rank halves, `blend` with alpha for a tensor of the same name)
     TensorGpu<f16> load_matrix_f16(const std::string &name) const {
-        const auto bytes = f16_bytes(name);
-        const Shape shape = tensor_shape(name);
-        TensorGpu<f16> t = TensorGpu<f16>::init(shape);
-        if (hipMemcpy(t.data(), bytes.first, bytes.second, hipMemcpyHostToDevice) != hipSuccess) throw TensorError(WRQ_ERR_DEVICE, "hipMemcpy failed");
+        TensorGpu<f16> t = upload_f16(model_, name);
+        blend_adapters(t, name, 1.0f);
         return t;
     }
     // src/runtime/loader.rs:594-621, :651-686: x -> f16(discount * f32(x))
     // The file's bytes go to the device as they are and the discount is applied there (`TensorOp::affine`
     // multiplies in f32 and rounds to f16 like the host expression): a host loop over the elements would
     // bound the load at under 1 GB/s against 20+ GB/s for the copy.
+    // The adapters join the discounted matrix with factors discount * alpha (/ rank), as in the reference (loader.rs:605-617).
     TensorGpu<f16> load_matrix_f16_discount(const std::string &name, float discount) const {
-        TensorGpu<f16> t = load_matrix_f16(name);
+        TensorGpu<f16> t = upload_f16(model_, name);
         queue_.submit(TensorOp::affine(t, discount, 0.0f));
+        blend_adapters(t, name, discount);
         return t;
     }
     // the same values computed on the host (no device): the reference expression, element by element
@@ -340,10 +419,41 @@ class Loader {
     }
 
   private:
-    std::pair<const uint8_t *, size_t> f16_bytes(const std::string &name) const {
-        if (model_.entry(name).dtype != "F16") // `TensorCpu::<f16>::from_reader`: TensorErrorKind::Type
-            throw TensorError(WRQ_ERR_TYPE, "`" + name + "`: data type mismatch (" + model_.entry(name).dtype + ", expected F16)");
-        return model_.tensor(name);
+    std::pair<const uint8_t *, size_t> f16_bytes(const std::string &name) const { return f16_bytes_of(model_, name); }
+    static std::pair<const uint8_t *, size_t> f16_bytes_of(const SafeTensors &file, const std::string &name) {
+        if (file.entry(name).dtype != "F16") // `TensorCpu::<f16>::from_reader`: TensorErrorKind::Type
+            throw TensorError(WRQ_ERR_TYPE, "`" + name + "`: data type mismatch (" + file.entry(name).dtype + ", expected F16)");
+        return file.tensor(name);
+    }
+    static Shape shape_of(const SafeTensors &file, const std::string &name) {
+        const auto s = file.shape(name);
+        if (s.empty() || s.size() > 4) throw LoaderError("`" + name + "`: " + std::to_string(s.size()) + " axes (1 to 4 are tensors)");
+        uint32_t d[4] = {1, 1, 1, 1};
+        for (size_t i = 0; i < s.size(); i++) {
+            if (s[s.size() - 1 - i] > 0xffffffffull) throw LoaderError("`" + name + "`: extent beyond 32 bits");
+            d[i] = (uint32_t)s[s.size() - 1 - i];
+        }
+        return Shape(d[0], d[1], d[2], d[3]);
+    }
+    static TensorGpu<f16> upload_f16(const SafeTensors &file, const std::string &name) {
+        const auto bytes = f16_bytes_of(file, name);
+        TensorGpu<f16> t = TensorGpu<f16>::init(shape_of(file, name));
+        if (hipMemcpy(t.data(), bytes.first, bytes.second, hipMemcpyHostToDevice) != hipSuccess) throw TensorError(WRQ_ERR_DEVICE, "hipMemcpy failed");
+        return t;
+    }
+    void blend_adapters(const TensorGpu<f16> &t, const std::string &name, float scale) const {
+        for (const LoraMatrixRef &l : lora_matrices(name)) {
+            const TensorGpu<float> factor = TensorGpu<float>::from_data(Shape(4, 1, 1, 1), {scale * l.alpha / (float)l.rank, 1.0f, 0.0f, 0.0f});
+            const TensorGpu<f16> x = upload_f16(*l.data, l.x), y = upload_f16(*l.data, l.y);
+            queue_.submit(TensorOp::blend_lora(factor, TensorGpuView<f16>(x), TensorGpuView<f16>(y), TensorGpuView<f16>(t)));
+            queue_.sync(); // the adapter halves and the factor are released here
+        }
+        for (const LoraVectorRef &l : lora_vectors(name)) {
+            const TensorGpu<float> factor = TensorGpu<float>::from_data(Shape(4, 1, 1, 1), {scale * l.alpha, 1.0f, 0.0f, 0.0f});
+            const TensorGpu<f16> v = upload_f16(*l.data, name);
+            queue_.submit(TensorOp::blend(factor, v, t));
+            queue_.sync();
+        }
     }
     Matrix pack(const TensorGpu<f16> &buffer, Quant quant) const {
         switch (quant) {
@@ -356,6 +466,7 @@ class Loader {
     }
     const SafeTensors &model_;
     Queue &queue_;
+    std::vector<Lora> lora_;
 };
 
 } // namespace wrq

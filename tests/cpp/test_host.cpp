@@ -661,6 +661,59 @@ static void test_loader_host(const std::string &model_path, const std::string &d
     EXPECT(threw);
 }
 
+// Adapter plumbing on the host: which pattern counts, how a matrix name maps to the adapter's tensor names (loader.rs:328-386)
+static void test_lora_host(const std::string &model_path, const std::string &dir) {
+    SafeTensors model(model_path), adapter(dir + "/lora.st");
+    Queue queue;
+    EXPECT(Loader::lora_stem("blocks.6.att.output.weight") == "blocks.6.att.output");
+    EXPECT(Loader::lora_stem("head.weight") == "head");
+    float a = 0.0f;
+    EXPECT(LoraBlend::full(0.25f).factor_of("blocks.6.att.output.weight", a) && a == 0.25f); // the last matching pattern counts
+    EXPECT(LoraBlend::full(0.25f).factor_of("blocks.6.att.time_first", a) && a == 1.0f);     // only the nominal pattern matches
+    EXPECT(!LoraBlend().add_layer(5, 0.5f).factor_of("blocks.6.att.output.weight", a));
+    EXPECT(LoraBlend().add_layer(6, 0.5f).factor_of("blocks.6.ffn.value.weight", a) && a == 0.5f);
+    Loader loader(model, queue, {Lora{&adapter, LoraBlend::full(0.5f)}});
+    const auto ms = loader.lora_matrices("blocks.6.ffn.value.weight");
+    EXPECT(ms.size() == 1 && ms[0].rank == 8 && ms[0].alpha == 0.5f && ms[0].x == "blocks.6.ffn.value.lora.0" && ms[0].y == "blocks.6.ffn.value.lora.1");
+    EXPECT(loader.lora_matrices("blocks.6.att.output.weight").empty()); // the adapter file has no halves for it
+    const auto vs = loader.lora_vectors("blocks.6.att.output.weight");
+    EXPECT(vs.size() == 1 && vs[0].alpha == 0.5f); // ... but a whole tensor of that name
+    EXPECT(loader.lora_vectors("blocks.6.ffn.value.weight").empty());
+}
+
+// An adapter blended in while loading: out = f16(alpha / rank * xa^T xb + w) for the low-rank halves, f16(alpha * v + w) for a
+// whole tensor, with the discount in both factors; against numpy's float32 evaluation of the same expressions (one f16 ulp:
+// the order of the rank-8 sum is free)
+static void test_lora_gpu(const std::string &model_path, const std::string &dir) {
+    SafeTensors model(model_path), adapter(dir + "/lora.st");
+    Queue queue;
+    Loader loader(model, queue, {Lora{&adapter, LoraBlend::full(0.5f)}});
+    struct Case {
+        const char *name, *tag;
+        float discount;
+    };
+    for (const Case &c : {Case{"blocks.6.ffn.value.weight", ".lora.f16", 1.0f}, Case{"blocks.6.ffn.value.weight", ".lora_half.f16", 0.5f},
+                          Case{"blocks.6.att.output.weight", ".lora.f16", 1.0f}, Case{"blocks.6.att.output.weight", ".lora_half.f16", 0.5f}}) {
+        const TensorGpu<f16> t = c.discount == 1.0f ? loader.load_matrix_f16(c.name) : loader.load_matrix_f16_discount(c.name, c.discount);
+        queue.sync();
+        const auto got = t.back();
+        const auto want = file_bytes(dir + "/" + c.name + c.tag);
+        EXPECT(want.size() == got.size() * 2);
+        int off = 0;
+        for (size_t i = 0; i < got.size() && want.size() == got.size() * 2; i++) {
+            f16 w;
+            std::memcpy(&w.bits, want.data() + 2 * i, 2);
+            const float g = f16_to_f32(got[i]), e = f16_to_f32(w);
+            off += std::fabs(g - e) > 1e-3f * std::max(1.0f, std::fabs(e)) * 0.5f + 6e-8f ? 1 : 0; // half a per mille: an f16 ulp is 4.9e-4 relative
+        }
+        EXPECT(off == 0);
+    }
+    // packed through the same path: an Int8 matrix of the blended weights loads without error
+    const Matrix mx = loader.load_matrix(std::string("blocks.6.ffn.value.weight"), Quant::Int8);
+    queue.sync();
+    EXPECT(mx.kind == Matrix::Kind::Int8);
+}
+
 // file -> discount -> pack on the device, against the packed bytes the CPU restatement gives for numpy's discount
 static void test_loader_gpu(const std::string &model_path, const std::string &dir) {
     check(wrq_init());
@@ -730,7 +783,11 @@ int main(int argc, char **argv) {
         try {
             test_f16_conversions();
             test_loader_host(argv[2], argv[3]);
-            if (std::string(argv[1]) == "--loader-gpu") test_loader_gpu(argv[2], argv[3]);
+            test_lora_host(argv[2], argv[3]);
+            if (std::string(argv[1]) == "--loader-gpu") {
+                test_loader_gpu(argv[2], argv[3]);
+                test_lora_gpu(argv[2], argv[3]);
+            }
         } catch (const std::exception &e) {
             std::printf("FAIL: %s\n", e.what());
             failures++;

@@ -39,6 +39,19 @@ def write_model(tmp_path, oracle):
         for tag, d in ((".half.f16", 0.5), (".x03.f16", 0.3)):
             # Loader::load_matrix_f16_discount: f16::from_f32(discount * x.to_f32()), src/runtime/loader.rs:660-661
             (np.float32(d) * tensors[name].astype(np.float32)).astype(np.float16).tofile(tmp_path / (name + tag))
+    # an adapter file (src/runtime/loader.rs:355-386): low-rank halves `<stem>.lora.0` [in, rank] and `.lora.1` [out, rank] for
+    # ffn.value, a whole tensor of the same name for att.output; blended with LoraBlend::full(0.5): out = alpha / rank * xa^T xb + w
+    rank, alpha = 8, np.float32(0.5)
+    xa = (rng.standard_normal((384, rank), dtype=np.float32) * np.float32(0.1)).astype(np.float16)  # [in, rank]
+    xb = (rng.standard_normal((256, rank), dtype=np.float32) * np.float32(0.1)).astype(np.float16)  # [out, rank]
+    ov = (rng.standard_normal((256, 256), dtype=np.float32) * np.float32(0.02)).astype(np.float16)
+    save_file({"blocks.6.ffn.value.lora.0": xa, "blocks.6.ffn.value.lora.1": xb, "blocks.6.att.output.weight": ov}, str(tmp_path / "lora.st"))
+    for tag, d in ((".lora.f16", np.float32(1.0)), (".lora_half.f16", np.float32(0.5))):
+        base = (d * ffn_v.astype(np.float32)).astype(np.float16).astype(np.float32)  # the discounted matrix is an f16 tensor before the blend
+        low = xb.astype(np.float32) @ xa.astype(np.float32).T  # [out, in]
+        (np.float32(d * alpha / rank) * low + base).astype(np.float16).tofile(tmp_path / ("blocks.6.ffn.value.weight" + tag))
+        base = (d * out_w.astype(np.float32)).astype(np.float16).astype(np.float32)
+        (np.float32(d * alpha) * ov.astype(np.float32) + base).astype(np.float16).tofile(tmp_path / ("blocks.6.att.output.weight" + tag))
     if oracle is not None:
         name = "blocks.6.ffn.value.weight"
         half = (np.float32(0.5) * ffn_v.astype(np.float32)).astype(np.float16)
