@@ -471,6 +471,79 @@ def schedule(wrq, torch, args, layers, C, H):
     print(json.dumps(out), flush=True)
 
 
+def stamps_timeline(wrq, torch, args, layers, C, H):
+    """Timeline of one Int8 decode step from wall-clock stamps written by stamped builds of the same kernels
+    (wrq_debug_stamps): per launch of a layer, when its first wave started and its last wave ended, the gap to
+    the launch before, and where a wave's lifetime goes.  Stamps cost time: the step is slower than the product's."""
+    import ctypes as C_
+    assert args.quant == "int8" and args.tokens == 1, "--stamps covers the Int8 one-token step"
+    L = wrq.lib()
+    L.wrq_debug_stamps.argtypes = [C_.c_void_p, C_.c_uint64]
+    dec = Decode(wrq, torch, layers, C, H, 1)
+    n_launch = 4 * len(layers)
+    slot = 1 << 20
+    buf = torch.zeros(n_launch * slot, dtype=torch.uint8, device="cuda")
+
+    def graph_of(fn):
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
+
+    plain = graph_of(dec.step_grouped)
+    plain_ms, _ = time_steps(torch, plain.replay, args.steps, args.warmup)
+    assert L.wrq_debug_stamps(C_.c_void_p(buf.data_ptr()), buf.numel()) == 0, L.wrq_last_error().decode()
+    dec.step_grouped()  # warm the stamped kernels (slots 0..n_launch-1)
+    torch.cuda.synchronize()
+    assert L.wrq_debug_stamps(C_.c_void_p(buf.data_ptr()), buf.numel()) == 0  # restart the slot counter
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        dec.step_grouped()
+    stamped_ms, _ = time_steps(torch, g.replay, args.steps, args.warmup)
+    torch.cuda.synchronize()
+    assert L.wrq_debug_stamps(None, 0) == 0
+    rec = buf.view(torch.int64).view(n_launch, slot // 32, 4).cpu().numpy()
+    kinds = [("{att.w_k, w_v, w_r, w_g}", 4 * C // 4, 4), ("att.w_o", C // 4, 4), ("{ffn.w_k, ffn.w_r}", (H + C) // 4, 4), ("ffn.w_v", C // 8, 14)]
+    tick_us = 0.01  # the wall-clock counter runs at 100 MHz
+    import numpy as np
+    rows = {k: [] for k in range(4)}
+    last_end = None
+    for i in range(n_launch):
+        name, wgs, waves = kinds[i % 4]
+        r = rec[i, :wgs * waves].astype(np.float64) * tick_us
+        assert (r[:, 0] > 0).all() and (r[:, 3] >= r[:, 0]).all(), "launch %d left stamp records unwritten" % i
+        first, end = r[:, 0].min(), r[:, 3].max()
+        if i >= 4:  # the first layer starts from an idle machine
+            life = r[:, 3] - r[:, 0]
+            rows[i % 4].append(dict(span=end - first, gap=first - last_end, last_start=r[:, 0].max() - first, issue=np.median(r[:, 1] - r[:, 0]),
+                                    data=np.median(r[:, 2] - r[:, 1]), finish=np.median(r[:, 3] - r[:, 2]), life=np.median(life),
+                                    life95=np.percentile(life, 95), first_done=r[:, 2].min() - first))
+        last_end = end
+    step_span = (rec[n_launch - 1, :kinds[3][1] * kinds[3][2], 3].max() - rec[0, :kinds[0][1] * kinds[0][2], 0].min()) * tick_us
+    print("Int8 decode step, %d layers, graph replay: %.4f ms with the product kernels, %.4f ms with the stamped builds; "
+          "first stamp to last stamp of the stamped step %.4f ms" % (len(layers), plain_ms, stamped_ms, step_span / 1e3))
+    print("per launch, microseconds, mean over layers 1..%d (medians over the waves of a launch where marked):" % (len(layers) - 1))
+    hdr = "%-26s %6s %6s %9s %9s %10s %9s %9s %9s %9s %9s %10s" % ("launch", "wgs", "waves", "gap", "span", "last_start", "issue~", "data~", "finish~", "life~", "life95", "first_done")
+    print(hdr)
+    out = {}
+    tot_gap = tot_span = 0.0
+    for k in range(4):
+        name, wgs, waves = kinds[k]
+        m = {f: float(np.mean([r[f] for r in rows[k]])) for f in rows[k][0]}
+        out[name] = {f: round(v, 3) for f, v in m.items()}
+        tot_gap += m["gap"]
+        tot_span += m["span"]
+        print("%-26s %6d %6d %9.2f %9.2f %10.2f %9.2f %9.2f %9.2f %9.2f %9.2f %10.2f" % (name, wgs, wgs * waves, m["gap"], m["span"], m["last_start"], m["issue"],
+              m["data"], m["finish"], m["life"], m["life95"], m["first_done"]))
+    print("layer: gaps %.2f us + spans %.2f us = %.2f us (stamped); the product step is %.2f us per layer" % (tot_gap, tot_span, tot_gap + tot_span, plain_ms * 1e3 / len(layers)))
+    print("gap: first wave start minus last wave end of the launch before; span: first wave start to last wave end; last_start: when the last wave of")
+    print("the launch started, after the first; issue~: entry to every load requested; data~: from there to every row accumulated; finish~: reduction")
+    print("and store; life~/life95: wave lifetime, median and 95th percentile; first_done: first wave anywhere with every row accumulated, after the first start.")
+    print(json.dumps({"stamps": out, "plain_ms": round(plain_ms, 4), "stamped_ms": round(stamped_ms, 4)}))
+
+
 def full_layers(wrq, torch, args, C, H):
     """Every op of the v6 layers, dispatched like the reference (src/runtime/v6.rs:758-955): 35 ops
     per layer, 8 of them the quantized products.  One run of `--tokens` tokens of one request per
@@ -721,7 +794,11 @@ def main():
                     help="the C++ loader: the f16 matrices of --layers 7B-shape layers from a safetensors file into Int8 matrices (file -> device -> pack)")
     ap.add_argument("--v5-model", action="store_true",
                     help="config 1: the RWKV-v5-shape model (12 layers, 768 channels, FFN 2688, vocabulary 65536), every op: a 32-token prompt run, then decode steps")
+    ap.add_argument("--stamps", action="store_true",
+                    help="timeline of the Int8 decode step from wall-clock stamps written by stamped builds of its kernels (sets WRQ_TEST_HOOKS=1)")
     args = ap.parse_args()
+    if args.stamps:
+        os.environ["WRQ_TEST_HOOKS"] = "1"
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus above 1 is not supported: the path would shard by weight rows, one all-gather of the outputs per product")
 
@@ -757,6 +834,9 @@ def main():
     layers = build_model(wrq, torch, args.quant, args.layers, C, H)
     if args.schedule:
         schedule(wrq, torch, args, layers, C, H)
+        return
+    if args.stamps:
+        stamps_timeline(wrq, torch, args, layers, C, H)
         return
     dec = Decode(wrq, torch, layers, C, H, args.tokens)
 

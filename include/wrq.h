@@ -40,6 +40,9 @@ extern "C" {
 #endif
 
 #define WRQ_ABI_VERSION 1
+/* Counts additions that leave every existing signature as it is (new entry points, new override keys);
+ * a binding built against minor m runs on any library of the same WRQ_ABI_VERSION with minor >= m. */
+#define WRQ_ABI_MINOR 3
 #define WRQ_INT8_BLOCK_SIZE 128u /* TensorOp::INT8_BLOCK_SIZE, src/tensor/ops.rs:292 */
 #define WRQ_NF4_BLOCK_SIZE 64u   /* TensorOp::NF4_BLOCK_SIZE, src/tensor/ops.rs:291 */
 
@@ -114,7 +117,20 @@ int wrq_init(void);
  */
 int wrq_debug_override(const char *key, int value);
 
+/*
+ * Measurement hook; no counterpart in the reference, and refused unless WRQ_TEST_HOOKS=1 was in the
+ * environment when the library first looked.  While a buffer is set, the one-token int8 products of the
+ * 7B shapes (the wave-owns-rows kernel at K = 4096, the K-split kernel at K = 14336) launch builds of
+ * the same kernels that also write four wall-clock readings (100 MHz counter) per wave: entry, every
+ * load requested, every row accumulated, result stored.  `buffer` is device memory of `bytes` bytes, a
+ * multiple of 1 MiB; launch i after the call writes slot i mod (bytes >> 20), record
+ * (workgroup * waves_per_workgroup + wave) of 4 x uint64 each.  NULL switches the hook off.  The
+ * product kernels carry no stamp code; `python3 bench.py --stamps` prints the timeline of a decode step.
+ */
+int wrq_debug_stamps(void *buffer, uint64_t bytes);
+
 int wrq_abi_version(void);
+int wrq_abi_minor(void); /* WRQ_ABI_MINOR of the loaded library */
 const char *wrq_status_string(int status);
 const char *wrq_last_error(void);
 

@@ -22,6 +22,7 @@ def test_library_exports_every_declared_symbol(wrq):
     for n in names:
         assert hasattr(L, n), n
     assert L.wrq_abi_version() == 1
+    assert L.wrq_abi_minor() >= 3  # entry points were added since minor 0; signatures never changed
     assert L.wrq_status_string(0) == b"ok"
     assert L.wrq_status_string(1) == b"tensor shape not match"
 

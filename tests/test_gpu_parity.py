@@ -304,6 +304,53 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
     assert_close(run(gpu, gpu_matrix(gpu, "int8", wpb, sb), xb, R, "vec", np.float32), truth, EPS, "batched")
 
 
+def test_stamped_builds_of_the_decode_kernels(gpu, oracle):
+    # wrq_debug_stamps swaps in builds of the one-token int8 kernels (K = 4096 rows kernel, single and grouped; K = 14336
+    # K-split kernel) that also write wall-clock records: results must be bit-identical to the product kernels', every
+    # wave of every launch must leave a record with ordered readings, and nothing is written once the hook is off
+    import ctypes as C
+    import torch
+
+    announce("int8 stamped decode kernels")
+    L = gpu.lib()
+    L.wrq_debug_stamps.argtypes = [C.c_void_p, C.c_uint64]
+    rng = np.random.default_rng(SEED + 79)
+    shapes = [(4096, 204), (4096, 64), (14336, 36)]
+    mats, xs = [], []
+    for K, R in shapes:
+        wp, scale, _ = pack(oracle, "int8", gen_f16(rng, (R, K), 0.02))
+        mats.append(gpu_matrix(gpu, "int8", wp, scale))
+        xs.append(gen_f16(rng, (1, K), 1.0))
+
+    def products():
+        outs = [run(gpu, m, x, R, "vec", np.float32) for m, x, (K, R) in zip(mats, xs, shapes)]
+        go = [torch.full((1, R), float("nan"), dtype=torch.float32, device="cuda") for K, R in shapes[:2]]
+        gpu.matmul_vec_group([(m, dev(x), o, gpu.ACT_NONE, False, {}) for m, x, o in zip(mats[:2], xs[:2], go)])
+        return outs + [host(o) for o in go]
+
+    want = products()
+    slot = 1 << 20
+    buf = torch.zeros(4 * slot, dtype=torch.uint8, device="cuda")
+    assert L.wrq_debug_stamps(C.c_void_p(buf.data_ptr()), slot + 5) != 0, "a size that is no multiple of 1 MiB must be refused"
+    assert L.wrq_debug_stamps(C.c_void_p(buf.data_ptr()), buf.numel()) == 0, L.wrq_last_error().decode()
+    try:
+        got = products()
+    finally:
+        assert L.wrq_debug_stamps(None, 0) == 0
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b), "stamped build changed a result"
+    rec = buf.view(torch.int64).view(4, slot // 32, 4).cpu().numpy()
+    waves = [(-(-204 // 4)) * 4, (64 // 4) * 4, -(-36 // 8) * 14, (-(-204 // 4) + 64 // 4) * 4]  # records per launch, in launch order
+    for i, n in enumerate(waves):
+        r = rec[i]
+        assert (r[:n, 0] > 0).all(), f"launch {i}: a wave left no record"
+        assert (np.diff(r[:n], axis=1) >= 0).all(), f"launch {i}: readings out of order"
+        assert (r[n:] == 0).all(), f"launch {i}: records beyond its waves"
+    buf.zero_()
+    products()
+    assert int(buf.count_nonzero()) == 0, "stamps written with the hook off"
+
+
 def test_int8_wave_rows_groups_of_mixed_k(gpu, oracle):
     # products of different K in one grouped call: the launch is cut where K changes, every product still gets its result
     import torch

@@ -23,8 +23,11 @@ def _case(gpu, oracle, torch, K, R, T, seed):
     want = torch.full((T, R), float("nan"), dtype=torch.float32, device="cuda")
     got = torch.full((T, R), float("nan"), dtype=torch.float32, device="cuda")
     gpu.TensorOp.matmul_mat_int8(wd, md, xd, want)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]  # hipMemGetInfo: what the device has left, whoever allocates
     gpu.TensorOp.matmul_mat_int8_noalloc(wd, md, xd, got)
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the no-alloc entry point changed the device's free memory"
     return got.cpu().numpy(), want.cpu().numpy(), truth_matmul(int8_dequant64(u8, mm), x)
 
 
@@ -34,7 +37,9 @@ def test_no_alloc_entry_matches_plain_entry_twice(gpu, oracle):
     # first call: 4096 x 4096 at 32 tokens -- 32 row tiles on 256 CUs, so K is split over workgroups and
     # the partial sums pass through the fixed array; second call: a smaller product right behind it,
     # which finds the first call's partial sums in the array and must not read them
-    for K, R, T in ((4096, 4096, 32), (1024, 512, 16)):
+    # third: 288 row tiles x 2 token tiles = 576 workgroups, a little above two per CU: the launch is cut in
+    # two and the tail's partial sums pass through the array as well
+    for K, R, T in ((4096, 4096, 32), (1024, 512, 16), (1024, 18432, 128)):
         print("case: no_alloc", K, R, T, flush=True)
         got, want, truth = _case(gpu, oracle, torch, K, R, T, SEED + K + R + T)
         assert np.isfinite(got).all()

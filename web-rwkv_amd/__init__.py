@@ -36,8 +36,9 @@ NF4_QUANT = [
 ]
 
 EXPORTS = [
-    "wrq_init", "wrq_abi_version", "wrq_status_string", "wrq_last_error",
+    "wrq_init", "wrq_abi_version", "wrq_abi_minor", "wrq_status_string", "wrq_last_error",
     "wrq_debug_override",
+    "wrq_debug_stamps",
     "wrq_quantize_mat_int8", "wrq_quantize_mat_nf4",
     "wrq_matmul_vec_int8", "wrq_matmul_vec_nf4", "wrq_matmul_mat_int8", "wrq_matmul_mat_nf4", "wrq_matmul_mat_int8_noalloc",
     "wrq_matmul_vec_int8_group", "wrq_matmul_vec_nf4_group",
@@ -179,6 +180,7 @@ def lib():
         L.wrq_status_string.argtypes = [i]
         L.wrq_last_error.restype = C.c_char_p
         L.wrq_debug_override.argtypes = [C.c_char_p, i]
+        L.wrq_debug_stamps.argtypes = [vp, C.c_uint64]
         L.wrq_quantize_mat_int8.argtypes = [vp, T, T, T]
         L.wrq_quantize_mat_nf4.argtypes = [vp, T, T, T, T]
         L.wrq_matmul_vec_int8.argtypes = [vp, T, T, V, V, i, i]
@@ -222,8 +224,9 @@ def lib():
         L.wrq_v6_decay.argtypes = [vp, u, u, u, vp, vp, vp, vp]
         L.wrq_v6_wkv_gate.argtypes = [vp, u, u, u, vp, vp, vp, V, vp, vp, vp, vp, vp, vp, C.c_float, vp]
         L.wrq_v6_post_ffn.argtypes = [vp, u, u, vp, V, vp, vp, vp, vp, vp, i]
-        for name in EXPORTS[4:]:
-            getattr(L, name).restype = i
+        for name in EXPORTS:
+            if name not in ("wrq_status_string", "wrq_last_error"):
+                getattr(L, name).restype = i
         _lib = L
     return _lib
 

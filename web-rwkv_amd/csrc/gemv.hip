@@ -480,9 +480,14 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
 // rows, i.e. whole 128-byte lines of an f16 output, and no output line is dirty in two L2s.
 // The scalar arguments come first so that they arrive preloaded in SGPRs (no dependent scalar load in front of the first
 // vector load); a single product needs no descriptor load at all.
-template <int BPL, int RW>
+// STAMP builds (separate kernels behind wrq_debug_stamps, never the ones a product call launches) record four wall-clock
+// readings per wave: entry, every load requested, every row accumulated, result stored.
+template <int BPL, int RW, bool STAMP = false>
 __device__ __forceinline__ void rows_task_int8(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
-                                               const int out_f16, const int act, const uint32_t task, uint4 *xs) {
+                                               const int out_f16, const int act, const uint32_t task, uint4 *xs,
+                                               unsigned long long *stamps = nullptr) {
+    unsigned long long t0 = 0, t1 = 0, t2 = 0;
+    if constexpr (STAMP) { t0 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
     constexpr int K = BPL * 1024;
     constexpr int XP = (K / 8 + 255) / 256; // 16-byte pieces of the activations per thread
     const uint32_t tid = threadIdx.x, lane = tid & 63, g = lane >> 3, sub = lane & 7;
@@ -526,6 +531,7 @@ __device__ __forceinline__ void rows_task_int8(const uint8_t *w, const uint32_t 
 #pragma unroll
         for (int r = 0; r < RW; r++) wv[r][j] = load128_stream(wrow[r] + j * 128);
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (STAMP) { t1 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll
     for (int i = 0; i < XP; i++) {
         const uint32_t idx = tid + i * 256;
@@ -561,6 +567,7 @@ __device__ __forceinline__ void rows_task_int8(const uint8_t *w, const uint32_t 
             acc[r] = fmaf(s, pr, fmaf(c0, sx, acc[r]));
         }
     }
+    if constexpr (STAMP) { __builtin_amdgcn_sched_barrier(0); t2 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
     float mine = 0.0f;
 #pragma unroll
     for (int r = 0; r < RW; r++) {
@@ -568,6 +575,14 @@ __device__ __forceinline__ void rows_task_int8(const uint8_t *w, const uint32_t 
         if (lane == (uint32_t)r) mine = s;
     }
     if (lane < (uint32_t)RW && row0 + lane < R) store_out(out, out_f16, row0 + lane, act_apply(act, mine));
+    if constexpr (STAMP) {
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned long long t3 = wall_clock64();
+        if (lane == 0) {
+            ulonglong4 *st = reinterpret_cast<ulonglong4 *>(stamps) + (blockIdx.x * 4 + wave);
+            *st = ulonglong4{t0, t1, t2, t3};
+        }
+    }
 }
 
 // Runs of `run` consecutive tasks per XCD (workgroup b starts on XCD b % 8); the tail that does not fill 8 runs keeps its numbers.
@@ -606,16 +621,49 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_
                             p.out_f16, p.act, task - p.task_begin, xs);
 }
 
+// The same two kernels with wall-clock stamps (one 32-byte record per wave at stamps[(workgroup * 4 + wave) * 4]).
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_single_stamped_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
+                                                                            const uint32_t R, const uint32_t total_tasks, const uint32_t flags,
+                                                                            unsigned long long *stamps) {
+    __shared__ uint4 xs[BPL * 128];
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    rows_task_int8<BPL, RW, true>(w, mm, x, out, R, (int)(flags & 1u), (int)(flags >> 1), task, xs, stamps);
+}
+
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_group_stamped_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3,
+                                                                           const uint32_t tb4, const uint32_t tb5, const uint32_t tb6,
+                                                                           const uint32_t tb7, const uint32_t total_tasks,
+                                                                           unsigned long long *stamps, const GemvGroup g) {
+    __shared__ uint4 xs[BPL * 128];
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    uint32_t pi = 0;
+    pi = task >= tb1 ? 1u : pi;
+    pi = task >= tb2 ? 2u : pi;
+    pi = task >= tb3 ? 3u : pi;
+    pi = task >= tb4 ? 4u : pi;
+    pi = task >= tb5 ? 5u : pi;
+    pi = task >= tb6 ? 6u : pi;
+    pi = task >= tb7 ? 7u : pi;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const GemvProblem p = g.p[pi];
+    rows_task_int8<BPL, RW, true>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out,
+                                  p.R, p.out_f16, p.act, task - p.task_begin, xs, stamps);
+}
+
 // int8, one token, f16 activations, long rows (K = WK * 1024, 8192 < K <= 16384): the WK waves of a workgroup split K, every wave
 // takes all RWG rows of the task over its 1024 elements -- one 16-byte chunk per lane and row, the lane's 16 activations in
 // registers for all rows (each activation crosses into the workgroup once, no LDS staging), one (min, max) word per chunk.
 // Request order: activations, scale words, weights; rows are consumed in arrival order; the partial sums of the waves meet in
 // LDS behind one barrier.  Same task numbering and argument passing as the wave-owns-rows kernel.
-template <int RWG, int WK>
-__global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
-                                                                  const uint32_t total_tasks, const uint32_t flags) {
+template <int RWG, int WK, bool STAMP = false>
+__device__ __forceinline__ void ksplit_task_int8(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
+                                                 const uint32_t total_tasks, const uint32_t flags, float (*red)[RWG],
+                                                 unsigned long long *stamps = nullptr) {
+    unsigned long long t0 = 0, t1 = 0, t2 = 0;
+    if constexpr (STAMP) { t0 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
     constexpr int K = WK * 1024;
-    __shared__ float red[WK][RWG];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t task = xcd_task(blockIdx.x, total_tasks, 64 / RWG);
@@ -637,6 +685,7 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
 #pragma unroll
     for (int r = 0; r < RWG; r++) wv[r] = load128_stream(wrow[r]);
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (STAMP) { t1 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
     const uint32_t xd[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
     float sx = 0.0f;
 #pragma unroll
@@ -661,6 +710,7 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
         const float sum = wave_sum(fmaf(s, pr, c0 * sx));
         if (lane == (uint32_t)r) mine = sum;
     }
+    if constexpr (STAMP) { __builtin_amdgcn_sched_barrier(0); t2 = wall_clock64(); __builtin_amdgcn_sched_barrier(0); }
     if (lane < (uint32_t)RWG) red[wave][lane] = mine;
     __syncthreads();
     if (tid < (uint32_t)RWG) {
@@ -669,6 +719,30 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
         for (int q = 0; q < WK; q++) s += red[q][tid];
         if (row0 + tid < R) store_out(out, (int)(flags & 1u), row0 + tid, act_apply((int)(flags >> 1), s));
     }
+    if constexpr (STAMP) {
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned long long t3 = wall_clock64();
+        if (lane == 0) {
+            ulonglong4 *st = reinterpret_cast<ulonglong4 *>(stamps) + (blockIdx.x * WK + wave);
+            *st = ulonglong4{t0, t1, t2, t3};
+        }
+    }
+}
+
+template <int RWG, int WK>
+__global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out, const uint32_t R,
+                                                                  const uint32_t total_tasks, const uint32_t flags) {
+    __shared__ float red[WK][RWG];
+    ksplit_task_int8<RWG, WK>(w, mm, x, out, R, total_tasks, flags, red);
+}
+
+// ... and with wall-clock stamps (one record per wave at stamps[(workgroup * WK + wave) * 4]).
+template <int RWG, int WK>
+__global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_stamped_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
+                                                                          const uint32_t R, const uint32_t total_tasks, const uint32_t flags,
+                                                                          unsigned long long *stamps) {
+    __shared__ float red[WK][RWG];
+    ksplit_task_int8<RWG, WK, true>(w, mm, x, out, R, total_tasks, flags, red, stamps);
 }
 
 // nf4, one token: the same one-shot shape (one workgroup per task of ROWS rows, NT lanes along
@@ -1046,9 +1120,49 @@ int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt
     return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
 
+// Timeline measurements (wrq_debug_stamps): while a stamp buffer is set, the launches of the 7B decode shapes (wave-owns-rows
+// at K = 4096, K-split at K = 14336) run their stamped builds, each into the next slot of the buffer.
+constexpr uint64_t kStampSlotBytes = 1u << 20; // 32768 records of 32 bytes: enough for 8192 workgroups of 4 waves
+unsigned long long *g_stamp_buf = nullptr;
+uint64_t g_stamp_slots = 0, g_stamp_next = 0;
+
+unsigned long long *next_stamp_slot(uint32_t records) {
+    if (!g_stamp_buf || records * 32ull > kStampSlotBytes) return nullptr;
+    const uint64_t slot = g_stamp_next++ % g_stamp_slots;
+    return g_stamp_buf + slot * (kStampSlotBytes / 8);
+}
+
+} // namespace
+
+int stamps_set(void *buf, uint64_t bytes) {
+    if (buf && (bytes < kStampSlotBytes || bytes % kStampSlotBytes != 0))
+        return fail(WRQ_ERR_SIZE, "stamp buffer of %llu bytes is not a multiple of %llu", (unsigned long long)bytes,
+                    (unsigned long long)kStampSlotBytes);
+    g_stamp_buf = static_cast<unsigned long long *>(buf);
+    g_stamp_slots = buf ? bytes / kStampSlotBytes : 0;
+    g_stamp_next = 0;
+    return WRQ_OK;
+}
+
+namespace {
+
 template <int BPL, int RW>
 int launch_rows_int8(hipStream_t stream, const GemvGroup &g) {
     const dim3 grid(g.total_tasks);
+    if constexpr (BPL == 4) {
+        if (unsigned long long *st = next_stamp_slot(g.total_tasks * 4)) {
+            if (g.n == 1) {
+                const GemvProblem &p = g.p[0];
+                hipLaunchKernelGGL((gemv_int8_rows_single_stamped_kernel<BPL, RW>), grid, dim3(256), 0, stream, p.w,
+                                   reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out,
+                                   p.R, g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), st);
+            } else {
+                hipLaunchKernelGGL((gemv_int8_rows_group_stamped_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2],
+                                   g.task_begin[3], g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, st, g);
+            }
+            return check_launch("matmul_vec_int8");
+        }
+    }
     if (g.n == 1) {
         const GemvProblem &p = g.p[0];
         hipLaunchKernelGGL((gemv_int8_rows_single_kernel<BPL, RW>), grid, dim3(256), 0, stream, p.w,
@@ -1086,6 +1200,14 @@ bool ksplit_kernel_has(uint32_t K) { return K % 1024 == 0 && (K == 10240 || K ==
 template <int WK>
 int launch_ksplit_int8(hipStream_t stream, const GemvGroup &g) {
     const GemvProblem &p = g.p[0];
+    if constexpr (WK == 14) {
+        if (unsigned long long *st = next_stamp_slot(g.total_tasks * WK)) {
+            hipLaunchKernelGGL((gemv_int8_ksplit_stamped_kernel<8, WK>), dim3(g.total_tasks), dim3(WK * 64), 0, stream, p.w,
+                               reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R,
+                               g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), st);
+            return check_launch("matmul_vec_int8");
+        }
+    }
     hipLaunchKernelGGL((gemv_int8_ksplit_kernel<8, WK>), dim3(g.total_tasks), dim3(WK * 64), 0, stream, p.w,
                        reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R, g.total_tasks,
                        (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1));

@@ -303,6 +303,7 @@ using namespace wrq;
 extern "C" {
 
 int wrq_abi_version(void) { return WRQ_ABI_VERSION; }
+int wrq_abi_minor(void) { return WRQ_ABI_MINOR; }
 
 const char *wrq_last_error(void) { return g_error; }
 
@@ -323,6 +324,13 @@ const char *wrq_status_string(int status) {
 int wrq_debug_override(const char *key, int value) {
     if (!key) return fail(WRQ_ERR_NULL, "null pointer: key");
     return tune_set(key, value);
+}
+
+int wrq_debug_stamps(void *buffer, uint64_t bytes) {
+    (void)tune(kTuneGemvOneshot, 0); // makes sure the environment has been read
+    if (!g_test_hooks.load(std::memory_order_relaxed))
+        return fail(WRQ_ERR_UNSUPPORTED, "wrq_debug_stamps needs WRQ_TEST_HOOKS=1 in the environment");
+    return stamps_set(buffer, bytes);
 }
 
 int wrq_init(void) {

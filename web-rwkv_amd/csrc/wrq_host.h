@@ -71,6 +71,10 @@ bool tune_is_set(TuneKey key);
 // Sets (value >= 0) or clears (value < 0) the override called `name`; unknown names fail.
 int tune_set(const char *name, int value);
 
+// Timeline measurement hook of the one-token int8 kernels (gemv.hip): `buf` (device memory, `bytes` long, a multiple of 1 MiB)
+// takes the wall-clock records of the following launches, one 1 MiB slot per launch, round-robin; nullptr switches it off.
+int stamps_set(void *buf, uint64_t bytes);
+
 // Resolves the split-K scratch array of the current device (also done lazily by the first
 // chunk product; calling it from wrq_init keeps the lookup out of stream capture).
 int prepare_gemm_scratch();
