@@ -37,9 +37,7 @@ def test_no_alloc_entry_matches_plain_entry_twice(gpu, oracle):
     # first call: 4096 x 4096 at 32 tokens -- 32 row tiles on 256 CUs, so K is split over workgroups and
     # the partial sums pass through the fixed array; second call: a smaller product right behind it,
     # which finds the first call's partial sums in the array and must not read them
-    # third: 288 row tiles x 2 token tiles = 576 workgroups, a little above two per CU: the launch is cut in
-    # two and the tail's partial sums pass through the array as well
-    for K, R, T in ((4096, 4096, 32), (1024, 512, 16), (1024, 18432, 128)):
+    for K, R, T in ((4096, 4096, 32), (1024, 512, 16)):
         print("case: no_alloc", K, R, T, flush=True)
         got, want, truth = _case(gpu, oracle, torch, K, R, T, SEED + K + R + T)
         assert np.isfinite(got).all()
