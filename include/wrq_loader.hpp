@@ -10,7 +10,7 @@
 // The discount (2^-(layer / rescale) on att.output and ffn.value) multiplies in f32 and rounds to
 // f16 (nearest even, subnormals kept: `half::f16::from_f32`) before the matrix is packed; the loader does
 // it on the device, `Loader::discounted` is the same expression on the host.
-//   Lora, LoraBlend, lora_matrices, lora_vectors      src/runtime/loader.rs:76-167, :328-386 (adapters blended in at load time:
+//   Lora, LoraBlend, lora_matrices, lora_vectors      src/runtime/loader.rs:106-186, :328-386 (adapters blended in at load time:
 //                                                     `blend_lora` with alpha / rank for the low-rank halves, `blend` for whole tensors)
 //
 // The file format (safetensors): 8 bytes little-endian header length N, N bytes of JSON
@@ -293,7 +293,7 @@ class SafeTensors {
 
 enum class Quant { None, Int8, NF4, SF4 }; // src/runtime/model.rs:122-135
 
-// Low-rank adapters blended into the weights while they are loaded (src/runtime/loader.rs:76-167).
+// Low-rank adapters blended into the weights while they are loaded (src/runtime/loader.rs:106-186).
 // A blend pattern is a regular expression over tensor names and a factor; of the patterns of one adapter that match a name,
 // the LAST one counts (`rfind`, loader.rs:336-343).
 struct LoraBlendPattern {
