@@ -304,6 +304,53 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
     assert_close(run(gpu, gpu_matrix(gpu, "int8", wpb, sb), xb, R, "vec", np.float32), truth, EPS, "batched")
 
 
+@pytest.mark.parametrize("K", WAVE_ROWS_K)
+def test_int8_wave_rows_kernels_on_short_runs(gpu, oracle, K, overrides):
+    # runs of 2 tokens of f16 activations on int8 rows of a multiple of 1024 take the wave-owns-rows layout (up to 8192, both
+    # tokens' activations in LDS) or the K-split layout (10240 .. 16384); runs of 3 and 4 stay on the one-shot kernel.
+    # Single products and groups, ragged last tasks, both output types, an activation, token strides through views --
+    # against the oracle and float64, and the kernel they replace (gemv_rows_tokens = 0) on the same inputs
+    import torch
+
+    announce("int8 wave-owns-rows, short runs", K)
+    rng = np.random.default_rng(SEED + 177 + K)
+    rows = [204, 64, 8, 4, 132]
+    packed, mats = [], []
+    for R in rows:
+        wp, scale, wdeq = pack(oracle, "int8", gen_f16(rng, (R, K), 0.02))
+        packed.append((wp, scale, wdeq))
+        mats.append(gpu_matrix(gpu, "int8", wp, scale))
+    for T in (2, 3, 4):
+        xs = [gen_f16(rng, (T, K), 1.0) for _ in rows]
+        truths = [truth_matmul(wdeq, x) for (_, _, wdeq), x in zip(packed, xs)]
+        wants = [oracle.matmul_vec_int8(wp, scale, x, out_dtype=np.float32)[0] for (wp, scale, _), x in zip(packed, xs)]
+        for tokens_kernel in (1, 0):
+            overrides(gemv_rows_tokens=tokens_kernel)
+            for m, x, R, truth, want in zip(mats, xs, rows, truths, wants):
+                for out_dtype in (np.float16, np.float32):
+                    got = run(gpu, m, x, R, "vec", out_dtype)
+                    assert_close(got, want, EPS, f"K={K} R={R} T={T} tokens_kernel={tokens_kernel} vs oracle")
+                    assert_close(got, truth, EPS, f"K={K} R={R} T={T} tokens_kernel={tokens_kernel} vs float64")
+                got = run(gpu, m, x, R, "vec", np.float32, act=1)
+                assert_close(got, np.square(np.maximum(truth, 0.0)), EPS, f"K={K} R={R} T={T} squared relu")
+            outs = [torch.full((T, R), float("nan"), dtype=torch.float16 if i % 2 else torch.float32, device="cuda") for i, R in enumerate(rows)]
+            gpu.matmul_vec_group([(m, dev(x), o, gpu.ACT_SQUARED_RELU if i == 2 else gpu.ACT_NONE, False, {})
+                                  for i, (m, x, o) in enumerate(zip(mats, xs, outs))])
+            for i, (o, truth) in enumerate(zip(outs, truths)):
+                assert_close(host(o).astype(np.float32), np.square(np.maximum(truth, 0.0)) if i == 2 else truth, EPS, f"K={K} T={T} group member {i}")
+        overrides(gemv_rows_tokens=1)
+        # token strides that differ from the row lengths: the i-th of 5 interleaved activation sets (v6: att_sx.view(.., .., i, ..),
+        # src/runtime/v6.rs:806-829) into a slice of a wider output
+        parent = gen_f16(rng, (5, T, K), 1.0)
+        out = torch.full((3, T + 2, rows[0]), -7.0, dtype=torch.float32, device="cuda")
+        mats[0].matmul_vec_op(dev(parent), out, input_view=((K, T, 1), (K, T, 5), (0, 0, 3)),
+                              output_view=((rows[0], T, 1), (rows[0], T + 2, 3), (0, 1, 2)))
+        got = host(out)
+        assert_close(got[2, 1:1 + T], oracle.matmul_vec_int8(packed[0][0], packed[0][1], parent[3], out_dtype=np.float32)[0], EPS, f"T={T} offset views")
+        got[2, 1:1 + T] = -7.0
+        assert (got == -7.0).all(), "wrote outside the output view"
+
+
 def test_stamped_builds_of_the_decode_kernels(gpu, oracle):
     # wrq_debug_stamps swaps in builds of the one-token int8 kernels (K = 4096 rows kernel, single and grouped; K = 14336
     # K-split kernel) that also write wall-clock records: results must be bit-identical to the product kernels', every

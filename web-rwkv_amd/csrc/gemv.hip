@@ -621,6 +621,138 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_
                             p.out_f16, p.act, task - p.task_begin, xs);
 }
 
+// Runs of TT tokens on the same layout (tokens past the run repeat the last one and are not stored; built for TT = 2):
+// the activations of all tokens reach LDS once per workgroup, a wave converts the codes of a chunk once and meets every
+// token's 32 bytes with them, two rows per wave share each activation read.  Per 16 weight bytes that is 8 permutes,
+// 10 TT dot products and fmas and 8 TT / RW dot products for the activation sums.
+template <int BPL, int RW, int TT>
+__device__ __forceinline__ void rows_tokens_task_int8(const uint8_t *w, const uint32_t *mm, const uint16_t *x, const uint64_t x_token_stride,
+                                                      void *out, const uint64_t out_token_stride, const uint32_t R, const uint32_t T,
+                                                      const int out_f16, const int act, const uint32_t task, uint4 *xs) {
+    constexpr int K = BPL * 1024;
+    constexpr int PIECES = TT * (K / 8);       // 16-byte pieces of the activations, all tokens
+    constexpr int XP = (PIECES + 255) / 256;   // ... per thread
+    const uint32_t tid = threadIdx.x, lane = tid & 63, g = lane >> 3, sub = lane & 7;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t row0 = task * (4 * RW) + wave * RW;
+    uint4 xp[XP];
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const uint32_t idx = tid + i * 256;
+        if (XP * 256 == PIECES || idx < (uint32_t)PIECES) {
+            const uint32_t tok = min(idx / (K / 8), T - 1); // tokens past the run repeat the last one
+            xp[i] = load128(reinterpret_cast<const uint4 *>(x + (uint64_t)tok * x_token_stride) + idx % (K / 8));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t sc[RW][BPL];
+    const uint8_t *wrow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        const uint32_t row = min(row0 + r, R - 1); // rows past the end repeat the last one and are not stored
+        wrow[r] = w + (uint64_t)row * K + (g * BPL) * 128 + sub * 16;
+        const uint32_t *sp = mm + (uint64_t)row * (K / 128) + g * BPL;
+        if constexpr (BPL % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < BPL / 4; q++) {
+                const uint4 v = load128(sp + 4 * q);
+                sc[r][4 * q] = v.x, sc[r][4 * q + 1] = v.y, sc[r][4 * q + 2] = v.z, sc[r][4 * q + 3] = v.w;
+            }
+        } else if constexpr (BPL % 2 == 0) {
+#pragma unroll
+            for (int q = 0; q < BPL / 2; q++) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(sp + 2 * q);
+                sc[r][2 * q] = v.x, sc[r][2 * q + 1] = v.y;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < BPL; j++) sc[r][j] = sp[j];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint4 wv[RW][BPL];
+#pragma unroll
+    for (int j = 0; j < BPL; j++)
+#pragma unroll
+        for (int r = 0; r < RW; r++) wv[r][j] = load128_stream(wrow[r] + j * 128);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < XP; i++) {
+        const uint32_t idx = tid + i * 256;
+        if (XP * 256 == PIECES || idx < (uint32_t)PIECES) xs[idx] = xp[i];
+    }
+    lds_barrier();
+    float acc[RW][TT];
+#pragma unroll
+    for (int r = 0; r < RW; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[r][t] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < BPL; j++) {
+        uint32_t code[RW][8]; // f16 pairs (1024 + u0, 1024 + u1)
+        float s[RW], c0[RW];
+#pragma unroll
+        for (int r = 0; r < RW; r++) {
+            const uint32_t wd[4] = {wv[r][j].x, wv[r][j].y, wv[r][j].z, wv[r][j].w};
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                code[r][2 * d] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04010400u);
+                code[r][2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04030402u);
+            }
+            const float mn = h2f((uint16_t)(sc[r][j] & 0xffffu));
+            const float mx = h2f((uint16_t)(sc[r][j] >> 16));
+            s[r] = (mx - mn) * (1.0f / 255.0f);
+            c0[r] = fmaf(-1024.0f, s[r], mn);
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const uint4 *xt = xs + t * (K / 8);
+            const uint4 x0 = xt[((g * BPL + j) * 8 + sub) * 2], x1 = xt[((g * BPL + j) * 8 + sub) * 2 + 1];
+            const uint32_t xd[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            float sx = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 8; q++) sx = dot2(xd[q], 0x3c003c00u, sx); // (1.0, 1.0)
+#pragma unroll
+            for (int r = 0; r < RW; r++) {
+                float pr = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 8; q++) pr = dot2(code[r][q], xd[q], pr);
+                acc[r][t] = fmaf(s[r], pr, fmaf(c0[r], sx, acc[r][t]));
+            }
+        }
+    }
+    float mine = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RW; r++)
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float v = wave_sum(acc[r][t]);
+            if (lane == (uint32_t)(r * TT + t)) mine = v;
+        }
+    const uint32_t r = lane / TT, t = lane % TT;
+    if (lane < (uint32_t)(RW * TT) && row0 + r < R && t < T) store_out(out, out_f16, (uint64_t)t * out_token_stride + row0 + r, act_apply(act, mine));
+}
+
+template <int BPL, int RW, int TT>
+__global__ __launch_bounds__(256) void gemv_int8_rows_tokens_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t tb4,
+                                                                    const uint32_t tb5, const uint32_t tb6, const uint32_t tb7,
+                                                                    const uint32_t total_tasks, const uint32_t T, const GemvGroup g) {
+    __shared__ uint4 xs[TT * BPL * 128];
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    uint32_t pi = 0;
+    pi = task >= tb1 ? 1u : pi;
+    pi = task >= tb2 ? 2u : pi;
+    pi = task >= tb3 ? 3u : pi;
+    pi = task >= tb4 ? 4u : pi;
+    pi = task >= tb5 ? 5u : pi;
+    pi = task >= tb6 ? 6u : pi;
+    pi = task >= tb7 ? 7u : pi;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
+    rows_tokens_task_int8<BPL, RW, TT>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
+                                       p.x_token_stride, p.out, p.out_token_stride, p.R, T, p.out_f16, p.act, task - p.task_begin, xs);
+}
+
 // The same two kernels with wall-clock stamps (one 32-byte record per wave at stamps[(workgroup * 4 + wave) * 4]).
 template <int BPL, int RW>
 __global__ __launch_bounds__(256) void gemv_int8_rows_single_stamped_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
@@ -734,6 +866,87 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
                                                                   const uint32_t total_tasks, const uint32_t flags) {
     __shared__ float red[WK][RWG];
     ksplit_task_int8<RWG, WK>(w, mm, x, out, R, total_tasks, flags, red);
+}
+
+// Runs of TT tokens on the K-split layout (built for TT = 2): a lane keeps its 16 activations of every token in registers, converts a
+// row's codes once and meets every token with them; the RWG x TT partial sums of a wave close inside DPP rows and meet in LDS.
+template <int RWG, int WK, int TT>
+__global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_tokens_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
+                                                                         const uint32_t R, const uint32_t total_tasks, const uint32_t flags,
+                                                                         const uint32_t T, const uint32_t x_token_stride,
+                                                                         const uint32_t out_token_stride) {
+    constexpr int K = WK * 1024;
+    __shared__ float red[RWG * TT][WK * 4]; // per output: one partial sum per DPP row of 16 lanes
+    static_assert(RWG * TT * 16 <= WK * 64, "16 lanes per output close the sums");
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 64 / RWG);
+    const uint32_t row0 = task * RWG;
+    const uint32_t k0 = wave * 1024 + lane * 16; // first element of this lane's chunk
+    uint4 xv[TT][2];
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+        const uint32_t tok = min((uint32_t)t, T - 1); // tokens past the run repeat the last one
+        const uint4 *xp = reinterpret_cast<const uint4 *>(x + (uint64_t)tok * x_token_stride + k0);
+        xv[t][0] = load128(xp), xv[t][1] = load128(xp + 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t sc[RWG];
+    const uint8_t *wrow[RWG];
+#pragma unroll
+    for (int r = 0; r < RWG; r++) {
+        const uint32_t row = min(row0 + r, R - 1); // rows past the end repeat the last one and are not stored
+        wrow[r] = w + (uint64_t)row * K + k0;
+        sc[r] = mm[(uint64_t)row * (K / 128) + (k0 >> 7)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint4 wv[RWG];
+#pragma unroll
+    for (int r = 0; r < RWG; r++) wv[r] = load128_stream(wrow[r]);
+    __builtin_amdgcn_sched_barrier(0);
+    float sx[TT];
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+        const uint32_t xd[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
+        sx[t] = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 8; q++) sx[t] = dot2(xd[q], 0x3c003c00u, sx[t]); // (1.0, 1.0)
+    }
+#pragma unroll
+    for (int r = 0; r < RWG; r++) {
+        const uint32_t wd[4] = {wv[r].x, wv[r].y, wv[r].z, wv[r].w};
+        uint32_t code[8]; // f16 pairs (1024 + u0, 1024 + u1)
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            code[2 * d] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04010400u);
+            code[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, wd[d], 0x04030402u);
+        }
+        const float mn = h2f((uint16_t)(sc[r] & 0xffffu));
+        const float mx = h2f((uint16_t)(sc[r] >> 16));
+        const float s = (mx - mn) * (1.0f / 255.0f);
+        const float c0 = fmaf(-1024.0f, s, mn);
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const uint32_t xd[8] = {xv[t][0].x, xv[t][0].y, xv[t][0].z, xv[t][0].w, xv[t][1].x, xv[t][1].y, xv[t][1].z, xv[t][1].w};
+            float pr = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 8; q++) pr = dot2(code[q], xd[q], pr);
+            const float v = row_sum(fmaf(s, pr, c0 * sx[t])); // over the 16 lanes of a DPP row
+            if ((lane & 15) == 0) red[r * TT + t][wave * 4 + (lane >> 4)] = v;
+        }
+    }
+    __syncthreads();
+    if (tid < (uint32_t)(RWG * TT * 16)) { // whole waves: RWG * TT is a multiple of 4
+        const uint32_t o = tid >> 4, l = tid & 15;
+        float v = 0.0f;
+#pragma unroll
+        for (int q = 0; q < (WK * 4 + 15) / 16; q++)
+            if (l + 16 * q < (uint32_t)(WK * 4)) v += red[o][l + 16 * q];
+        v = row_sum(v);
+        const uint32_t r = o / TT, t = o % TT;
+        if (l == 0 && row0 + r < R && t < T)
+            store_out(out, (int)(flags & 1u), (uint64_t)t * out_token_stride + row0 + r, act_apply((int)(flags >> 1), v));
+    }
 }
 
 // ... and with wall-clock stamps (one record per wave at stamps[(workgroup * WK + wave) * 4]).
@@ -1224,6 +1437,44 @@ int launch_ksplit_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     }
 }
 
+template <int BPL, int TT>
+int launch_rows_tokens_int8(hipStream_t stream, const GemvGroup &g) {
+    hipLaunchKernelGGL((gemv_int8_rows_tokens_kernel<BPL, 2, TT>), dim3(g.total_tasks), dim3(256), 0, stream, g.task_begin[1], g.task_begin[2],
+                       g.task_begin[3], g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, g.T, g);
+    return check_launch("matmul_vec_int8");
+}
+
+// Runs of two tokens.  (Four tokens per pass were built on the same layout and measured at 1.93 against 1.96 ms per 7B step for
+// the one-shot kernel at 4 tokens, 1.92 against 1.94 at 3: there the vector ALU is as busy as the memory system whichever
+// way the lanes are laid out, and the launches are single rounds of workgroups that load, then compute, in step.  Not kept.)
+int launch_rows_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
+    switch (K / 1024) {
+#define WRQ_ROWS_CASE(B) case B: return launch_rows_tokens_int8<B, 2>(stream, g);
+    WRQ_ROWS_CASE(1) WRQ_ROWS_CASE(2) WRQ_ROWS_CASE(3) WRQ_ROWS_CASE(4) WRQ_ROWS_CASE(5) WRQ_ROWS_CASE(6) WRQ_ROWS_CASE(7) WRQ_ROWS_CASE(8)
+#undef WRQ_ROWS_CASE
+    default: return fail(WRQ_ERR_UNSUPPORTED, "no wave-owns-rows kernel for K = %u at %u tokens", K, g.T);
+    }
+}
+
+template <int WK, int TT>
+int launch_ksplit_tokens_int8(hipStream_t stream, const GemvGroup &g) {
+    const GemvProblem &p = g.p[0];
+    hipLaunchKernelGGL((gemv_int8_ksplit_tokens_kernel<8, WK, TT>), dim3(g.total_tasks), dim3(WK * 64), 0, stream, p.w,
+                       reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R,
+                       g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), g.T, (uint32_t)p.x_token_stride,
+                       (uint32_t)p.out_token_stride);
+    return check_launch("matmul_vec_int8");
+}
+
+int launch_ksplit_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
+    switch (K / 1024) {
+#define WRQ_KSPLIT_CASE(B) case B: return launch_ksplit_tokens_int8<B, 2>(stream, g);
+    WRQ_KSPLIT_CASE(10) WRQ_KSPLIT_CASE(12) WRQ_KSPLIT_CASE(14) WRQ_KSPLIT_CASE(16)
+#undef WRQ_KSPLIT_CASE
+    default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u at %u tokens", K, g.T);
+    }
+}
+
 int launch_rows_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
 #define WRQ_ROWS_CASE(B) case B: return launch_rows_int8<B, rows_per_wave(B)>(stream, g);
@@ -1291,10 +1542,13 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
-        const bool waverows = oneshot && quant == kInt8 && in_f16 && T == 1 && rows_kernel_has(args[i].K) &&
+        // (runs of 2 tokens take the same layouts with both tokens in one pass)
+        const bool tokens_ok = T == 1 || (T == 2 && tune(kTuneGemvRowsTokens, 1) && args[i].x_token_stride <= 0xffffffffull &&
+                                          args[i].out_token_stride <= 0xffffffffull);
+        const bool waverows = oneshot && quant == kInt8 && in_f16 && tokens_ok && rows_kernel_has(args[i].K) && (T == 1 || args[i].K <= 8192) &&
                               ((uintptr_t)args[i].scale % 16 == 0) && tune(kTuneGemvWaveRows, 1);
         // ... and long rows (8192 < K <= 16384, a multiple of 2048): the K-split kernel, one product per launch
-        const bool ksplit = oneshot && !waverows && quant == kInt8 && in_f16 && T == 1 && ksplit_kernel_has(args[i].K) && args[i].B == 1 &&
+        const bool ksplit = oneshot && !waverows && quant == kInt8 && in_f16 && tokens_ok && ksplit_kernel_has(args[i].K) && args[i].B == 1 &&
                             tune(kTuneGemvWaveRows, 1);
         // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
         if (oneshot && quant == kInt8 && args[i].K / 16 > 512) rows = 8;
@@ -1311,7 +1565,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (oneshot && quant == kInt8 && ott == 2 && !tune_is_set(kTuneGemvRows)) rows = 4;
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
-        if (waverows) rows = 4 * rows_per_wave((int)(args[i].K / 1024));
+        if (waverows) rows = T == 1 ? 4 * rows_per_wave((int)(args[i].K / 1024)) : 8; // several tokens: two rows per wave
         if (ksplit) rows = 8;
         while (i < n && g.n < (uint32_t)kMaxGroup) {
             const MatmulArgs &a = args[i];
@@ -1392,11 +1646,16 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             continue;
         }
         if (ksplit && g.n == 1 && ksplit_kernel_has(g.p[0].K) && rows == 8) {
-            const int s1 = launch_ksplit_int8_k(stream, g, g.p[0].K);
+            const int s1 = T == 1 ? launch_ksplit_int8_k(stream, g, g.p[0].K) : launch_ksplit_tokens_int8_k(stream, g, g.p[0].K);
             if (s1 != WRQ_OK) return s1;
             continue;
         }
-        if (waverows && rows_kernel_has(g.p[0].K) && rows == 4 * rows_per_wave((int)(g.p[0].K / 1024))) {
+        if (waverows && rows_kernel_has(g.p[0].K) && T > 1 && rows == 8) {
+            const int s1 = launch_rows_tokens_int8_k(stream, g, g.p[0].K);
+            if (s1 != WRQ_OK) return s1;
+            continue;
+        }
+        if (waverows && rows_kernel_has(g.p[0].K) && T == 1 && rows == 4 * rows_per_wave((int)(g.p[0].K / 1024))) {
             const int s1 = launch_rows_int8_k(stream, g, g.p[0].K);
             if (s1 != WRQ_OK) return s1;
             continue;
