@@ -349,6 +349,13 @@ def test_int8_wave_rows_kernels_on_short_runs(gpu, oracle, K, overrides):
         assert_close(got[2, 1:1 + T], oracle.matmul_vec_int8(packed[0][0], packed[0][1], parent[3], out_dtype=np.float32)[0], EPS, f"T={T} offset views")
         got[2, 1:1 + T] = -7.0
         assert (got == -7.0).all(), "wrote outside the output view"
+        # batch axis: matrix [K, R, B], activations [K, T, B]
+        B, R = 3, 36
+        wb = gen_f16(rng, (B, R, K), 0.02)
+        xb = gen_f16(rng, (B, T, K), 1.0)
+        wpb, sb, wdq = pack(oracle, "int8", wb)
+        truth = np.stack([truth_matmul(wdq[b], xb[b]) for b in range(B)])
+        assert_close(run(gpu, gpu_matrix(gpu, "int8", wpb, sb), xb, R, "vec", np.float32), truth, EPS, f"T={T} batched")
 
 
 def test_stamped_builds_of_the_decode_kernels(gpu, oracle):
