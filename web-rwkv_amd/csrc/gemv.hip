@@ -621,14 +621,14 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_
                             p.out_f16, p.act, task - p.task_begin, xs);
 }
 
-// Runs of TT tokens on the same layout (tokens past the run repeat the last one and are not stored; built for TT = 2):
+// Runs of TT tokens on the same layout (tokens past the run repeat the last one and are not stored; built for TT = 2 and 4):
 // the activations of all tokens reach LDS once per workgroup, a wave converts the codes of a chunk once and meets every
-// token's 32 bytes with them, two rows per wave share each activation read.  Per 16 weight bytes that is 8 permutes,
-// 10 TT dot products and fmas and 8 TT / RW dot products for the activation sums.
+// token's 32 bytes with them, two rows per wave share each activation read.  Per 16 weight bytes that is 8 permutes
+// and 10 TT dot products and fmas; the sums of a chunk's activations are taken once per workgroup while they are staged.
 template <int BPL, int RW, int TT>
 __device__ __forceinline__ void rows_tokens_task_int8(const uint8_t *w, const uint32_t *mm, const uint16_t *x, const uint64_t x_token_stride,
                                                       void *out, const uint64_t out_token_stride, const uint32_t R, const uint32_t T,
-                                                      const int out_f16, const int act, const uint32_t task, uint4 *xs) {
+                                                      const int out_f16, const int act, const uint32_t task, uint4 *xs, float *sxs) {
     constexpr int K = BPL * 1024;
     constexpr int PIECES = TT * (K / 8);       // 16-byte pieces of the activations, all tokens
     constexpr int XP = (PIECES + 255) / 256;   // ... per thread
@@ -676,10 +676,20 @@ __device__ __forceinline__ void rows_tokens_task_int8(const uint8_t *w, const ui
 #pragma unroll
         for (int r = 0; r < RW; r++) wv[r][j] = load128_stream(wrow[r] + j * 128);
     __builtin_amdgcn_sched_barrier(0);
+    // the sum of a chunk's 16 activations (the offset term of the dequantisation) is taken once per workgroup: a piece is
+    // half a chunk, its other half sits in the neighbouring lane
 #pragma unroll
     for (int i = 0; i < XP; i++) {
         const uint32_t idx = tid + i * 256;
-        if (XP * 256 == PIECES || idx < (uint32_t)PIECES) xs[idx] = xp[i];
+        if (XP * 256 == PIECES || idx < (uint32_t)PIECES) {
+            xs[idx] = xp[i];
+            float h = dot2(xp[i].x, 0x3c003c00u, 0.0f); // (1.0, 1.0)
+            h = dot2(xp[i].y, 0x3c003c00u, h);
+            h = dot2(xp[i].z, 0x3c003c00u, h);
+            h = dot2(xp[i].w, 0x3c003c00u, h);
+            h += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(h), 0xB1, 0xf, 0xf, true)); // quad_perm [1,0,3,2]
+            if ((tid & 1u) == 0) sxs[idx >> 1] = h;
+        }
     }
     lds_barrier();
     float acc[RW][TT];
@@ -709,9 +719,7 @@ __device__ __forceinline__ void rows_tokens_task_int8(const uint8_t *w, const ui
             const uint4 *xt = xs + t * (K / 8);
             const uint4 x0 = xt[((g * BPL + j) * 8 + sub) * 2], x1 = xt[((g * BPL + j) * 8 + sub) * 2 + 1];
             const uint32_t xd[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-            float sx = 0.0f;
-#pragma unroll
-            for (int q = 0; q < 8; q++) sx = dot2(xd[q], 0x3c003c00u, sx); // (1.0, 1.0)
+            const float sx = sxs[t * (K / 16) + (g * BPL + j) * 8 + sub];
 #pragma unroll
             for (int r = 0; r < RW; r++) {
                 float pr = 0.0f;
@@ -738,6 +746,7 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_tokens_kernel(const uint32
                                                                     const uint32_t tb5, const uint32_t tb6, const uint32_t tb7,
                                                                     const uint32_t total_tasks, const uint32_t T, const GemvGroup g) {
     __shared__ uint4 xs[TT * BPL * 128];
+    __shared__ float sxs[TT * BPL * 64];
     const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
     uint32_t pi = 0;
     pi = task >= tb1 ? 1u : pi;
@@ -750,7 +759,7 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_tokens_kernel(const uint32
     pi = __builtin_amdgcn_readfirstlane(pi);
     const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
     rows_tokens_task_int8<BPL, RW, TT>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
-                                       p.x_token_stride, p.out, p.out_token_stride, p.R, T, p.out_f16, p.act, task - p.task_begin, xs);
+                                       p.x_token_stride, p.out, p.out_token_stride, p.R, T, p.out_f16, p.act, task - p.task_begin, xs, sxs);
 }
 
 // The same two kernels with wall-clock stamps (one 32-byte record per wave at stamps[(workgroup * 4 + wave) * 4]).
@@ -868,7 +877,7 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
     ksplit_task_int8<RWG, WK>(w, mm, x, out, R, total_tasks, flags, red);
 }
 
-// Runs of TT tokens on the K-split layout (built for TT = 2): a lane keeps its 16 activations of every token in registers, converts a
+// Runs of TT tokens on the K-split layout (built for TT = 2 and 4): a lane keeps its 16 activations of every token in registers, converts a
 // row's codes once and meets every token with them; the RWG x TT partial sums of a wave close inside DPP rows and meet in LDS.
 template <int RWG, int WK, int TT>
 __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_tokens_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
@@ -1444,12 +1453,14 @@ int launch_rows_tokens_int8(hipStream_t stream, const GemvGroup &g) {
     return check_launch("matmul_vec_int8");
 }
 
-// Runs of two tokens.  (Four tokens per pass were built on the same layout and measured at 1.93 against 1.96 ms per 7B step for
-// the one-shot kernel at 4 tokens, 1.92 against 1.94 at 3: there the vector ALU is as busy as the memory system whichever
-// way the lanes are laid out, and the launches are single rounds of workgroups that load, then compute, in step.  Not kept.)
+// Runs of 2 tokens take two tokens per pass, runs of 3 and 4 four.  7B step against the one-shot kernel: 1.50 / 1.89 / 1.90 ms
+// at 2 / 3 / 4 tokens against 1.55 / 1.95 / 1.95.  At 4 tokens the activations a workgroup stages equal its weight bytes and a
+// launch is one or two rounds of workgroups that load, then compute, in step: memory, LDS and vector time add up instead
+// of overlapping (taking the activation sums once per workgroup instead of once per wave removed a quarter of the vector
+// instructions and 2.6 % of the time; capping the occupancy to stagger the rounds lost 0 - 5 %).
 int launch_rows_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
-#define WRQ_ROWS_CASE(B) case B: return launch_rows_tokens_int8<B, 2>(stream, g);
+#define WRQ_ROWS_CASE(B) case B: return g.T <= 2 ? launch_rows_tokens_int8<B, 2>(stream, g) : launch_rows_tokens_int8<B, 4>(stream, g);
     WRQ_ROWS_CASE(1) WRQ_ROWS_CASE(2) WRQ_ROWS_CASE(3) WRQ_ROWS_CASE(4) WRQ_ROWS_CASE(5) WRQ_ROWS_CASE(6) WRQ_ROWS_CASE(7) WRQ_ROWS_CASE(8)
 #undef WRQ_ROWS_CASE
     default: return fail(WRQ_ERR_UNSUPPORTED, "no wave-owns-rows kernel for K = %u at %u tokens", K, g.T);
@@ -1468,7 +1479,7 @@ int launch_ksplit_tokens_int8(hipStream_t stream, const GemvGroup &g) {
 
 int launch_ksplit_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
-#define WRQ_KSPLIT_CASE(B) case B: return launch_ksplit_tokens_int8<B, 2>(stream, g);
+#define WRQ_KSPLIT_CASE(B) case B: return g.T <= 2 ? launch_ksplit_tokens_int8<B, 2>(stream, g) : launch_ksplit_tokens_int8<B, 4>(stream, g);
     WRQ_KSPLIT_CASE(10) WRQ_KSPLIT_CASE(12) WRQ_KSPLIT_CASE(14) WRQ_KSPLIT_CASE(16)
 #undef WRQ_KSPLIT_CASE
     default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u at %u tokens", K, g.T);
@@ -1542,8 +1553,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
-        // (runs of 2 tokens take the same layouts with both tokens in one pass)
-        const bool tokens_ok = T == 1 || (T == 2 && tune(kTuneGemvRowsTokens, 1) && args[i].x_token_stride <= 0xffffffffull &&
+        // (runs of 2 .. 4 tokens take the same layouts with 2 or 4 tokens per pass; K up to 8192: their activations have to fit LDS)
+        const bool tokens_ok = T == 1 || (T <= 4 && tune(kTuneGemvRowsTokens, 1) && args[i].x_token_stride <= 0xffffffffull &&
                                           args[i].out_token_stride <= 0xffffffffull);
         const bool waverows = oneshot && quant == kInt8 && in_f16 && tokens_ok && rows_kernel_has(args[i].K) && (T == 1 || args[i].K <= 8192) &&
                               ((uintptr_t)args[i].scale % 16 == 0) && tune(kTuneGemvWaveRows, 1);

@@ -63,7 +63,7 @@ enum TuneKey {
     kTuneGemmTail,     // gemm_tail: 0 keeps a grid a little above two workgroups per CU in one launch
     kTuneGemvWaveRows, // gemv_waverows: 0 keeps one-token int8 products off the wave-owns-rows kernel, 2 sends every K it is built for there
     kTuneGemmPrio,     // gemm_prio: 0 leaves the wave priority alone around the matrix work of a chunk step (default: raised)
-    kTuneGemvRowsTokens, // gemv_rows_tokens: 0 keeps int8 runs of 2 tokens off the wave-owns-rows and K-split kernels
+    kTuneGemvRowsTokens, // gemv_rows_tokens: 0 keeps int8 runs of 2 .. 4 tokens off the wave-owns-rows and K-split kernels
     kTuneCount
 };
 // The override of `key`, or `fallback` when it is unset.
