@@ -18,7 +18,9 @@
  * products on further streams run unsplit: correct, slower).  A call recorded into a HIP graph keeps
  * the slice of the stream it was captured on, so two graphs captured on ONE stream must not be
  * replayed at the same time on different streams; wrq_matmul_mat_int8_noalloc has one fixed array
- * per device and its calls must not overlap at all.
+ * per device and its calls must not overlap at all.  Streams are told apart by their handle:
+ * hipStreamPerThread is one handle for every thread, so split products issued on it from several
+ * threads share a slice and must not overlap either (give such threads streams of their own).
  *
  * Shapes use the reference's order, x fastest (src/tensor/shape.rs:97): a matrix
  * `[K, R, B, 1]` holds B * R rows of K contiguous elements.
