@@ -509,6 +509,8 @@ def stamps_timeline(wrq, torch, args, layers, C, H):
     tick_us = 0.01  # the wall-clock counter runs at 100 MHz
     import numpy as np
     rows = {k: [] for k in range(4)}
+    xcd_ends = {k: [] for k in range(4)}
+    xcd_starts = {k: [] for k in range(4)}
     last_end = None
     for i in range(n_launch):
         name, wgs, waves = kinds[i % 4]
@@ -517,7 +519,12 @@ def stamps_timeline(wrq, torch, args, layers, C, H):
         first, end = r[:, 0].min(), r[:, 3].max()
         if i >= 4:  # the first layer starts from an idle machine
             life = r[:, 3] - r[:, 0]
-            rows[i % 4].append(dict(span=end - first, gap=first - last_end, last_start=r[:, 0].max() - first, issue=np.median(r[:, 1] - r[:, 0]),
+            xcd = (np.arange(wgs * waves) // waves) % 8  # workgroup b runs on XCD b mod 8
+            xcd_end = np.array([r[xcd == q, 3].max() for q in range(8)])
+            xcd_ends[i % 4].append(xcd_end - first)
+            xcd_starts[i % 4].append(np.array([r[xcd == q, 0].min() for q in range(8)]) - first)
+            rows[i % 4].append(dict(span=end - first, gap=first - last_end, xcd_spread=float(xcd_end.max() - xcd_end.min()),
+                                    last_start=r[:, 0].max() - first, issue=np.median(r[:, 1] - r[:, 0]),
                                     data=np.median(r[:, 2] - r[:, 1]), finish=np.median(r[:, 3] - r[:, 2]), life=np.median(life),
                                     life95=np.percentile(life, 95), first_done=r[:, 2].min() - first))
         last_end = end
@@ -525,7 +532,7 @@ def stamps_timeline(wrq, torch, args, layers, C, H):
     print("Int8 decode step, %d layers, graph replay: %.4f ms with the product kernels, %.4f ms with the stamped builds; "
           "first stamp to last stamp of the stamped step %.4f ms" % (len(layers), plain_ms, stamped_ms, step_span / 1e3))
     print("per launch, microseconds, mean over layers 1..%d (medians over the waves of a launch where marked):" % (len(layers) - 1))
-    hdr = "%-26s %6s %6s %9s %9s %10s %9s %9s %9s %9s %9s %10s" % ("launch", "wgs", "waves", "gap", "span", "last_start", "issue~", "data~", "finish~", "life~", "life95", "first_done")
+    hdr = "%-26s %6s %6s %9s %9s %10s %9s %9s %9s %9s %9s %10s %10s" % ("launch", "wgs", "waves", "gap", "span", "last_start", "issue~", "data~", "finish~", "life~", "life95", "first_done", "xcd_spread")
     print(hdr)
     out = {}
     tot_gap = tot_span = 0.0
@@ -535,12 +542,16 @@ def stamps_timeline(wrq, torch, args, layers, C, H):
         out[name] = {f: round(v, 3) for f, v in m.items()}
         tot_gap += m["gap"]
         tot_span += m["span"]
-        print("%-26s %6d %6d %9.2f %9.2f %10.2f %9.2f %9.2f %9.2f %9.2f %9.2f %10.2f" % (name, wgs, wgs * waves, m["gap"], m["span"], m["last_start"], m["issue"],
-              m["data"], m["finish"], m["life"], m["life95"], m["first_done"]))
+        print("%-26s %6d %6d %9.2f %9.2f %10.2f %9.2f %9.2f %9.2f %9.2f %9.2f %10.2f %10.2f" % (name, wgs, wgs * waves, m["gap"], m["span"], m["last_start"], m["issue"],
+              m["data"], m["finish"], m["life"], m["life95"], m["first_done"], m["xcd_spread"]))
+    for k in range(4):
+        print("%-26s last wave end per XCD 0..7, after the launch's first start: %s; first wave start: %s" % (
+            kinds[k][0], " ".join("%.2f" % v for v in np.mean(xcd_ends[k], axis=0)), " ".join("%.2f" % v for v in np.mean(xcd_starts[k], axis=0))))
     print("layer: gaps %.2f us + spans %.2f us = %.2f us (stamped); the product step is %.2f us per layer" % (tot_gap, tot_span, tot_gap + tot_span, plain_ms * 1e3 / len(layers)))
     print("gap: first wave start minus last wave end of the launch before; span: first wave start to last wave end; last_start: when the last wave of")
     print("the launch started, after the first; issue~: entry to every load requested; data~: from there to every row accumulated; finish~: reduction")
-    print("and store; life~/life95: wave lifetime, median and 95th percentile; first_done: first wave anywhere with every row accumulated, after the first start.")
+    print("and store; life~/life95: wave lifetime, median and 95th percentile; first_done: first wave anywhere with every row accumulated, after the first start;")
+    print("xcd_spread: between the XCD whose last wave ends first and the one whose last wave ends last.")
     print(json.dumps({"stamps": out, "plain_ms": round(plain_ms, 4), "stamped_ms": round(stamped_ms, 4)}))
 
 
