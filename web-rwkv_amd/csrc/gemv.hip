@@ -793,6 +793,46 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_stamped_kernel(const
                                   p.R, p.out_f16, p.act, task - p.task_begin, xs, stamps);
 }
 
+// Groups of up to four products: the descriptor of the FIRST product arrives with the kernel arguments (14 dwords, all preloaded
+// in SGPRs), so the workgroups that start a launch -- the first tasks belong to the first product -- issue their loads without
+// waiting for a scalar load of cold argument memory (0.35 - 0.45 us, measured as the difference in first-wave start between this
+// kernel and the single-product one); workgroups of the other products fetch their descriptor as before, when the machine is busy.
+template <int BPL, int RW, bool STAMP>
+__device__ __forceinline__ void rows_group4_body(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t total_tasks,
+                                                 const uint8_t *w0, const uint32_t *mm0, const uint16_t *x0, void *out0, const uint32_t R0,
+                                                 const uint32_t flags0, const GemvGroup &g, uint4 *xs, unsigned long long *stamps) {
+    const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    uint32_t pi = 0;
+    pi = task >= tb1 ? 1u : pi;
+    pi = task >= tb2 ? 2u : pi;
+    pi = task >= tb3 ? 3u : pi;
+    pi = __builtin_amdgcn_readfirstlane(pi);
+    if (pi == 0) {
+        rows_task_int8<BPL, RW, STAMP>(w0, mm0, x0, out0, R0, (int)(flags0 & 1u), (int)(flags0 >> 1), task, xs, stamps);
+    } else {
+        const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
+        rows_task_int8<BPL, RW, STAMP>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
+                                       p.out, p.R, p.out_f16, p.act, task - p.task_begin, xs, stamps);
+    }
+}
+
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_group4_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t total_tasks,
+                                                                    const uint8_t *w0, const uint32_t *mm0, const uint16_t *x0, void *out0,
+                                                                    const uint32_t R0, const uint32_t flags0, const GemvGroup g) {
+    __shared__ uint4 xs[BPL * 128];
+    rows_group4_body<BPL, RW, false>(tb1, tb2, tb3, total_tasks, w0, mm0, x0, out0, R0, flags0, g, xs, nullptr);
+}
+
+template <int BPL, int RW>
+__global__ __launch_bounds__(256) void gemv_int8_rows_group4_stamped_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3,
+                                                                            const uint32_t total_tasks, const uint8_t *w0, const uint32_t *mm0,
+                                                                            const uint16_t *x0, void *out0, const uint32_t R0, const uint32_t flags0,
+                                                                            unsigned long long *stamps, const GemvGroup g) {
+    __shared__ uint4 xs[BPL * 128];
+    rows_group4_body<BPL, RW, true>(tb1, tb2, tb3, total_tasks, w0, mm0, x0, out0, R0, flags0, g, xs, stamps);
+}
+
 // int8, one token, f16 activations, long rows (K = WK * 1024, 8192 < K <= 16384): the WK waves of a workgroup split K, every wave
 // takes all RWG rows of the task over its 1024 elements -- one 16-byte chunk per lane and row, the lane's 16 activations in
 // registers for all rows (each activation crosses into the workgroup once, no LDS staging), one (min, max) word per chunk.
@@ -1378,6 +1418,11 @@ int launch_rows_int8(hipStream_t stream, const GemvGroup &g) {
                 hipLaunchKernelGGL((gemv_int8_rows_single_stamped_kernel<BPL, RW>), grid, dim3(256), 0, stream, p.w,
                                    reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out,
                                    p.R, g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), st);
+            } else if (g.n <= 4 && tune(kTuneGemvWaveRows, 1) != 3) {
+                const GemvProblem &p = g.p[0];
+                hipLaunchKernelGGL((gemv_int8_rows_group4_stamped_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2],
+                                   g.task_begin[3], g.total_tasks, p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7),
+                                   reinterpret_cast<const uint16_t *>(p.x), p.out, p.R, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), st, g);
             } else {
                 hipLaunchKernelGGL((gemv_int8_rows_group_stamped_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2],
                                    g.task_begin[3], g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, st, g);
@@ -1390,6 +1435,11 @@ int launch_rows_int8(hipStream_t stream, const GemvGroup &g) {
         hipLaunchKernelGGL((gemv_int8_rows_single_kernel<BPL, RW>), grid, dim3(256), 0, stream, p.w,
                            reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x), p.out, p.R,
                            g.total_tasks, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1));
+    } else if (g.n <= 4 && tune(kTuneGemvWaveRows, 1) != 3) { // (gemv_waverows = 3 keeps every group on the general kernel)
+        const GemvProblem &p = g.p[0];
+        hipLaunchKernelGGL((gemv_int8_rows_group4_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2], g.task_begin[3],
+                           g.total_tasks, p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
+                           p.out, p.R, (uint32_t)(p.out_f16 ? 1u : 0u) | ((uint32_t)p.act << 1), g);
     } else {
         hipLaunchKernelGGL((gemv_int8_rows_group_kernel<BPL, RW>), grid, dim3(256), 0, stream, g.task_begin[1], g.task_begin[2], g.task_begin[3],
                            g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, g);
