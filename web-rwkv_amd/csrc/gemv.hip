@@ -741,25 +741,35 @@ __device__ __forceinline__ void rows_tokens_task_int8(const uint8_t *w, const ui
     if (lane < (uint32_t)(RW * TT) && row0 + r < R && t < T) store_out(out, out_f16, (uint64_t)t * out_token_stride + row0 + r, act_apply(act, mine));
 }
 
+// tflags: the run's token count in bits 0 .. 7, f16 output of the first product in bit 8, its activation in bits 9 .. 11, bit 31:
+// more than four products.  As in the one-token kernel the first product's descriptor comes with the (preloaded) arguments.
 template <int BPL, int RW, int TT>
-__global__ __launch_bounds__(256) void gemv_int8_rows_tokens_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t tb4,
-                                                                    const uint32_t tb5, const uint32_t tb6, const uint32_t tb7,
-                                                                    const uint32_t total_tasks, const uint32_t T, const GemvGroup g) {
+__global__ __launch_bounds__(256) void gemv_int8_rows_tokens_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t total_tasks,
+                                                                    const uint8_t *w0, const uint32_t *mm0, const uint16_t *x0, const uint32_t R0,
+                                                                    const uint32_t tflags, const uint32_t x_token_stride0, const GemvGroup g) {
     __shared__ uint4 xs[TT * BPL * 128];
     __shared__ float sxs[TT * BPL * 64];
     const uint32_t task = xcd_task(blockIdx.x, total_tasks, 16 / RW);
+    const uint32_t T = tflags & 0xffu;
     uint32_t pi = 0;
     pi = task >= tb1 ? 1u : pi;
     pi = task >= tb2 ? 2u : pi;
     pi = task >= tb3 ? 3u : pi;
-    pi = task >= tb4 ? 4u : pi;
-    pi = task >= tb5 ? 5u : pi;
-    pi = task >= tb6 ? 6u : pi;
-    pi = task >= tb7 ? 7u : pi;
+    if (tflags >> 31) {
+#pragma unroll
+        for (uint32_t i = 4; i < (uint32_t)kMaxGroup; i++)
+            if (task >= g.task_begin[i]) pi = i;
+    }
     pi = __builtin_amdgcn_readfirstlane(pi);
-    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
-    rows_tokens_task_int8<BPL, RW, TT>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
-                                       p.x_token_stride, p.out, p.out_token_stride, p.R, T, p.out_f16, p.act, task - p.task_begin, xs, sxs);
+    if (pi == 0) {
+        // the output pointer and its token stride are needed last: their scalar load is in flight all the while
+        rows_tokens_task_int8<BPL, RW, TT>(w0, mm0, x0, x_token_stride0, g.p[0].out, g.p[0].out_token_stride, R0, T, (int)((tflags >> 8) & 1u),
+                                           (int)((tflags >> 9) & 7u), task, xs, sxs);
+    } else {
+        const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
+        rows_tokens_task_int8<BPL, RW, TT>(p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7), reinterpret_cast<const uint16_t *>(p.x),
+                                           p.x_token_stride, p.out, p.out_token_stride, p.R, T, p.out_f16, p.act, task - p.task_begin, xs, sxs);
+    }
 }
 
 // The same two kernels with wall-clock stamps (one 32-byte record per wave at stamps[(workgroup * 4 + wave) * 4]).
@@ -1524,8 +1534,11 @@ int launch_ksplit_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
 
 template <int BPL, int TT>
 int launch_rows_tokens_int8(hipStream_t stream, const GemvGroup &g) {
+    const GemvProblem &p = g.p[0];
+    const uint32_t tflags = (g.T & 0xffu) | ((uint32_t)(p.out_f16 ? 1u : 0u) << 8) | (((uint32_t)p.act & 7u) << 9) | (g.n > 4 ? 0x80000000u : 0u);
     hipLaunchKernelGGL((gemv_int8_rows_tokens_kernel<BPL, 2, TT>), dim3(g.total_tasks), dim3(256), 0, stream, g.task_begin[1], g.task_begin[2],
-                       g.task_begin[3], g.task_begin[4], g.task_begin[5], g.task_begin[6], g.task_begin[7], g.total_tasks, g.T, g);
+                       g.task_begin[3], g.total_tasks, p.w, reinterpret_cast<const uint32_t *>(p.scale) + (p.e_base >> 7),
+                       reinterpret_cast<const uint16_t *>(p.x), p.R, tflags, (uint32_t)p.x_token_stride, g);
     return check_launch("matmul_vec_int8");
 }
 
