@@ -362,7 +362,12 @@ __device__ __forceinline__ void oneshot_reduce_store(float (&acc)[ROWS][TT], flo
 // TT > 1 (f16 activations only): the same pass serves up to TT tokens of a short run -- the
 // converted codes of a row meet the activations of every token, (TT + 1) / 2 VALU ops per weight.
 template <typename XT, int ROWS, int NT, bool SINGLE, int TT>
-__global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g) {
+__global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const uint32_t tb1, const uint32_t tb2, const uint32_t tb3, const uint32_t kflags,
+                                                               const uint8_t *w0, const uint16_t *scale0, const void *x0, const uint32_t R0,
+                                                               const GemvGroup g) {
+    // The scalar arguments in front describe the launch's first product (kflags: K in bits 0 .. 23, f16 output in bit 24, the
+    // activation in bits 25 .. 27, bit 31: more than four products) and arrive preloaded in SGPRs: the workgroups that open a
+    // launch belong to the first product and request their loads without waiting for a scalar load of cold argument memory.
     static_assert(TT == 1 || sizeof(XT) == 2, "several tokens per pass: f16 activations only");
     constexpr int NROW16 = NT / 16; // DPP rows per workgroup
     constexpr int XW = sizeof(XT) == 2 ? 2 : 4; // 16-byte loads per token and chunk
@@ -371,12 +376,26 @@ __global__ __launch_bounds__(NT) void gemv_int8_oneshot_kernel(const GemvGroup g
     const uint32_t task = blockIdx.x;
     uint32_t pi = 0;
     if constexpr (!SINGLE) {
+        pi = task >= tb1 ? 1u : pi;
+        pi = task >= tb2 ? 2u : pi;
+        pi = task >= tb3 ? 3u : pi;
+        if (kflags >> 31) {
 #pragma unroll
-        for (uint32_t i = 1; i < (uint32_t)kMaxGroup; i++)
-            if (task >= g.task_begin[i]) pi = i;
+            for (uint32_t i = 4; i < (uint32_t)kMaxGroup; i++)
+                if (task >= g.task_begin[i]) pi = i;
+        }
         pi = __builtin_amdgcn_readfirstlane(pi);
     }
-    const GemvProblem p = g.p[pi]; // by value: one batch of scalar loads
+    GemvProblem p;
+    if (pi == 0) {
+        p = g.p[0]; // the fields not among the scalar arguments (output, token strides) are needed late or not at all
+        p.w = w0, p.scale = scale0, p.x = x0;
+        p.e_base = 0, p.task_begin = 0;
+        p.K = kflags & 0xffffffu, p.R = R0;
+        p.out_f16 = (int)((kflags >> 24) & 1u), p.act = (int)((kflags >> 25) & 7u);
+    } else {
+        p = g.p[pi]; // by value: one batch of scalar loads
+    }
     const uint32_t K = p.K, nchunk = K >> 4;
     const uint32_t row0 = (task - p.task_begin) * ROWS;
     const uint32_t rows_valid = min((uint32_t)ROWS, p.R - row0);
@@ -1365,16 +1384,22 @@ int launch_group_xt(hipStream_t stream, const GemvGroup &g, int rows, int sl, in
 template <typename XT, int ROWS, bool SINGLE, int TT>
 int launch_oneshot_nt_n(hipStream_t stream, const GemvGroup &g, int nt) {
     const dim3 grid(g.total_tasks);
+    const GemvProblem &p = g.p[0];
+    if (p.K > 0xffffffu) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", p.K, 0xffffffu);
+    const uint32_t kflags = p.K | ((uint32_t)(p.out_f16 ? 1u : 0u) << 24) | (((uint32_t)p.act & 7u) << 25) | (g.n > 4 ? 0x80000000u : 0u);
+#define WRQ_I8_LAUNCH(N, T_) hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, N, SINGLE, T_>), grid, dim3(N), 0, stream, g.task_begin[1], g.task_begin[2], \
+                                                g.task_begin[3], kflags, p.w, p.scale, p.x, p.R, g)
     if (nt >= 1024 && TT == 1)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 1024, SINGLE, 1>), grid, dim3(1024), 0, stream, g);
+        WRQ_I8_LAUNCH(1024, 1);
     else if (nt >= 512)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 512, SINGLE, TT>), grid, dim3(512), 0, stream, g);
+        WRQ_I8_LAUNCH(512, TT);
     else if (nt >= 256)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 256, SINGLE, TT>), grid, dim3(256), 0, stream, g);
+        WRQ_I8_LAUNCH(256, TT);
     else if (nt >= 128)
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 128, SINGLE, TT>), grid, dim3(128), 0, stream, g);
+        WRQ_I8_LAUNCH(128, TT);
     else
-        hipLaunchKernelGGL((gemv_int8_oneshot_kernel<XT, ROWS, 64, SINGLE, TT>), grid, dim3(64), 0, stream, g);
+        WRQ_I8_LAUNCH(64, TT);
+#undef WRQ_I8_LAUNCH
     return check_launch("matmul_vec_int8");
 }
 
