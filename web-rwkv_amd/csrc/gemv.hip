@@ -9,8 +9,12 @@
 // own costs about as much again.
 //
 // Every packed byte is read once, 16 bytes per lane, 1 KiB per wave instruction, contiguous
-// along a weight row; accumulation is f32 throughout.  Three kernel families:
+// along a weight row; accumulation is f32 throughout.  Four kernel families:
 //
+//   * the wave-owns-rows and K-split kernels (gemv_int8_rows_*_kernel, gemv_int8_ksplit_*_kernel) -- int8 decode with f16
+//     activations and K a multiple of 1024, one token or a run of up to 4: a wave streams whole rows (or, for long rows, a
+//     1024-element slice of 8 rows) with full-line loads and closes its sums without a workgroup-wide exchange.  Their
+//     arguments are scalars that arrive preloaded in SGPRs, for groups the first product's descriptor among them.
 //   * one-shot kernels (gemv_int8_oneshot_kernel, gemv_nf4_oneshot_kernel,
 //     gemv_fp16_oneshot_kernel) -- the decode path: one token, or a run of up to 4 (int8) /
 //     2 (nf4) tokens of f16 activations.  One short-lived workgroup per task (4 or 8 rows over
