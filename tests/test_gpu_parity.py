@@ -286,6 +286,13 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
                               for i, (m, x, o) in enumerate(zip(mats, xs, outs))])
         for i, (o, truth) in enumerate(zip(outs, truths)):
             assert_close(host(o).astype(np.float32), np.square(np.maximum(truth, 0.0)) if i == 2 else truth, EPS, f"K={K} group member {i}")
+        # groups of two to four take a kernel of their own (the first product's descriptor travels with the arguments)
+        for n in (2, 3, 4):
+            outs = [torch.full((1, R), float("nan"), dtype=torch.float16 if i % 2 else torch.float32, device="cuda") for i, R in enumerate(rows[:n])]
+            gpu.matmul_vec_group([(m, dev(x), o, gpu.ACT_SQUARED_RELU if i == 0 else gpu.ACT_NONE, False, {})
+                                  for i, (m, x, o) in enumerate(zip(mats[:n], xs[:n], outs))])
+            for i, (o, truth) in enumerate(zip(outs, truths[:n])):
+                assert_close(host(o).astype(np.float32), np.square(np.maximum(truth, 0.0)) if i == 0 else truth, EPS, f"K={K} group of {n}, member {i}")
     overrides(gemv_waverows=2)
     # a z-offset input view and an offset output view (v6: att_sx.view(.., .., i, ..), src/runtime/v6.rs:806-829)
     parent = gen_f16(rng, (5, 1, K), 1.0)
