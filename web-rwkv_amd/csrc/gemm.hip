@@ -698,12 +698,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 
 // Second half of a split-K launch: sum of the partial tiles over the splits, activation, output type, for every
 // product of the launch (blockIdx.y).  One thread per lane slot of the first kernel's tiles (same decoding).
-__global__ __launch_bounds__(256) void gemm_finish_kernel(const GemmArgs ga, uint32_t splits, uint32_t rw, uint32_t mrt, uint32_t ntile) {
+// The launch is a few microseconds long, so the scalar load of cold argument memory in front of its first load counts: what the
+// first product needs (its partial tiles, output, extents) comes as leading scalar arguments, preloaded in SGPRs; the other
+// products of a group read their descriptor.  geom: rw | mrt << 4 | ntile << 8 | f16 output of the first product << 16 | its
+// activation << 17.
+__global__ __launch_bounds__(256) void gemm_finish_kernel(uint32_t splits, const uint32_t geom, const float *scratch0, void *out0, const uint32_t row_tiles0,
+                                                          const uint32_t tblocks, const uint32_t B0, const uint32_t T0, const uint32_t R0,
+                                                          const uint32_t out_token_stride0, const uint32_t split_from, const uint32_t splits_low,
+                                                          const GemmArgs ga) {
+    const uint32_t rw = geom & 15u, mrt = (geom >> 4) & 15u, ntile = (geom >> 8) & 255u;
     const uint32_t pi = blockIdx.y;
-    const MatmulArgs a = ga.m[pi];
-    const float *scratch = ga.scratch[pi];
+    MatmulArgs a;
+    const float *scratch;
+    uint32_t row_tiles, tile_begin;
+    if (pi == 0) {
+        a.out = out0, a.B = B0, a.T = T0, a.R = R0, a.out_token_stride = out_token_stride0;
+        a.out_batch_stride = B0 > 1 ? ga.m[0].out_batch_stride : 0;
+        a.out_f16 = (int)((geom >> 16) & 1u), a.act = (int)((geom >> 17) & 7u);
+        scratch = scratch0, row_tiles = row_tiles0, tile_begin = 0;
+    } else {
+        a = ga.m[pi];
+        scratch = ga.scratch[pi], row_tiles = ga.row_tiles[pi], tile_begin = ga.tile_begin[pi];
+    }
     if (!scratch) return; // no tile of this product was split
-    const uint32_t tblocks = ga.tblocks, row_tiles = ga.row_tiles[pi];
     const uint32_t nwg = (row_tiles + 7) / 8 * 8 * tblocks;
     const uint32_t per_wg = rw * mrt * ntile * 64; // lane slots per workgroup tile
     const uint64_t slots = (uint64_t)a.B * nwg * per_wg;
@@ -714,7 +731,7 @@ __global__ __launch_bounds__(256) void gemm_finish_kernel(const GemmArgs ga, uin
     const uint64_t bw = q / per_wg;
     const uint32_t wg = (uint32_t)(bw % nwg), b = (uint32_t)(bw / nwg);
     const uint32_t n = tp % ntile, wi = tp / ntile; // wi = wave * mrt + i
-    if (ga.tile_begin[pi] + wg < ga.split_from) splits = ga.splits_low;
+    if (tile_begin + wg < split_from) splits = splits_low;
     if (splits <= 1) return; // stored directly by a launch without a split
     uint32_t row_tile, tblock;
     tile_of_block(wg, tblocks, row_tile, tblock);
@@ -871,6 +888,14 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     }
     if (a0.B > 65535u || splits > 65535u) return fail(WRQ_ERR_SIZE, "data size not match: %u vs. %u", a0.B > splits ? a0.B : splits, 65535u);
     ga.tile_offset = 0;
+    auto launch_finish = [&](const GemmArgs &gx, uint32_t nsplits, uint64_t slots) {
+        const MatmulArgs &m0 = gx.m[0];
+        const uint32_t geom = (uint32_t)G::RW | ((uint32_t)MRT << 4) | ((uint32_t)NTILE << 8) | ((uint32_t)(m0.out_f16 ? 1u : 0u) << 16) |
+                              (((uint32_t)m0.act & 7u) << 17);
+        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256), (uint32_t)n), dim3(256), 0, stream, nsplits, geom,
+                           (const float *)gx.scratch[0], m0.out, gx.row_tiles[0], gx.tblocks, m0.B, m0.T, m0.R, (uint32_t)m0.out_token_stride,
+                           gx.split_from, gx.splits_low, gx);
+    };
     ga.split_from = 0;
     ga.splits_low = 0;
     ga.prio = (uint32_t)tune(kTuneGemmPrio, 1);
@@ -919,8 +944,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
             uint64_t slots = 0;
             for (int i = 0; i < n; i++)
                 if (gb.scratch[i]) slots = std::max(slots, slice[i] / 4);
-            hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256), (uint32_t)n), dim3(256), 0, stream, gb, ks,
-                               (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
+            launch_finish(gb, ks, slots);
             return check_launch("matmul_mat (finish)");
         }
     }
@@ -931,8 +955,7 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
     if (splits > 1) {
         uint64_t slots = 0; // of the largest product: smaller ones leave the rest of their grid row idle
         for (int i = 0; i < n; i++) slots = std::max(slots, slice[i] / 4);
-        hipLaunchKernelGGL(gemm_finish_kernel, dim3((uint32_t)((slots + 255) / 256), (uint32_t)n), dim3(256), 0, stream, ga, splits,
-                           (uint32_t)G::RW, (uint32_t)MRT, (uint32_t)NTILE);
+        launch_finish(ga, splits, slots);
         s = check_launch("matmul_mat (finish)");
     }
     return s;
