@@ -644,7 +644,7 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group_kernel(const uint32_
                             p.out_f16, p.act, task - p.task_begin, xs);
 }
 
-// Runs of TT tokens on the same layout (tokens past the run repeat the last one and are not stored; built for TT = 2 and 4):
+// Runs of TT tokens on the same layout (tokens past the run repeat the last one and are not stored; built for TT = 2, 3 and 4):
 // the activations of all tokens reach LDS once per workgroup, a wave converts the codes of a chunk once and meets every
 // token's 32 bytes with them, two rows per wave share each activation read.  Per 16 weight bytes that is 8 permutes
 // and 10 TT dot products and fmas; the sums of a chunk's activations are taken once per workgroup while they are staged.
@@ -950,7 +950,7 @@ __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_kernel(const uint8_t
     ksplit_task_int8<RWG, WK>(w, mm, x, out, R, total_tasks, flags, red);
 }
 
-// Runs of TT tokens on the K-split layout (built for TT = 2 and 4): a lane keeps its 16 activations of every token in registers, converts a
+// Runs of TT tokens on the K-split layout (built for TT = 2, 3 and 4): a lane keeps its 16 activations of every token in registers, converts a
 // row's codes once and meets every token with them; the RWG x TT partial sums of a wave close inside DPP rows and meet in LDS.
 template <int RWG, int WK, int TT>
 __global__ __launch_bounds__(WK * 64) void gemv_int8_ksplit_tokens_kernel(const uint8_t *w, const uint32_t *mm, const uint16_t *x, void *out,
@@ -1571,14 +1571,14 @@ int launch_rows_tokens_int8(hipStream_t stream, const GemvGroup &g) {
     return check_launch("matmul_vec_int8");
 }
 
-// Runs of 2 tokens take two tokens per pass, runs of 3 and 4 four.  7B step against the one-shot kernel: 1.50 / 1.89 / 1.90 ms
-// at 2 / 3 / 4 tokens against 1.55 / 1.95 / 1.95.  At 4 tokens the activations a workgroup stages equal its weight bytes and a
-// launch is one or two rounds of workgroups that load, then compute, in step: memory, LDS and vector time add up instead
-// of overlapping (taking the activation sums once per workgroup instead of once per wave removed a quarter of the vector
-// instructions and 2.6 % of the time; capping the occupancy to stagger the rounds lost 0 - 5 %).
+// A run of T = 2, 3 or 4 tokens takes T tokens per pass.  7B step against the one-shot kernel: 1.47 / 1.67 / 1.87 ms at 2 / 3 / 4
+// tokens against 1.55 / 1.95 / 1.95.  At 4 tokens the activations a workgroup stages equal its weight bytes and a launch is one
+// or two rounds of workgroups that load, then compute, in step: memory, LDS and vector time add up instead of overlapping
+// (taking the activation sums once per workgroup instead of once per wave removed a quarter of the vector instructions and
+// 2.6 % of the time; capping the occupancy to stagger the rounds lost 0 - 5 %; one row per wave at 2 tokens 1.51 against 1.47 ms).
 int launch_rows_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
-#define WRQ_ROWS_CASE(B) case B: return g.T <= 2 ? launch_rows_tokens_int8<B, 2>(stream, g) : launch_rows_tokens_int8<B, 4>(stream, g);
+#define WRQ_ROWS_CASE(B) case B: return g.T <= 2 ? launch_rows_tokens_int8<B, 2>(stream, g) : g.T == 3 ? launch_rows_tokens_int8<B, 3>(stream, g) : launch_rows_tokens_int8<B, 4>(stream, g);
     WRQ_ROWS_CASE(1) WRQ_ROWS_CASE(2) WRQ_ROWS_CASE(3) WRQ_ROWS_CASE(4) WRQ_ROWS_CASE(5) WRQ_ROWS_CASE(6) WRQ_ROWS_CASE(7) WRQ_ROWS_CASE(8)
 #undef WRQ_ROWS_CASE
     default: return fail(WRQ_ERR_UNSUPPORTED, "no wave-owns-rows kernel for K = %u at %u tokens", K, g.T);
@@ -1597,7 +1597,7 @@ int launch_ksplit_tokens_int8(hipStream_t stream, const GemvGroup &g) {
 
 int launch_ksplit_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
-#define WRQ_KSPLIT_CASE(B) case B: return g.T <= 2 ? launch_ksplit_tokens_int8<B, 2>(stream, g) : launch_ksplit_tokens_int8<B, 4>(stream, g);
+#define WRQ_KSPLIT_CASE(B) case B: return g.T <= 2 ? launch_ksplit_tokens_int8<B, 2>(stream, g) : g.T == 3 ? launch_ksplit_tokens_int8<B, 3>(stream, g) : launch_ksplit_tokens_int8<B, 4>(stream, g);
     WRQ_KSPLIT_CASE(10) WRQ_KSPLIT_CASE(12) WRQ_KSPLIT_CASE(14) WRQ_KSPLIT_CASE(16)
 #undef WRQ_KSPLIT_CASE
     default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u at %u tokens", K, g.T);
@@ -1671,7 +1671,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
-        // (runs of 2 .. 4 tokens take the same layouts with 2 or 4 tokens per pass; K up to 8192: their activations have to fit LDS)
+        // (runs of 2 .. 4 tokens take the same layouts with all their tokens in one pass; K up to 8192: their activations have to fit LDS)
         const bool tokens_ok = T == 1 || (T <= 4 && tune(kTuneGemvRowsTokens, 1) && args[i].x_token_stride <= 0xffffffffull &&
                                           args[i].out_token_stride <= 0xffffffffull);
         const bool waverows = oneshot && quant == kInt8 && in_f16 && tokens_ok && rows_kernel_has(args[i].K) && (T == 1 || args[i].K <= 8192) &&
