@@ -184,7 +184,7 @@ def dominant_kernel(quant, tokens):
         if tokens == 1:
             return "gemv_int8_rows_group4_kernel"  # K = 4096 and 14336 are multiples of 1024: the wave-owns-rows kernel (single products: gemv_int8_rows_single_kernel)
         return "gemv_int8_rows_tokens_kernel" if tokens <= 4 else "gemm_kernel"  # the same layout with 2 or 4 tokens per pass
-    return "gemv_nf4_oneshot_kernel" if tokens <= 2 else "gemm_kernel"
+    return "gemv_nf4_oneshot_kernel" if tokens <= 3 else "gemm_kernel"
 
 
 # What a plain streaming read of the same bytes reaches in the same kind of graph on this machine (measured with the probe kernels):

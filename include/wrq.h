@@ -12,7 +12,7 @@
  * and must stay valid until the stream has passed the call.  No entry point
  * allocates, frees or copies to the host.  All may be called from several threads at
  * once, and calls on different streams may overlap in time: products on the matrix-core kernel
- * (wrq_matmul_mat_*, and wrq_matmul_vec_* from 5 tokens on, nf4: 3) may split K over workgroups
+ * (wrq_matmul_mat_*, and wrq_matmul_vec_* from 5 tokens on, nf4: 4) may split K over workgroups
  * and keep partial sums in library-owned scratch memory, of which every stream gets a slice of its
  * own (4 per device, 32 MiB each, handed out in order of first use and kept until the process ends;
  * products on further streams run unsplit: correct, slower).  A call recorded into a HIP graph keeps

@@ -885,7 +885,7 @@ def test_grouped_nf4_products_keep_their_own_tables(gpu, oracle, T, x_dtype):
         assert_close(host(out), truth, EPS, f"op {j} vs float64 with its own table")
 
 
-@pytest.mark.parametrize("T", [1, 2, 4, 5, 32])
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 5, 32])
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
 def test_grouped_decode_products_equal_single_calls(gpu, oracle, kind, T):
     # the independent products of a layer in shared launches: same results as one call each;

@@ -1443,6 +1443,9 @@ template <typename XT, int ROWS>
 int launch_oneshot_nf4_nt(hipStream_t stream, const GemvGroup &g, int nt, int tt) {
     if constexpr (sizeof(XT) == 2) {
         if (tt == 2) return launch_oneshot_nf4_nt_n<XT, ROWS, false, 2>(stream, g, nt);
+        if constexpr (ROWS == 4) {
+            if (tt == 3) return launch_oneshot_nf4_nt_n<XT, ROWS, false, 3>(stream, g, nt);
+        }
     }
     return g.n == 1 ? launch_oneshot_nf4_nt_n<XT, ROWS, true, 1>(stream, g, nt) : launch_oneshot_nf4_nt_n<XT, ROWS, false, 1>(stream, g, nt);
 }
@@ -1665,9 +1668,10 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // one token or a short run: the one-shot kernels (4 rows per workgroup; 8 once that still gives
         // every CU eight workgroups)
         // up to 8 tokens of f16 activations: the same kernel, several tokens per pass
-        // (nf4: 2; at 3 - 4 tokens the activations crowd the registers and the matrix-core kernel is as fast)
-        const bool oneshot = (T == 1 || (in_f16 && T <= (quant == kNf4 ? 2u : 4u))) && tune(kTuneGemvOneshot, 1);
-        const int ott = T == 1 ? 1 : T == 2 ? 2 : 4; // tokens per pass of the one-shot kernel
+        // (nf4: 3, with 4 rows per task at 3 tokens -- 7B step 1.87 ms against 2.02 with 8 rows and 2.26 on the matrix-core kernel;
+        // at 4 tokens the activations crowd the registers: 2.76 - 3.11 ms against 2.28)
+        const bool oneshot = (T == 1 || (in_f16 && T <= (quant == kNf4 ? 3u : 4u))) && tune(kTuneGemvOneshot, 1);
+        const int ott = T == 1 ? 1 : T == 2 ? 2 : (quant == kNf4 ? 3 : 4); // tokens per pass of the one-shot kernel
         int rows = tt > 1 ? 4 : (rows_total / 4 >= 256u * 2 * kGemvWaves ? 4 : 2);
         if (oneshot) rows = rows_total / 8 >= 2048u ? 8 : 4;
         // one token of f16 activations on int8 rows of a multiple of 1024: the wave-owns-rows kernel (all products of a launch share K)
@@ -1692,6 +1696,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // int8, two tokens per pass: 4 rows per task measured faster than 8 (7B step 1.62 against 1.86 ms;
         // nf4 the other way round, 1.82 against 1.65)
         if (oneshot && quant == kInt8 && ott == 2 && !tune_is_set(kTuneGemvRows)) rows = 4;
+        if (oneshot && quant == kNf4 && ott == 3) rows = 4; // three tokens per pass are built for 4 rows per task only
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
         if (waverows) rows = T == 1 ? 4 * rows_per_wave((int)(args[i].K / 1024)) : 8; // several tokens: two rows per wave

@@ -241,11 +241,11 @@ int prepare(Entry entry, Quant quant, const void *w, const Shape4 &mshape, const
                          ((a.x_token_stride * xs) % 16 == 0) && ((a.x_batch_stride * xs) % 16 == 0) &&
                          ((uintptr_t)a.out % (4 * osz) == 0) && ((a.out_token_stride * osz) % (4 * osz) == 0) &&
                          ((a.out_batch_stride * osz) % (4 * osz) == 0);
-    // decode entry point with several tokens: up to 4 (int8, fp16) or 2 (nf4) tokens of f16
+    // decode entry point with several tokens: up to 4 (int8, fp16) or 3 (nf4) tokens of f16
     // activations share one pass of the one-shot VALU kernels (7B int8 step: 1.8 - 2.1 ms at 2 - 4
     // tokens against 2.8 ms; f16 head: 97 us at 4 tokens against 120); longer runs go to the
     // matrix-core kernel.
-    const uint64_t chunk_min_t = (uint64_t)tune(kTuneVecChunkMinT, quant == kNf4 ? 3 : 5);
+    const uint64_t chunk_min_t = (uint64_t)tune(kTuneVecChunkMinT, quant == kNf4 ? 4 : 5);
     // f32 activations cost the matrix-core kernel a second LDS tile and a second product chain (they are split
     // into two f16 halves there, exact to 2^-22 for |x| <= 65535): below 16 tokens the VALU kernels, which take
     // f32 as it is, are the faster choice and have no range limit
