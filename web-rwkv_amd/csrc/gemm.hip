@@ -977,9 +977,10 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
     // long rows against 256 tokens and more also take the 128-token tile (measured on 4096 x 14336: 7 % faster)
-    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128 && n == 1) ? 2 : (T > 64 && (rt >= (1u << 23) || (T >= 256 && a.K >= 8192))) ? 8 : 4;
+    // (long rows from 193 tokens on: two 128-token blocks, 4096 x 14336 at 224 tokens 54.0 against 56.6 - 59.6 us)
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128 && n == 1) ? 2 : (T > 64 && (rt >= (1u << 23) || (T > 192 && a.K >= 8192))) ? 8 : 4;
     int mrt = 2, kg = 1;
-    uint32_t ksplit = 1;
+    uint32_t ksplit = 1, pinned_split = 0; // pinned_split: a measured choice that the rule of split_for() does not produce
     uint64_t wgs = 0; // workgroups of one split
     auto tblocks_of = [&](int nt) { return (uint64_t)(T + 16 * nt - 1) / (16 * nt); };
     // K is split over the grid until there are one (narrow tiles) to four workgroups per CU, at most
@@ -989,10 +990,13 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     // CUs stays unsplit
     auto split_for = [&]() {
         wgs = (uint64_t)((rows * kg + 64 * mrt - 1) / (64 * mrt)) * tblocks_of(ntile) * a.B;
-        const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? 640 : 1024;
+        // (64-token tiles of long rows: three workgroups per CU still pay -- 4096 x 14336 at 160 and 192 tokens, 96 tiles: an
+        // 8-way split 50.4 / 51.2 us against 53.7 / 54.0 us with 4)
+        const uint64_t target = ntile <= 2 ? 256 : ntile == 4 ? (steps >= 64 ? 768 : 640) : 1024;
         ksplit = 1;
         while (kg == 1 && ksplit < 8 && wgs * ksplit * 2 <= target && steps / (ksplit * 2) >= 4) ksplit *= 2;
         if (n >= 2 && wgs >= 200 && ntile != 4) ksplit = 1;
+        if (pinned_split) ksplit = pinned_split;
     };
     // 64-row tiles where they give about one workgroup per CU without a split of K (a 16-token tile:
     // also below that); otherwise 128-row tiles, fewer activation copies per weight byte, and more splits
@@ -1001,6 +1005,46 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     if (QUANT != kFp16 && wgs64 >= 200 && wgs64 <= 320 && (ntile == 1 || (QUANT == kNf4 && ntile == 2))) {
         // about one 64-row workgroup per CU at a narrow token tile: two workgroups of 32 rows with two
         // k groups each keep twice the weight bytes in flight per CU
+        mrt = 1;
+        kg = 2;
+    }
+    // The choices below were checked against a sweep of all sixteen tile shapes x four splits per launch kind of the 7B layer
+    // ({att.k, v, r, g}, att.output, {ffn.key, ffn.receptance}, ffn.value) at 4 .. 256 tokens, both formats.
+    if (QUANT == kInt8 && ntile == 2 && wgs64 >= 200 && wgs64 <= 256) {
+        // int8, 17 .. 32 tokens, about 16384 rows: 64 rows x 32 tokens with two k groups (the attention group 20.2 - 20.7 us
+        // against 22.6 - 22.9 us with 64-row tiles of one k group)
+        mrt = 2;
+        kg = 2;
+    }
+    if (QUANT == kNf4 && ntile == 2 && wgs64 > 256 && wgs64 <= 320) {
+        // nf4, 17 .. 32 tokens, a little more than one 64-row tile per CU ({ffn.key, ffn.receptance}): the same tile with K
+        // split four ways over the grid, 29.4 - 30.4 us against 33.0 - 34.2 us unsplit with 32-row tiles
+        mrt = 2;
+        kg = 2;
+        pinned_split = 4;
+    }
+    if (QUANT == kNf4 && n == 1 && a.B == 1 && a.K > 8192 && rows > 2048 && rows <= 4096 && T <= 32) {
+        // nf4, a small product with long rows (ffn.value) at up to 32 tokens: 64 rows x two k groups, K split 8 ways
+        // (19.4 - 19.7 us against 21.1 - 21.5 us up to 16 tokens, 22.2 - 22.8 against 24.0 from 17 on)
+        mrt = 2;
+        kg = 2;
+        pinned_split = 8;
+    }
+    if (QUANT != kFp16 && T > 64 && T <= 96 && ntile == 4 && a.B == 1) {
+        // 65 .. 96 tokens are three 32-token blocks or two 64-token blocks, the second one at most half full.  Where the wide
+        // blocks give a little more than one 128-row tile per CU (and the grid then needs a split and a cut), the narrow ones
+        // fill the CUs unsplit: {ffn.key, ffn.receptance} 40.5 - 41.2 us against 48 - 50 us (int8), 56 against 60 - 61 us (nf4)
+        const uint64_t row_tiles = (rows + 127) / 128;
+        if (row_tiles * 2 > 256 && row_tiles * 3 <= 512) {
+            ntile = 2;
+            pinned_split = 1;
+        }
+    }
+    if (QUANT == kInt8 && n == 1 && a.B == 1 && a.K <= 8192 && rows > 2048 && rows <= 4096 && T > 16 && T <= 64) {
+        // int8, a small single product (att.output) at 17 .. 64 tokens: 32 rows x 16 tokens with two k groups and no split over
+        // the grid -- no partial sums, no finish launch (11.7 - 11.9 us against 12.8 - 13.4 us up to 32 tokens, 14.2 - 14.7
+        // against 14.3 - 15.3 us up to 64)
+        ntile = 1;
         mrt = 1;
         kg = 2;
     }
@@ -1032,7 +1076,10 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     if (kg != 1 && kg != 2 && kg != 4) kg = 1;
     if (kg == 4 && (mrt != 1 || ntile > 2)) kg = 2;
     if (kg == 2 && ntile > 4) kg = 1;
-    if (tune_is_set(kTuneGemmNtile) || tune_is_set(kTuneGemmMrt) || tune_is_set(kTuneGemmKg)) split_for();
+    if (tune_is_set(kTuneGemmNtile) || tune_is_set(kTuneGemmMrt) || tune_is_set(kTuneGemmKg)) {
+        pinned_split = 0; // a pinned tile shape takes the split of the general rule
+        split_for();
+    }
     ksplit = (uint32_t)tune(kTuneGemmKsplit, (int)ksplit);
     if (ksplit < 1) ksplit = 1;
 
