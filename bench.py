@@ -50,6 +50,9 @@ def nf4_bytes(K, R, T=1, out_size=2):
     return K * R // 2 + 2 * K * R // 64 + 64 + 2 * K * T + out_size * R * T
 
 
+MODEL_SHAPES = {"0b4": (1024, 3584, 24), "1b6": (2048, 7168, 24), "3b": (2560, 8960, 32), "7b": (4096, 14336, 32), "14b": (5120, 17920, 61)}  # d_model, FFN, layers (v6)
+
+
 class Layer:
     pass
 
@@ -779,7 +782,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--quant", choices=["int8", "nf4"], default="int8")
     ap.add_argument("--tokens", type=int, default=1, help="tokens per step (1 = decode; 128 = a prefill chunk)")
-    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=None, help="default: the model's depth (32 for the 7B shape of the metric)")
+    ap.add_argument("--model", choices=sorted(MODEL_SHAPES), default="7b",
+                    help="layer shape of the step; 7b is the metric's config 4, 1b6 the shape of configs 2 and 3")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-group", action="store_true", help="one launch per product instead of grouped launches of independent products")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -829,7 +834,9 @@ def main():
         return
     probe = run_probe(torch) if args.probe else None
 
-    C, H = 4096, 14336
+    C, H, depth = MODEL_SHAPES[args.model]
+    if args.layers is None:
+        args.layers = depth
     if args.ops:
         ops_table(wrq, torch, args, C)
         return
@@ -901,7 +908,7 @@ def main():
     # counter runs of their own, scaled by the same counters on a 256 MiB plain copy).  The figure is read
     # from the tracked summary of those runs for this workload, which states its commands; null without one.
     traffic = None
-    if args.tokens == 1 and grouped and not args.with_head and args.layers == 32:
+    if args.tokens == 1 and grouped and not args.with_head and args.layers == 32 and args.model == "7b":
         traffic = read_traffic(args.quant)
     kernel = dominant_kernel(args.quant, args.tokens)
     out = {
@@ -918,7 +925,7 @@ def main():
         "dtype": "u8" if args.quant == "int8" else "u4",
         "data": "synthetic",
         "config": {
-            "workload": f"config 4: RWKV-v6 7B-shape ({args.layers} layers, d_model 4096, FFN 14336), all layers {args.quant}, "
+            "workload": f"{'config 4: ' if args.model == '7b' else ''}RWKV-v6 {args.model.upper().replace('B', '.', 1) + 'B' if 'b' in args.model[:-1] else args.model.upper()}-shape ({args.layers} layers, d_model {C}, FFN {H}), all layers {args.quant}, "
                         f"batch 1, {args.tokens} token(s) per step, quantized-matrix path only (8 products per layer)",
             "quant": args.quant, "tokens_per_step": args.tokens, "hip_graph": not args.no_graph, "grouped_launches": grouped,
             "fp16_head": bool(args.with_head),
@@ -952,7 +959,7 @@ def main():
                       "hbm_gbps": round(nbytes4 / (ms4 * 1e-3) / 1e9, 1), "bytes_per_step": nbytes4,
                       "roofline": {"bound": "hbm", "achieved": round(nbytes4 / (ms4 * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                    "frac": round(nbytes4 / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                                   "traffic": read_traffic("nf4") if args.layers == 32 else None,
+                                   "traffic": read_traffic("nf4") if args.layers == 32 and args.model == "7b" else None,
                                    "kernel": dominant_kernel("nf4", 1), "launches_per_step": n4,
                                    "avg_launch_us": round(ms4 * 1e3 / n4, 3), "bytes_per_launch": nbytes4 // n4,
                                    "plain_read_model_frac": plain_read_frac(nbytes4, n4)}}

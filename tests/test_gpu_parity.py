@@ -671,6 +671,40 @@ def test_chunk_k_groups_by_default(gpu, oracle, kind, T):
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("C,H", [(1024, 3584), (2048, 7168), (2560, 8960)], ids=str)
+def test_chunk_tiles_from_the_measured_table(gpu, oracle, kind, C, H, overrides):
+    # the launches of the smaller model sizes take their tile shape and split from the measured table
+    # (csrc/gemm_tuned.inc): {k, v, r, g}, att.output, {ffn.key, ffn.receptance} and ffn.value at run lengths
+    # in several buckets, against float64 on sampled rows -- and once more with the table switched off
+    # (gemm_table = 0), where the rules pick the tile
+    import torch
+
+    announce("chunk tiles from the table", kind, C, H)
+    rng = np.random.default_rng(SEED + 47 + C)
+    mats = {}
+    for R, K in ((C, C), (H, C), (C, H)):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        rows = np.sort(rng.choice(R, 64, replace=False))
+        mats[(R, K)] = (gpu_matrix(gpu, kind, wp, scale), wdeq[rows], rows)
+    for table in (1, 0):
+        overrides(gemm_table=table)
+        for T in (6, 24, 40, 96, 130, 256):
+            for group in ([(C, C)] * 4, [(C, C)], [(H, C), (C, C)], [(C, H)]):
+                xs = [gen_f16(rng, (T, K), 1.0) for _, K in group]
+                outs = [torch.full((T, R), float("nan"), dtype=torch.float32 if i % 2 else torch.float16, device="cuda") for i, (R, _) in enumerate(group)]
+                if len(group) == 1:
+                    mats[group[0]][0].matmul_op(dev(xs[0]), outs[0], turbo=gpu.turbo(T))
+                else:
+                    gpu.matmul_vec_group([(mats[g][0], dev(x), o, gpu.ACT_NONE, False, {}) for g, x, o in zip(group, xs, outs)])
+                for g, x, o in zip(group, xs, outs):
+                    _, wsub, rows = mats[g]
+                    got = host(o)
+                    assert np.isfinite(got).all(), f"{kind} {group} T={T} table={table}"
+                    assert_close(got[:, rows], truth_matmul(wsub, x), EPS, f"{kind} {group} T={T} table={table} vs float64")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
 @pytest.mark.parametrize("T,ksplit", [(128, 2), (256, 1), (252, 1)], ids=str)
 def test_chunk_grid_a_little_above_two_workgroups_per_cu(gpu, oracle, kind, T, ksplit, overrides):
     # 576 workgroups (288 tiles of 128 rows x 64 tokens split in two, or 576 tiles) run as two launches:

@@ -962,6 +962,36 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
 }
 
 // `n` products with one K, token count and batch count (the caller groups them so).
+// Measured tile choices.  web-rwkv_amd/tune_gemm.py times every tile shape and split for the launches of the RWKV model sizes
+// (the four attention projections, att.output, {ffn.key, ffn.receptance}, ffn.key, ffn.value, the head; 8 .. 256 tokens) and
+// writes the fastest per (format, rows, K, run-length bucket) into gemm_tuned.inc.  A launch of f16 activations on one batch
+// whose rows and K lie within 7 % of a measured product takes that entry; everything else goes by the rules below.
+struct TunedRow {
+    uint32_t quant, rows, K;
+    uint16_t cfg[14]; // MRT | NTILE << 4 | KG << 8 | split << 12 per bucket; 0: not measured
+};
+constexpr uint32_t kTunedBuckets[14] = {8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256};
+const TunedRow kTuned[] = {
+#include "gemm_tuned.inc"
+    {~0u, 0u, 0u, {0}}, // end marker
+};
+
+uint32_t tuned_lookup(int quant, uint64_t rows, uint64_t K, uint32_t T) {
+    if (T > kTunedBuckets[13] || rows == 0 || K == 0) return 0;
+    int b = 0;
+    while (kTunedBuckets[b] < T) b++;
+    uint32_t best = 0;
+    uint64_t best_d = ~0ull;
+    for (const TunedRow &r : kTuned) {
+        if (r.quant != (uint32_t)quant || !r.cfg[b]) continue;
+        const uint64_t dr = rows > r.rows ? rows - r.rows : r.rows - rows, dk = K > r.K ? K - r.K : r.K - K;
+        if (dr * 100 > (uint64_t)r.rows * 7 || dk * 100 > (uint64_t)r.K * 7) continue;
+        const uint64_t d = dr * 1000 / r.rows + dk * 1000 / r.K; // per mille off the measured shape
+        if (d < best_d) best_d = d, best = r.cfg[b];
+    }
+    return best;
+}
+
 template <int QUANT, typename XT>
 int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const ScratchPolicy *sp) {
     // Tile choice, from sweeps over the launch shapes of this path (rows 4096 .. 65536, K 2048 ..
@@ -1061,8 +1091,15 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
         mrt = 2;
         kg = 2;
     }
+    bool measured = false;
+    if (QUANT != kFp16 && sizeof(XT) == 2 && a.B == 1 && tune(kTuneGemmTable, 1)) {
+        if (const uint32_t c = tuned_lookup(QUANT, rows, a.K, T)) {
+            mrt = (int)(c & 15u), ntile = (int)((c >> 4) & 15u), kg = (int)((c >> 8) & 15u), pinned_split = c >> 12;
+            measured = true;
+        }
+    }
     split_for();
-    if (QUANT == kInt8 && kg == 1 && T > 64) {
+    if (QUANT == kInt8 && kg == 1 && T > 64 && !measured) {
         // two workgroups fit a CU (512 slots).  A grid of 64-token tiles that fills half of them runs at
         // one wave per SIMD: 32-token tiles double it.
         if (ntile == 4 && wgs * ksplit <= 256) {

@@ -64,6 +64,7 @@ enum TuneKey {
     kTuneGemvWaveRows, // gemv_waverows: 0 keeps one-token int8 products off the wave-owns-rows kernel, 2 sends every K it is built for there
     kTuneGemmPrio,     // gemm_prio: 0 leaves the wave priority alone around the matrix work of a chunk step (default: raised)
     kTuneGemvRowsTokens, // gemv_rows_tokens: 0 keeps int8 runs of 2 .. 4 tokens off the wave-owns-rows and K-split kernels
+    kTuneGemmTable,    // gemm_table: 0 leaves the measured tile table (gemm_tuned.inc) out and picks chunk tiles by the rules alone
     kTuneCount
 };
 // The override of `key`, or `fallback` when it is unset.
