@@ -1767,7 +1767,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         g.total_tasks = tasks;
         if (oneshot && quant == kNf4) {
             const uint32_t nchunk = g.p[0].K / 32;
-            int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk >= 128 ? 128 : 64;
+            // a row in one pass where a workgroup can hold its chunks (idle lanes cost less than a second pass)
+            int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk > 64 ? 128 : 64;
             nt = tune(kTuneGemvNt, nt);
             if (nt > 512) nt = 512;
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
@@ -1797,7 +1798,8 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         if (oneshot) {
             const uint32_t nchunk = g.p[0].K / 16;
             // one lane per 16-byte chunk of a row where a workgroup can hold that many
-            int nt = nchunk > 256 ? 512 : nchunk >= 256 ? 256 : nchunk >= 128 ? 128 : 64;
+            // (the smallest workgroup that takes a row in one pass: 160 chunks on 256 lanes beat two passes of 128 lanes)
+            int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk > 64 ? 128 : 64;
             nt = tune(kTuneGemvNt, nt);
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;
