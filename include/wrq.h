@@ -109,7 +109,7 @@ int wrq_init(void);
  * shape.  An override pins one choice so that a test can reach every instantiation: keys are
  * "gemm_ntile", "gemm_mrt", "gemm_kg", "gemm_ksplit", "gemv_rows", "gemv_nt", "gemv_oneshot",
  * "vec_chunk_min_t", "gemm_tail" (0: a chunk grid a little above two workgroups per CU stays one
- * launch), "gemv_waverows" (0: one-token int8 products stay off the wave-owns-rows kernel), "gemv_rows_tokens" (0: nor do runs of 2 .. 4 tokens), "gemm_prio", "gemm_table" (0: chunk tiles by the rules alone, without the measured table), ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
+ * launch), "gemv_waverows" (0: one-token int8 products stay off the wave-owns-rows kernel), "gemv_rows_tokens" (0: nor do runs of 2 .. 4 tokens), "gemm_prio", "gemm_table" / "gemv_table" (0: chunk tiles / one-shot decode tasks by the rules alone, without the measured tables), ...; value < 0 clears the key.  An environment variable WRQ_<KEY> seen when the
  * library first looks (wrq_init, or the first product) presets the same table; nothing on the launch
  * path reads the environment.  Overrides are process-wide and the launch path reads them without a lock,
  * so a product library must not have them changed under it: once the process has launched any kernel of

@@ -671,6 +671,39 @@ def test_chunk_k_groups_by_default(gpu, oracle, kind, T):
 
 
 @pytest.mark.parametrize("kind", ["int8", "nf4"])
+@pytest.mark.parametrize("C,H", [(2560, 8960), (5120, 17920)], ids=str)
+def test_decode_tasks_from_the_measured_table(gpu, oracle, kind, C, H, overrides):
+    # runs of 1 .. 4 tokens on the launches of model sizes whose lanes and rows per task come from the measured
+    # table of the one-shot kernels (csrc/gemv_tuned.inc), against float64 on sampled rows; once more with the
+    # table switched off (gemv_table = 0)
+    import torch
+
+    announce("decode tasks from the table", kind, C, H)
+    rng = np.random.default_rng(SEED + 53 + C)
+    mats = {}
+    for R, K in ((C, C), (H, C), (C, H)):
+        w = gen_f16(rng, (R, K), 0.02)
+        wp, scale, wdeq = pack(oracle, kind, w)
+        rows = np.sort(rng.choice(R, 64, replace=False))
+        mats[(R, K)] = (gpu_matrix(gpu, kind, wp, scale), wdeq[rows], rows)
+    for table in (1, 0):
+        overrides(gemv_table=table)
+        for T in (1, 2, 3, 4):
+            for group in ([(C, C)] * 4, [(C, C)], [(H, C), (C, C)], [(C, H)]):
+                xs = [gen_f16(rng, (T, K), 1.0) for _, K in group]
+                outs = [torch.full((T, R), float("nan"), dtype=torch.float32 if i % 2 else torch.float16, device="cuda") for i, (R, _) in enumerate(group)]
+                if len(group) == 1:
+                    mats[group[0]][0].matmul_op(dev(xs[0]), outs[0], turbo=False)
+                else:
+                    gpu.matmul_vec_group([(mats[g][0], dev(x), o, gpu.ACT_NONE, False, {}) for g, x, o in zip(group, xs, outs)])
+                for g, x, o in zip(group, xs, outs):
+                    _, wsub, rows = mats[g]
+                    got = host(o)
+                    assert np.isfinite(got).all(), f"{kind} {group} T={T} table={table}"
+                    assert_close(got[:, rows], truth_matmul(wsub, x), EPS, f"{kind} {group} T={T} table={table} vs float64")
+
+
+@pytest.mark.parametrize("kind", ["int8", "nf4"])
 @pytest.mark.parametrize("C,H", [(1024, 3584), (2048, 7168), (2560, 8960)], ids=str)
 def test_chunk_tiles_from_the_measured_table(gpu, oracle, kind, C, H, overrides):
     # the launches of the smaller model sizes take their tile shape and split from the measured table

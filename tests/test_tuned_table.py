@@ -36,6 +36,23 @@ def test_every_bucket_names_an_instantiated_tile():
             assert 16 * ntile < 2 * max(bucket, 16), f"{(quant, r, k)} bucket {bucket}: token tile wider than the run"
 
 
+def test_every_decode_cell_names_a_task_shape_the_kernels_have():
+    tune = importlib.import_module("web-rwkv_amd.tune_gemm")
+    text = open(os.path.join(ROOT, "web-rwkv_amd", "csrc", "gemv_tuned.inc")).read()
+    pat = re.compile(r"^\{(\d+),\s*(\d+)u,\s*(\d+)u,\s*\{([^}]*)\}\},\s*$", re.M)
+    rows = [(int(q), int(r), int(k), [int(c, 0) for c in cells.split(",")]) for q, r, k, cells in pat.findall(text)]
+    assert rows, "empty table"
+    seen = set()
+    for quant, r, k, cells in rows:
+        assert quant in (0, 1) and r > 0 and k > 0
+        assert (quant, r, k) not in seen
+        seen.add((quant, r, k))
+        assert len(cells) == len(tune.DECODE_T) and any(cells)
+        for c in cells:
+            if c:
+                assert (c & 0xfff) in tune.DECODE_LANES and (c >> 12) in tune.DECODE_ROWS
+
+
 def test_table_generation_keeps_the_rules_where_they_are_close(tmp_path, capsys):
     # `table` fills a bucket only where the fastest combination beats the rules by more than 4 %, prefers the smallest
     # grid among near ties, and lets a second-pass (refined) measurement replace the first pass of its case

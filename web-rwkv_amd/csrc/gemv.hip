@@ -1644,6 +1644,35 @@ int launch_generic(hipStream_t stream, Quant quant, int in_f16, const MatmulArgs
 
 } // namespace
 
+// Measured task shapes of the one-shot kernels.  web-rwkv_amd/tune_gemm.py (sweep --decode) times lanes per task x rows per
+// task for the launches of the RWKV model sizes at 1 .. 4 tokens and writes the fastest, where it beats the rules below by more
+// than 4 %, into gemv_tuned.inc; a launch of f16 activations on one batch whose rows and K lie within 7 % of a measured product
+// takes that entry.
+namespace {
+struct TunedDecodeRow {
+    uint32_t quant, rows, K;
+    uint16_t cfg[4]; // runs of 1, 2, 3, 4 tokens: lanes per task | rows per task << 12; 0: the rules decide
+};
+const TunedDecodeRow kTunedDecode[] = {
+#include "gemv_tuned.inc"
+    {~0u, 0u, 0u, {0, 0, 0, 0}}, // end marker
+};
+
+uint32_t tuned_decode_lookup(int quant, uint64_t rows, uint64_t K, uint32_t T) {
+    if (T < 1 || T > 4 || rows == 0 || K == 0) return 0;
+    uint32_t best = 0;
+    uint64_t best_d = ~0ull;
+    for (const TunedDecodeRow &r : kTunedDecode) {
+        if (r.quant != (uint32_t)quant || !r.cfg[T - 1]) continue;
+        const uint64_t dr = rows > r.rows ? rows - r.rows : r.rows - rows, dk = K > r.K ? K - r.K : r.K - K;
+        if (dr * 100 > (uint64_t)r.rows * 7 || dk * 100 > (uint64_t)r.K * 7) continue;
+        const uint64_t d = dr * 1000 / r.rows + dk * 1000 / r.K;
+        if (d < best_d) best_d = d, best = r.cfg[T - 1];
+    }
+    return best;
+}
+} // namespace
+
 // `n` independent products with the same quantisation, input type and token count.
 // Products that do not fit the streaming kernel (odd K, unaligned views, activations too
 // large for LDS together) are launched one by one on the generic kernel.
@@ -1699,6 +1728,10 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
         // nf4, two tokens per pass on long rows (more than 128 chunks of 32): 8 rows per task also where the product is small
         // (7B ffn.value 12.4 against 13.8 us, 1.6B ffn.value 5.8 against 6.5 us)
         if (oneshot && quant == kNf4 && ott == 2 && args[i].K / 32 > 128 && !tune_is_set(kTuneGemvRows)) rows = 8;
+        uint32_t measured = 0; // lanes | rows << 12 of a measured product of this shape (one-shot kernels only)
+        if (oneshot && in_f16 && args[i].B == 1 && !tune_is_set(kTuneGemvRows) && !tune_is_set(kTuneGemvNt) && tune(kTuneGemvTable, 1))
+            measured = tuned_decode_lookup(quant, rows_total, args[i].K, T);
+        if (measured) rows = (int)(measured >> 12);
         if (oneshot && quant == kNf4 && ott == 3) rows = 4; // three tokens per pass are built for 4 rows per task only
         // 8 rows per task need 128 lanes for the final reduction: short rows keep 4
         if (oneshot && args[i].K / (quant == kInt8 ? 16 : 32) < 128) rows = 4;
@@ -1773,6 +1806,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             // a row in one pass where a workgroup can hold its chunks (idle lanes cost less than a second pass)
             int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk > 64 ? 128 : 64;
             if (ott == 3 && nt == 512) nt = 256; // three tokens per pass: two passes of 256 lanes beat one of 512 (7B ffn.value 15.4 against 16.8 us)
+            if (measured) nt = (int)(measured & 0xfffu);
             nt = tune(kTuneGemvNt, nt);
             if (nt > 512) nt = 512;
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
@@ -1804,6 +1838,7 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
             // one lane per 16-byte chunk of a row where a workgroup can hold that many
             // (the smallest workgroup that takes a row in one pass: 160 chunks on 256 lanes beat two passes of 128 lanes)
             int nt = nchunk > 256 ? 512 : nchunk > 128 ? 256 : nchunk > 64 ? 128 : 64;
+            if (measured) nt = (int)(measured & 0xfffu);
             nt = tune(kTuneGemvNt, nt);
             if (rows == 8 && nt < 128) nt = 128; // the tasks were cut for 8 rows
             int s1;

@@ -30,7 +30,7 @@ int fail(int status, const char *fmt, ...) {
 // ---- tuning overrides: read from the environment once, then only from this table
 namespace {
 const char *const kTuneNames[kTuneCount] = {"gemv_oneshot", "gemv_rows", "gemv_sl", "gemv_nt", "gemv_grid", "gemm_ntile", "gemm_mrt",
-                                            "gemm_kg", "gemm_ksplit", "vec_chunk_min_t", "gemm_tail", "gemv_waverows", "gemm_prio", "gemv_rows_tokens", "gemm_table"};
+                                            "gemm_kg", "gemm_ksplit", "vec_chunk_min_t", "gemm_tail", "gemv_waverows", "gemm_prio", "gemv_rows_tokens", "gemm_table", "gemv_table"};
 std::atomic<int> g_tune[kTuneCount];
 std::once_flag g_tune_once;
 std::atomic<bool> g_test_hooks{false}; // WRQ_TEST_HOOKS was set when the library first looked: overrides stay allowed

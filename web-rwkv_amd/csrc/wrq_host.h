@@ -65,6 +65,7 @@ enum TuneKey {
     kTuneGemmPrio,     // gemm_prio: 0 leaves the wave priority alone around the matrix work of a chunk step (default: raised)
     kTuneGemvRowsTokens, // gemv_rows_tokens: 0 keeps int8 runs of 2 .. 4 tokens off the wave-owns-rows and K-split kernels
     kTuneGemmTable,    // gemm_table: 0 leaves the measured tile table (gemm_tuned.inc) out and picks chunk tiles by the rules alone
+    kTuneGemvTable,    // gemv_table: 0 leaves the measured table of the one-shot decode kernels (gemv_tuned.inc) out
     kTuneCount
 };
 // The override of `key`, or `fallback` when it is unset.

@@ -10,6 +10,10 @@ sizes and writes the winners as a table:
   python3 web-rwkv_amd/tune_gemm.py sweep --out gpurun_out/tune/refined.jsonl --refine gpurun_out/tune/sweep.jsonl
   python3 web-rwkv_amd/tune_gemm.py table gpurun_out/tune/sweep.jsonl gpurun_out/tune/refined.jsonl > web-rwkv_amd/csrc/gemm_tuned.inc
 
+The one-shot decode kernels (csrc/gemv.hip, runs of 1 .. 4 tokens on products the wave-owns-rows and K-split
+kernels do not take) have two such choices, lanes per task and rows per task; `sweep --decode` and
+`table --decode` do the same for them (gemv_tuned.inc).
+
 `sweep` pins every combination through wrq_debug_override (WRQ_TEST_HOOKS) and times one HIP graph
 of back-to-back launches over enough copies of the packed weights that none is cached; with --refine
 it measures the rules and the three fastest combinations of a first pass again, in turn and for
@@ -171,13 +175,126 @@ def sweep(args):
                 torch.cuda.empty_cache()
 
 
-def load(paths):
+DECODE_T = (1, 2, 3, 4)  # run lengths of the one-shot decode kernels
+DECODE_LANES = (64, 128, 256, 512)
+DECODE_ROWS = (4, 8)
+
+
+def sweep_decode(args):
+    """Lanes per task and rows per task of the one-shot decode kernels (gemv_*_oneshot_kernel), per launch kind and run length:
+    the library's own choice and the eight combinations, three rounds in turn of at least 20 ms each, median."""
+    os.environ.setdefault("WRQ_TEST_HOOKS", "1")
+    sys.path.insert(0, ROOT)
+    import torch
+
+    wrq = importlib.import_module("web-rwkv_amd")
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    out = open(args.out, "a")
+    wrq.debug_override("gemv_table", 0)
+
+    def timed(fn, launches, min_ms=20.0):
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps, ms = 3, 0.0
+        for attempt in range(2):
+            g.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(reps):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            if ms >= min_ms:
+                break
+            reps = int(reps * min_ms / max(ms, 1e-3)) + 1
+        return ms * 1e3 / reps / launches
+
+    sizes = [s for s in SIZES if not args.sizes or f"{s[0]}x{s[1]}" in args.sizes.split(",")]
+    for quant in args.quant.split(","):
+        pack = wrq.Matrix.quant_u8 if quant == "int8" else wrq.Matrix.quant_nf4
+        for C, H, kinds in sizes:
+            for kind in kinds:
+                prods = products(kind, C, H)
+                nbytes = sum(r * k for r, k in prods) // (1 if quant == "int8" else 2)
+                copies = max(8, min(256, (1 << 30) // nbytes + 1))
+                mats = [[pack((torch.randn((r, k), generator=gen, device="cuda") * 0.02).half()) for r, k in prods] for _ in range(copies)]
+                rows, K = sum(r for r, _ in prods), prods[0][1]
+                for T in DECODE_T:
+                    xs = [torch.randn((T, K), generator=gen, device="cuda").half() for _ in prods]
+                    outs = [torch.empty((T, r), dtype=torch.float16, device="cuda") for r, _ in prods]
+
+                    def fn():
+                        for ms in mats:
+                            if len(ms) == 1:
+                                ms[0].matmul_op(xs[0], outs[0], turbo=False)
+                            else:
+                                wrq.matmul_vec_group([(m, x, o, wrq.ACT_NONE, False, {}) for m, x, o in zip(ms, xs, outs)])
+
+                    timed(fn, copies, 5.0)
+                    acc = collections.defaultdict(list)
+                    for _ in range(3):
+                        acc["rule"].append(timed(fn, copies))
+                        for nt in DECODE_LANES:
+                            for nrows in DECODE_ROWS:
+                                wrq.debug_override("gemv_nt", nt)
+                                wrq.debug_override("gemv_rows", nrows)
+                                acc[(nt, nrows)].append(timed(fn, copies))
+                                wrq.debug_override("gemv_nt", -1)
+                                wrq.debug_override("gemv_rows", -1)
+                    rec = {"quant": quant, "kind": kind, "C": C, "H": H, "rows": rows, "K": K, "n": len(prods), "T": T, "decode": 1}
+                    med = {c: sorted(v)[1] for c, v in acc.items()}
+                    for c, us in med.items():
+                        out.write(json.dumps(dict(rec, cfg=c if isinstance(c, str) else list(c), us=round(us, 3))) + "\n")
+                    best = min((c for c in med if c != "rule"), key=med.get)
+                    print(f"{quant} {C:4d}x{H:5d} {kind:6s} rows={rows:6d} K={K:5d} T={T}  rule {med['rule']:7.2f} us  best {med[best]:7.2f} us {best}", flush=True)
+                    out.flush()
+                    del xs, outs
+                del mats
+                torch.cuda.empty_cache()
+
+
+def table_decode(args):
+    data = load(args.files, decode=True)
+    shapes = sorted({(q, rows, K) for q, rows, K, _ in data})
+    print("// Generated by web-rwkv_amd/tune_gemm.py (sweep --decode, table --decode) on an MI355X; do not edit by hand.")
+    print("// One row per (format, rows of the launch, K): for runs of 1, 2, 3 and 4 tokens on the one-shot decode kernels the fastest")
+    print("// lanes per task | rows per task << 12 where it beats the rules by more than 4 %; 0 = the rules decide.")
+    filled = 0
+    for q, rows, K in shapes:
+        cells = []
+        for T in DECODE_T:
+            e = data.get((q, rows, K, T), {})
+            cands = {c: u for c, u in e.items() if not isinstance(c, str)}
+            if not cands or "rule" not in e:
+                cells.append("0")
+                continue
+            best = min(cands, key=cands.get)
+            near = [c for c, u in cands.items() if u <= cands[best] * 1.01]
+            best = min(near, key=lambda c: (c[0], c[1]))  # the smallest task among near ties
+            if e["rule"] < cands[best] * 1.04:
+                cells.append("0")
+                continue
+            filled += 1
+            cells.append("0x%04x" % (best[0] | best[1] << 12))
+        if any(c != "0" for c in cells):
+            print("{%d, %6du, %6du, {%s}}," % (0 if q == "int8" else 1, rows, K, ", ".join(cells)))
+    print(f"// {filled} cells filled")
+
+
+def load(paths, decode=False):
     d = collections.defaultdict(dict)
     refined = set()
     for p in paths:
         for line in open(p):
             r = json.loads(line)
             if "us" not in r:
+                continue
+            if bool(r.get("decode")) != decode:
                 continue
             key = (r["quant"], r["rows"], r["K"], r["T"])
             if r.get("refined") and key not in refined:  # a second-pass measurement replaces the first pass of its case
@@ -233,12 +350,17 @@ def main():
     s.add_argument("--out", required=True)
     s.add_argument("--quant", default="int8,nf4")
     s.add_argument("--sizes", default="", help="comma-separated CxH subset, e.g. 4096x14336")
+    s.add_argument("--decode", action="store_true", help="sweep the one-shot decode kernels (lanes and rows per task at 1 .. 4 tokens) instead of the chunk kernel")
     s.add_argument("--refine", default="", help="comma-separated sweep files: measure only their three fastest combinations per case, longer and in turn")
     s.add_argument("--defaults-only", action="store_true", help="time only the library's own choices, with and without the table")
     t = sub.add_parser("table")
+    t.add_argument("--decode", action="store_true", help="write gemv_tuned.inc from a sweep --decode")
     t.add_argument("files", nargs="+")
     args = ap.parse_args()
-    (sweep if args.cmd == "sweep" else table)(args)
+    if args.cmd == "sweep":
+        (sweep_decode if args.decode else sweep)(args)
+    else:
+        (table_decode if args.decode else table)(args)
 
 
 if __name__ == "__main__":
