@@ -314,7 +314,7 @@ def test_int8_wave_rows_kernel(gpu, oracle, K, overrides):
 @pytest.mark.parametrize("K", WAVE_ROWS_K)
 def test_int8_wave_rows_kernels_on_short_runs(gpu, oracle, K, overrides):
     # runs of 2, 3 and 4 tokens of f16 activations on int8 rows of a multiple of 1024 take the wave-owns-rows layout (up to 8192, the
-    # tokens' activations in LDS) or the K-split layout (10240 .. 16384), all tokens of the run in one pass.
+    # tokens' activations in LDS) or, at three tokens, the K-split layout (10240 .. 14336), all tokens of the run in one pass.
     # Single products and groups, ragged last tasks, both output types, an activation, token strides through views, the batch axis --
     # against the oracle and float64, and the kernel they replace (gemv_rows_tokens = 0) on the same inputs
     import torch

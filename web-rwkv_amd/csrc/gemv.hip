@@ -866,7 +866,7 @@ __global__ __launch_bounds__(256) void gemv_int8_rows_group4_stamped_kernel(cons
     rows_group4_body<BPL, RW, true>(tb1, tb2, tb3, total_tasks, w0, mm0, x0, out0, R0, flags0, g, xs, stamps);
 }
 
-// int8, one token, f16 activations, long rows (K = WK * 1024, 8192 < K <= 16384): the WK waves of a workgroup split K, every wave
+// int8, one token, f16 activations, long rows (K = WK * 1024: 10240, 12288, 14336): the WK waves of a workgroup split K, every wave
 // takes all RWG rows of the task over its 1024 elements -- one 16-byte chunk per lane and row, the lane's 16 activations in
 // registers for all rows (each activation crosses into the workgroup once, no LDS staging), one (min, max) word per chunk.
 // Request order: activations, scale words, weights; rows are consumed in arrival order; the partial sums of the waves meet in
@@ -1535,7 +1535,8 @@ bool rows_kernel_built(uint32_t K) {
 bool rows_kernel_has(uint32_t K) { return rows_kernel_built(K) && (K <= 8192 || tune(kTuneGemvWaveRows, 1) == 2); }
 
 // Long rows of a single product: the K-split kernel (8 rows per task).
-bool ksplit_kernel_has(uint32_t K) { return K % 1024 == 0 && (K == 10240 || K == 12288 || K == 14336 || K == 16384); }
+// (K = 16384 would be 16 waves per workgroup: 15.6 us against 13.2 us for the one-shot kernel on 4096 x 16384)
+bool ksplit_kernel_has(uint32_t K) { return K == 10240 || K == 12288 || K == 14336; }
 
 template <int WK>
 int launch_ksplit_int8(hipStream_t stream, const GemvGroup &g) {
@@ -1559,7 +1560,6 @@ int launch_ksplit_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     case 10: return launch_ksplit_int8<10>(stream, g);
     case 12: return launch_ksplit_int8<12>(stream, g);
     case 14: return launch_ksplit_int8<14>(stream, g);
-    case 16: return launch_ksplit_int8<16>(stream, g);
     default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u", K);
     }
 }
@@ -1600,9 +1600,10 @@ int launch_ksplit_tokens_int8(hipStream_t stream, const GemvGroup &g) {
 
 int launch_ksplit_tokens_int8_k(hipStream_t stream, const GemvGroup &g, uint32_t K) {
     switch (K / 1024) {
-#define WRQ_KSPLIT_CASE(B) case B: return g.T <= 2 ? launch_ksplit_tokens_int8<B, 2>(stream, g) : g.T == 3 ? launch_ksplit_tokens_int8<B, 3>(stream, g) : launch_ksplit_tokens_int8<B, 4>(stream, g);
-    WRQ_KSPLIT_CASE(10) WRQ_KSPLIT_CASE(12) WRQ_KSPLIT_CASE(14) WRQ_KSPLIT_CASE(16)
-#undef WRQ_KSPLIT_CASE
+    // three tokens only: at two and four the one-shot kernel is faster (see launch_gemv_group)
+    case 10: return launch_ksplit_tokens_int8<10, 3>(stream, g);
+    case 12: return launch_ksplit_tokens_int8<12, 3>(stream, g);
+    case 14: return launch_ksplit_tokens_int8<14, 3>(stream, g);
     default: return fail(WRQ_ERR_UNSUPPORTED, "no K-split kernel for K = %u at %u tokens", K, g.T);
     }
 }
@@ -1709,9 +1710,12 @@ int launch_gemv_group(hipStream_t stream, Quant quant, int in_f16, const MatmulA
                                           args[i].out_token_stride <= 0xffffffffull);
         const bool waverows = oneshot && quant == kInt8 && in_f16 && tokens_ok && rows_kernel_has(args[i].K) && (T == 1 || args[i].K <= 8192) &&
                               ((uintptr_t)args[i].scale % 16 == 0) && tune(kTuneGemvWaveRows, 1);
-        // ... and long rows (8192 < K <= 16384, a multiple of 2048): the K-split kernel, one product per launch
+        // ... and long rows (K = 10240, 12288, 14336): the K-split kernel, one product per launch
+        // (one and three tokens only: measured against the one-shot kernel on 4096 x 14336, the K-split layout takes 10.9 against
+        // 11.9 us at one token but 14.0 / 18.3 against 13.0 / 15.9 us at two / four tokens -- the one-shot kernel has no
+        // three-token pass and spends a four-token one there; 7B step 1.47 -> 1.45 ms at two tokens, 1.87 -> 1.81 ms at four)
         const bool ksplit = oneshot && !waverows && quant == kInt8 && in_f16 && tokens_ok && ksplit_kernel_has(args[i].K) && args[i].B == 1 &&
-                            tune(kTuneGemvWaveRows, 1);
+                            (T == 1 || T == 3) && tune(kTuneGemvWaveRows, 1);
         // long rows (ffn.value, K = 14336): 8 rows x 512 lanes, two chunks per lane, measured best
         if (oneshot && quant == kInt8 && args[i].K / 16 > 512) rows = 8;
         // chunks per lane: cover a whole row at once when it is short enough
