@@ -6,9 +6,9 @@ one is fastest depends on the product's rows, its K, the run length and the form
 simple rule at the small end.  This tool measures all of them for the launch kinds of the RWKV model
 sizes and writes the winners as a table:
 
-  python3 web-rwkv_amd/tune_gemm.py sweep --out gpurun_out/tune/sweep.jsonl     (on an MI355X, about 12 minutes)
-  python3 web-rwkv_amd/tune_gemm.py sweep --out gpurun_out/tune/refined.jsonl --refine gpurun_out/tune/sweep.jsonl
-  python3 web-rwkv_amd/tune_gemm.py table gpurun_out/tune/sweep.jsonl gpurun_out/tune/refined.jsonl > web-rwkv_amd/csrc/gemm_tuned.inc
+  python3 web-rwkv_amd/tune_gemm.py sweep --out sweep.jsonl     (on an MI355X, about 12 minutes)
+  python3 web-rwkv_amd/tune_gemm.py sweep --out refined.jsonl --refine sweep.jsonl
+  python3 web-rwkv_amd/tune_gemm.py table sweep.jsonl refined.jsonl > web-rwkv_amd/csrc/gemm_tuned.inc
 
 The one-shot decode kernels (csrc/gemv.hip, runs of 1 .. 4 tokens on products the wave-owns-rows and K-split
 kernels do not take) have two such choices, lanes per task and rows per task; `sweep --decode` and
