@@ -40,9 +40,10 @@ T_GRID = (8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)  # a run 
 
 # (C, H, kinds): kinds of launches swept for a model size.  A kind is a list of (rows, K) products that share one launch.
 FULL = ("att4", "att3", "att_o", "ffn2", "ffn_k", "ffn_v", "head")
-MAIN = ("att4", "att_o", "ffn2", "ffn_v")
-SIZES = [(1024, 3584, MAIN), (2048, 7168, FULL), (2560, 8960, MAIN), (4096, 14336, FULL), (5120, 17920, MAIN), (2048, 8192, ("ffn_k", "ffn_v")),
-         (4096, 16384, ("ffn_k", "ffn_v"))]
+MAIN = ("att4", "att3", "att_o", "ffn2", "ffn_v")
+WIDE = ("ffn_k", "ffn_v")  # the layers with FFN = 4 x d_model (v7) share everything else with the 3.5 x ones
+SIZES = [(768, 2688, FULL), (1024, 3584, MAIN), (2048, 7168, FULL), (2560, 8960, MAIN), (4096, 14336, FULL), (5120, 17920, MAIN),
+         (768, 3072, WIDE), (1024, 4096, WIDE), (2048, 8192, WIDE), (2560, 10240, WIDE), (4096, 16384, WIDE)]
 
 
 def products(kind, C, H):
@@ -90,6 +91,8 @@ def sweep(args):
         pack = wrq.Matrix.quant_u8 if quant == "int8" else wrq.Matrix.quant_nf4
         for C, H, kinds in sizes:
             for kind in kinds:
+                if args.kinds and kind not in args.kinds.split(","):
+                    continue
                 prods = products(kind, C, H)
                 nbytes = sum(r * k for r, k in prods) // (1 if quant == "int8" else 2)
                 copies = max(8, min(256, (1 << 30) // nbytes + 1))  # a gigabyte of weights: nothing stays cached
@@ -219,6 +222,8 @@ def sweep_decode(args):
         pack = wrq.Matrix.quant_u8 if quant == "int8" else wrq.Matrix.quant_nf4
         for C, H, kinds in sizes:
             for kind in kinds:
+                if args.kinds and kind not in args.kinds.split(","):
+                    continue
                 prods = products(kind, C, H)
                 nbytes = sum(r * k for r, k in prods) // (1 if quant == "int8" else 2)
                 copies = max(8, min(256, (1 << 30) // nbytes + 1))
@@ -350,6 +355,7 @@ def main():
     s.add_argument("--out", required=True)
     s.add_argument("--quant", default="int8,nf4")
     s.add_argument("--sizes", default="", help="comma-separated CxH subset, e.g. 4096x14336")
+    s.add_argument("--kinds", default="", help="comma-separated launch kinds, e.g. att3,ffn_k")
     s.add_argument("--decode", action="store_true", help="sweep the one-shot decode kernels (lanes and rows per task at 1 .. 4 tokens) instead of the chunk kernel")
     s.add_argument("--refine", default="", help="comma-separated sweep files: measure only their three fastest combinations per case, longer and in turn")
     s.add_argument("--defaults-only", action="store_true", help="time only the library's own choices, with and without the table")
