@@ -230,8 +230,10 @@ int wrq_matmul_mat_int8(wrq_stream stream, const wrq_tensor_view *matrix, const 
  * When the product splits K over workgroups, the partial sums go to a fixed 16 MiB array that the
  * library's code object holds on every GPU it runs on, used by this entry point only; its address on
  * a device is looked up once (wrq_init, else the first call on that device).  A product whose
- * partial sums would not fit is refused with WRQ_ERR_SIZE before anything is launched (the plain
- * entry point takes fewer splits instead).  The array keeps nothing between calls and every call
+ * partial sums would not fit at the split the library prefers takes fewer splits (down to none: an
+ * unsplit product needs no array), so its result can differ from the plain entry point's in summation
+ * order; a split pinned through wrq_debug_override that does not fit is refused with WRQ_ERR_SIZE
+ * before anything is launched.  The array keeps nothing between calls and every call
  * writes the part it reads, but calls that overlap in time on one GPU share it: they race.
  */
 int wrq_matmul_mat_int8_noalloc(wrq_stream stream, const wrq_tensor_view *matrix, const wrq_tensor *minmax,

@@ -1,9 +1,9 @@
 """wrq_matmul_mat_int8_noalloc: the chunk product whose split-K partial sums live in a fixed array of
 the library (for callers that cannot allocate), against wrq_matmul_mat_int8 through the C ABI.
 
-The two entry points run the same kernels, so outputs must agree to the last bit; the bar that
-counts is the product bar, |a - b| <= max(eps, eps * max(|a|, |b|)), eps = 2e-3, also held against
-the float64 product of the dequantised weights."""
+The two entry points run the same kernels, so where they take the same split outputs must agree to the
+last bit; the bar that counts is the product bar, |a - b| <= max(eps, eps * max(|a|, |b|)), eps = 2e-3,
+also held against the float64 product of the dequantised weights."""
 import numpy as np
 import pytest
 
@@ -46,10 +46,23 @@ def test_no_alloc_entry_matches_plain_entry_twice(gpu, oracle):
         assert_close(got, truth, EPS, f"noalloc vs float64 {K}x{R}x{T}")
 
 
-def test_no_alloc_entry_refuses_what_does_not_fit(gpu, oracle, overrides):
+def test_no_alloc_entry_takes_fewer_splits_where_the_preferred_split_does_not_fit(gpu, oracle):
     import torch
 
-    # 65536 rows x 32 tokens split 8 ways would need 64 MiB of partial sums: the fixed array holds 16
+    # 4096 rows x 14336 at 192 tokens: the preferred 8-way split would put 24 MiB of partial sums into the 16 MiB array;
+    # the entry point splits 4 ways instead (the plain one, with more room, keeps 8): same bar, different summation order
+    K, R, T = 14336, 4096, 192
+    print("case: no_alloc, fewer splits", K, R, T, flush=True)
+    got, want, truth = _case(gpu, oracle, torch, K, R, T, SEED + 77)
+    assert np.isfinite(got).all()
+    assert_close(got, want, EPS, f"noalloc vs plain entry {K}x{R}x{T}")
+    assert_close(got, truth, EPS, f"noalloc vs float64 {K}x{R}x{T}")
+
+
+def test_no_alloc_entry_refuses_a_pinned_split_that_does_not_fit(gpu, oracle, overrides):
+    import torch
+
+    # 65536 rows x 32 tokens with the split pinned to 8 would need 64 MiB of partial sums: the fixed array holds 16
     K, R, T = 1024, 65536, 32
     rng = np.random.default_rng(SEED + 9)
     wd = torch.from_numpy(rng.integers(0, 256, (R, K), dtype=np.uint8)).cuda()

@@ -868,7 +868,9 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
         return slice_cached;
     };
     if (ksplit > 1 && !slice_base()) ksplit = 1;
-    if (sp && sp->strict && ksplit > 1 && slices * ksplit > cap)
+    // the fixed array of the no-allocation entry point: a split the caller pinned is not second-guessed and is refused when
+    // its partial sums do not fit; the library's own choice gives way to the largest split that fits, as on the plain path
+    if (sp && sp->strict && ksplit > 1 && slices * ksplit > cap && tune_is_set(kTuneGemmKsplit))
         return fail(WRQ_ERR_SIZE, "split-K partial sums of this product need %llu bytes of scratch, the fixed array holds %llu",
                     (unsigned long long)(slices * ksplit * sizeof(float)), (unsigned long long)(cap * sizeof(float)));
     while (ksplit > 1 && slices * ksplit > cap) ksplit /= 2;
