@@ -723,7 +723,7 @@ def test_chunk_tiles_from_the_measured_table(gpu, oracle, kind, C, H, overrides)
         mats[(R, K)] = (gpu_matrix(gpu, kind, wp, scale), wdeq[rows], rows)
     for table in (1, 0):
         overrides(gemm_table=table)
-        for T in (6, 24, 40, 96, 130, 256):
+        for T in (6, 24, 40, 96, 130, 256, 300, 500):
             for group in ([(C, C)] * 4, [(C, C)], [(H, C), (C, C)], [(C, H)]):
                 xs = [gen_f16(rng, (T, K), 1.0) for _, K in group]
                 outs = [torch.full((T, R), float("nan"), dtype=torch.float32 if i % 2 else torch.float16, device="cuda") for i, (R, _) in enumerate(group)]

@@ -965,21 +965,22 @@ int launch_one(hipStream_t stream, const MatmulArgs *args, int n, uint32_t kspli
 
 // `n` products with one K, token count and batch count (the caller groups them so).
 // Measured tile choices.  web-rwkv_amd/tune_gemm.py times every tile shape and split for the launches of the RWKV model sizes
-// (the four attention projections, att.output, {ffn.key, ffn.receptance}, ffn.key, ffn.value, the head; 8 .. 256 tokens) and
+// (the four attention projections, att.output, {ffn.key, ffn.receptance}, ffn.key, ffn.value, the head; 8 .. 512 tokens) and
 // writes the fastest per (format, rows, K, run-length bucket) into gemm_tuned.inc.  A launch of f16 activations on one batch
 // whose rows and K lie within 7 % of a measured product takes that entry; everything else goes by the rules below.
 struct TunedRow {
     uint32_t quant, rows, K;
-    uint16_t cfg[14]; // MRT | NTILE << 4 | KG << 8 | split << 12 per bucket; 0: not measured
+    uint16_t cfg[18]; // MRT | NTILE << 4 | KG << 8 | split << 12 per bucket; 0: the rules decide
 };
-constexpr uint32_t kTunedBuckets[14] = {8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256};
+constexpr int kTunedBucketCount = 18;
+constexpr uint32_t kTunedBuckets[kTunedBucketCount] = {8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256, 320, 384, 448, 512};
 const TunedRow kTuned[] = {
 #include "gemm_tuned.inc"
     {~0u, 0u, 0u, {0}}, // end marker
 };
 
 uint32_t tuned_lookup(int quant, uint64_t rows, uint64_t K, uint32_t T) {
-    if (T > kTunedBuckets[13] || rows == 0 || K == 0) return 0;
+    if (T > kTunedBuckets[kTunedBucketCount - 1] || rows == 0 || K == 0) return 0;
     int b = 0;
     while (kTunedBuckets[b] < T) b++;
     uint32_t best = 0;
@@ -1009,8 +1010,9 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
     const uint64_t rt = rows * a.B * T;
     const bool small = rt <= (1u << 20);
     // long rows against 256 tokens and more also take the 128-token tile (measured on 4096 x 14336: 7 % faster)
-    // (long rows from 193 tokens on: two 128-token blocks, 4096 x 14336 at 224 tokens 54.0 against 56.6 - 59.6 us)
-    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128 && n == 1) ? 2 : (T > 64 && (rt >= (1u << 23) || (T > 192 && a.K >= 8192))) ? 8 : 4;
+    // (long rows from 193 tokens on: two 128-token blocks, 4096 x 14336 at 224 tokens 54.0 against 56.6 - 59.6 us; beyond 256
+    // tokens the 128-token tile from 6 M outputs on: 16384 x 4096 at 384 tokens 92 against 106 us, 18432 rows 94 against 115 us)
+    int ntile = T <= 16 ? 1 : T <= 32 ? 2 : (small && a.K <= 8192 && T <= 128 && n == 1) ? 2 : (T > 64 && (rt >= (1u << 23) || (T > 256 && rt >= (6u << 20)) || (T > 192 && a.K >= 8192))) ? 8 : 4;
     int mrt = 2, kg = 1;
     uint32_t ksplit = 1, pinned_split = 0; // pinned_split: a measured choice that the rule of split_for() does not produce
     uint64_t wgs = 0; // workgroups of one split
@@ -1078,6 +1080,13 @@ int launch_shape(hipStream_t stream, const MatmulArgs *args, int n, const Scratc
         // against 14.3 - 15.3 us up to 64)
         ntile = 1;
         mrt = 1;
+        kg = 2;
+    }
+    if (QUANT != kFp16 && n == 1 && a.B == 1 && a.K <= 4096 && rows > 1024 && rows <= 2048 && T > 256) {
+        // a small single product with short rows beyond 256 tokens: 64 rows x 32 tokens with two k groups, unsplit
+        // (2048 x 2048 at 384 / 512 tokens: int8 14.9 / 15.1 against 19.6 / 20.4 us, nf4 18.5 / 18.9 against 21.8 / 24.2 us)
+        ntile = 2;
+        mrt = 2;
         kg = 2;
     }
     if (QUANT == kNf4 && n == 1 && a.B == 1 && a.K <= 8192 && rows > 2048 && rows <= 4096 && T <= 128) {

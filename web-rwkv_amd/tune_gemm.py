@@ -36,7 +36,7 @@ TILES = [(1, 1, 1), (1, 2, 1), (1, 4, 1), (1, 8, 1), (2, 1, 1), (2, 2, 1), (2, 4
          (2, 4, 2), (1, 1, 4), (1, 2, 4)]  # (MRT, NTILE, KG): the instantiations of gemm_kernel
 SPLITS = (1, 2, 4, 8)
 KEYS = ("gemm_mrt", "gemm_ntile", "gemm_kg", "gemm_ksplit")
-T_GRID = (8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)  # a run of T tokens takes the first bucket >= T
+T_GRID = (8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256, 320, 384, 448, 512)  # a run of T tokens takes the first bucket >= T
 
 # (C, H, kinds): kinds of launches swept for a model size.  A kind is a list of (rows, K) products that share one launch.
 FULL = ("att4", "att3", "att_o", "ffn2", "ffn_k", "ffn_v", "head")
@@ -99,6 +99,8 @@ def sweep(args):
                 mats = [[pack((torch.randn((r, k), generator=gen, device="cuda") * 0.02).half()) for r, k in prods] for _ in range(copies)]
                 rows, K = sum(r for r, _ in prods), prods[0][1]
                 for T in T_GRID:
+                    if args.tokens and str(T) not in args.tokens.split(","):
+                        continue
                     xs = [torch.randn((T, K), generator=gen, device="cuda").to(f16) for _ in prods]
                     outs = [torch.empty((T, r), dtype=f16, device="cuda") for r, _ in prods]
                     turbo = wrq.turbo(T)
@@ -316,8 +318,8 @@ def table(args):
     data = load(args.files)
     shapes = sorted({(q, rows, K) for q, rows, K, _ in data})
     print("// Generated by web-rwkv_amd/tune_gemm.py from a sweep of every tile shape and split on an MI355X; do not edit by hand.")
-    print("// One row per (format, rows of the launch, K): for each run-length bucket (8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160,")
-    print("// 192, 224, 256 tokens) the fastest combination, packed as MRT | NTILE << 4 | KG << 8 | split << 12; 0 = the rules decide.")
+    print("// One row per (format, rows of the launch, K): for each run-length bucket (" + ", ".join(str(t) for t in T_GRID[:10]) + ",")
+    print("// " + ", ".join(str(t) for t in T_GRID[10:]) + " tokens) the fastest combination, packed as MRT | NTILE << 4 | KG << 8 | split << 12; 0 = the rules decide.")
     gain = []
     for q, rows, K in shapes:
         cells = []
@@ -355,6 +357,7 @@ def main():
     s.add_argument("--out", required=True)
     s.add_argument("--quant", default="int8,nf4")
     s.add_argument("--sizes", default="", help="comma-separated CxH subset, e.g. 4096x14336")
+    s.add_argument("--tokens", default="", help="comma-separated run-length buckets, e.g. 320,384 (chunk sweep)")
     s.add_argument("--kinds", default="", help="comma-separated launch kinds, e.g. att3,ffn_k")
     s.add_argument("--decode", action="store_true", help="sweep the one-shot decode kernels (lanes and rows per task at 1 .. 4 tokens) instead of the chunk kernel")
     s.add_argument("--refine", default="", help="comma-separated sweep files: measure only their three fastest combinations per case, longer and in turn")
