@@ -6,7 +6,7 @@ one is fastest depends on the product's rows, its K, the run length and the form
 simple rule at the small end.  This tool measures all of them for the launch kinds of the RWKV model
 sizes and writes the winners as a table:
 
-  python3 web-rwkv_amd/tune_gemm.py sweep --out sweep.jsonl     (on an MI355X, about 12 minutes)
+  python3 web-rwkv_amd/tune_gemm.py sweep --out sweep.jsonl     (on an MI355X, about 20 minutes)
   python3 web-rwkv_amd/tune_gemm.py sweep --out refined.jsonl --refine sweep.jsonl
   python3 web-rwkv_amd/tune_gemm.py table sweep.jsonl refined.jsonl > web-rwkv_amd/csrc/gemm_tuned.inc
 
